@@ -1,0 +1,169 @@
+/*
+ * ofq.h -- C ABI of the MI355X (gfx950) kernels for OneFlow's quantized-inference op family.
+ *
+ * One entry point per OneFlow user op.  Each is what the op's `user_op::OpKernel::Compute`
+ * would call after unpacking its `KernelComputeContext`: raw DEVICE pointers to contiguous
+ * tensors, sizes, the op's attributes, and the HIP stream of `ctx->stream()`.
+ *
+ * Contract shared by every entry point (it mirrors what the OneFlow runtime guarantees a kernel,
+ * oneflow/core/framework/op_kernel.h:287-324, oneflow/core/vm/op_call_instruction_policy.cpp:49-82):
+ *   - the caller owns every buffer, including the workspace ("tmp_buffer"); nothing is allocated,
+ *     freed or synchronised here, work is only enqueued on `stream` (a hipStream_t, may be NULL
+ *     for the default stream), so the calls are safe under stream capture;
+ *   - the return value is an ofq_status; invalid arguments are reported, never aborted on, and
+ *     nothing is launched when the status is not OFQ_OK;
+ *   - there is no global state: calls on different streams may run concurrently.
+ * Pointers must be aligned to 16 bytes (OneFlow's allocator aligns to 512,
+ * oneflow/core/common/util.h:158-160).
+ */
+#ifndef OFQ_H_
+#define OFQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  OFQ_OK = 0,
+  OFQ_ERR_NULL_POINTER = 1,    /* a required tensor pointer is NULL, or an optional one is
+                                  present/absent against `symmetric` */
+  OFQ_ERR_BAD_DTYPE = 2,       /* dtype code not valid for this argument */
+  OFQ_ERR_BAD_SHAPE = 3,       /* sizes inconsistent (divisibility, packing, limits) */
+  OFQ_ERR_BAD_ATTR = 4,        /* attribute outside the op's domain */
+  OFQ_ERR_UNSUPPORTED = 5,     /* valid for the op, but no kernel covers the combination */
+  OFQ_ERR_WORKSPACE = 6,       /* workspace missing or smaller than *_workspace_bytes() */
+  OFQ_ERR_MISALIGNED = 7,      /* a pointer is not 16-byte aligned */
+  OFQ_ERR_LAUNCH = 8           /* hipGetLastError() after the launch was not hipSuccess */
+} ofq_status;
+
+/* element types; values follow no OneFlow enum on purpose (the adapter maps DataType) */
+typedef enum {
+  OFQ_F32 = 0,
+  OFQ_F16 = 1,
+  OFQ_BF16 = 2,
+  OFQ_F64 = 3,
+  OFQ_I8 = 4,
+  OFQ_U8 = 5
+} ofq_dtype;
+
+typedef enum { OFQ_SCHEME_SYMMETRIC = 0, OFQ_SCHEME_AFFINE = 1 } ofq_scheme;
+typedef enum { OFQ_FORMULA_GOOGLE = 0, OFQ_FORMULA_CAMBRICON = 1 } ofq_formula;
+/* how `quantization`/`fake_quantization` read an affine zero point:
+ *   OFQ_ZP_FLOAT     as stored (the rule of the CUDA kernels this library replaces,
+ *                    oneflow/user/kernels/quantization_kernel.cu:65-67),
+ *   OFQ_ZP_UINT8     rounded to uint8 first (the rule of the CPU kernels,
+ *                    oneflow/user/kernels/quantization_kernel.cpp:41-43). */
+typedef enum { OFQ_ZP_FLOAT = 0, OFQ_ZP_UINT8 = 1 } ofq_zp_mode;
+
+const char* ofq_status_string(int status);
+/* library ABI version; bumped on any signature change */
+int ofq_abi_version(void);
+
+/*
+ * groupwise_dequantize
+ * replaces GroupwiseDequantizeKernel<T>::Compute and its launchers,
+ *   oneflow/user/kernels/groupwise_quantization_kernels.cu:394-454 (and :170-392).
+ * The caller flattens the tensor the way the reference does (:436-437):
+ *   outer = Count(0, group_dim) * num_groups, inner = Count(group_dim + 1) of the OUTPUT shape;
+ *   out[outer][group_size][inner] = T(q) * scale[outer][inner] + zero[outer][inner], in T.
+ * in:      in_dtype OFQ_U8 | OFQ_I8, codes packed along the tensor's last axis
+ *          (num_bits 4: element 2i = high nibble of byte i); asymmetric requires OFQ_U8.
+ * scale:   t_dtype OFQ_F16 | OFQ_BF16 | OFQ_F32, `outer*inner` elements.
+ * zero:    same as scale; NULL iff symmetric != 0.
+ * out:     t_dtype, outer*group_size*inner elements.
+ */
+int ofq_groupwise_dequantize(void* stream, const void* in, const void* scale, const void* zero,
+                             void* out, int in_dtype, int t_dtype, int num_bits, int symmetric,
+                             int64_t outer, int64_t group_size, int64_t inner);
+
+/*
+ * fused_linear_with_groupwise_quantized_weight
+ * replaces FusedLinearWithGroupwiseQuantizedWeightKernel<T>::Compute and DispatchMatmulBias,
+ *   oneflow/user/kernels/groupwise_quantization_kernels.cu:760-839 (and :465-749),
+ * and, for m > 8, the dequantize -> matmul decomposition of the functor,
+ *   oneflow/core/functional/impl/quantization.cpp:341-350.
+ * x[m,k] (t_dtype), w[n, k*num_bits/8] (w_dtype OFQ_U8|OFQ_I8), w_scale / w_zero:
+ *   [n, k/group_size] for group_dim 1, [n/group_size, k] for group_dim 0 (t_dtype),
+ *   w_zero NULL iff symmetric, b[n] (t_dtype) or NULL, out[m,n] (t_dtype).
+ * out = T( sum_k float(x * w~) + float(b) ), w~ = T(T(q)*scale) + zero as in groupwise_dequantize.
+ * Any m is accepted (the reference kernel has no m limit either, :473,590).
+ * workspace: ofq_fused_linear_gq_workspace_bytes() bytes, may be NULL when that is 0.
+ */
+size_t ofq_fused_linear_gq_workspace_bytes(int w_dtype, int t_dtype, int num_bits, int symmetric,
+                                           int group_dim, int64_t group_size, int64_t m,
+                                           int64_t n, int64_t k);
+int ofq_fused_linear_gq(void* stream, const void* x, const void* w, const void* w_scale,
+                        const void* w_zero, const void* b, void* out, int w_dtype, int t_dtype,
+                        int num_bits, int symmetric, int group_dim, int64_t group_size, int64_t m,
+                        int64_t n, int64_t k, void* workspace, size_t workspace_bytes);
+
+/*
+ * min_max_observer
+ * replaces GpuMinMaxObserverKernel<T>::Compute,
+ *   oneflow/user/kernels/min_max_observer_kernel.cu:186-237 (arithmetic :117-163; CPU twin
+ *   oneflow/user/kernels/min_max_observer_kernel.cpp:22-58).
+ * in: in_dtype OFQ_F32 | OFQ_F64, elem_cnt elements; channels = 1 (per_layer_quantization) or
+ * in.shape[0]; scale, zero_point: `channels` elements of in_dtype.
+ * workspace: ofq_min_max_observer_workspace_bytes() (the op's "tmp_buffer", :247-254).
+ */
+size_t ofq_min_max_observer_workspace_bytes(int in_dtype, int64_t elem_cnt, int64_t channels);
+int ofq_min_max_observer(void* stream, const void* in, void* scale, void* zero_point,
+                         int in_dtype, int64_t elem_cnt, int64_t channels, int quantization_bit,
+                         int scheme, int formula, void* workspace, size_t workspace_bytes);
+
+/*
+ * quantization / fake_quantization
+ * replace GpuQuantizationKernel<T>::Compute, oneflow/user/kernels/quantization_kernel.cu:107-144
+ * (arithmetic :24-95) and GpuFakeQuantizationKernel<T>::Compute,
+ * oneflow/user/kernels/fake_quantization_kernel.cu:24-96.
+ * in: in_dtype OFQ_F32 | OFQ_F64 (the reference's types) or OFQ_F16 | OFQ_BF16 (dynamic
+ *     activation path: scale/zero_point are then fp32 and the divide is done in fp32).
+ * out: out_dtype == in_dtype (the reference: codes stored in the input type) or, for
+ *     `quantization` only, OFQ_I8 (symmetric) / OFQ_U8 (affine) integer codes.
+ * scale_size 1 = per-layer, else per-channel with scale_size == shape0 and panel = elem_cnt/shape0.
+ */
+int ofq_quantization(void* stream, const void* in, const void* scale, const void* zero_point,
+                     void* out, int in_dtype, int out_dtype, int64_t elem_cnt, int64_t scale_size,
+                     int quantization_bit, int scheme, int formula, int zp_mode);
+int ofq_fake_quantization(void* stream, const void* in, const void* scale,
+                          const void* zero_point, void* out, int in_dtype, int64_t elem_cnt,
+                          int64_t scale_size, int quantization_bit, int scheme, int formula,
+                          int zp_mode);
+
+/*
+ * fused_layer_norm_min_max_observer
+ * The op is named by the task but absent from the reference tree; it composes
+ *   LayerNorm over the last axis (oneflow/core/cuda/layer_norm.cuh:212-233,377-380 and the
+ *   affine store of oneflow/user/kernels/layer_norm_gpu_kernel.cu:40-70) with a per-tensor
+ *   symmetric min_max_observer (min_max_observer_kernel.cu:117-131) of the normalised output.
+ * x, y: [rows, cols] t_dtype OFQ_F16 | OFQ_BF16 | OFQ_F32; gamma, beta: [cols] t_dtype or NULL;
+ * scale, zero_point: one fp32 each.
+ */
+size_t ofq_fused_layer_norm_min_max_observer_workspace_bytes(int t_dtype, int64_t rows,
+                                                             int64_t cols);
+int ofq_fused_layer_norm_min_max_observer(void* stream, const void* x, const void* gamma,
+                                          const void* beta, void* y, float* scale,
+                                          float* zero_point, int t_dtype, int64_t rows,
+                                          int64_t cols, double epsilon, int quantization_bit,
+                                          void* workspace, size_t workspace_bytes);
+
+/*
+ * matmul_quant
+ * The op is named by the task but absent from the reference tree (only the env-var name
+ * ONEFLOW_MLIR_GROUP_MATMUL_QUANT, python/oneflow/framework/infer_compiler/with_fx_graph.py:63);
+ * operand conventions follow fused_matmul_bias (oneflow/ir/include/OneFlow/OneFlowUserOps.td:5615-5633):
+ * a[m,k] int8, b[n,k] int8 (weight layout), exact int32 accumulation,
+ * out[m,n] = T( float(acc) * (a_scale[0] * b_scale[n]) + float(bias[n]) ), out_dtype OFQ_F16 |
+ * OFQ_BF16 | OFQ_F32; a_scale: one fp32 on the device; b_scale: fp32[n]; bias: out_dtype[n] or NULL.
+ */
+int ofq_matmul_quant(void* stream, const void* a, const void* b, const float* a_scale,
+                     const float* b_scale, const void* bias, void* out, int out_dtype, int64_t m,
+                     int64_t n, int64_t k);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OFQ_H_ */

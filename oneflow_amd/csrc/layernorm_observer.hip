@@ -1,0 +1,230 @@
+// fused_layer_norm_min_max_observer for gfx950: LayerNorm over the last axis fused with a
+// per-tensor symmetric min/max observer of the normalised output.
+//
+// LayerNorm arithmetic (oneflow/core/cuda/layer_norm.cuh:212-233,377-380 and the affine store of
+// oneflow/user/kernels/layer_norm_gpu_kernel.cu:40-70): statistics in fp32,
+// var = max(M2/n, 0), inv = rsqrt(var + eps); the normalised value is rounded to T first and the
+// affine `* gamma + beta` is then carried out in T (two more roundings).
+// Observer (oneflow/user/kernels/min_max_observer_kernel.cu:117-131): scale = absmax / (2^(b-1)-1).
+//
+// One block per row.  The row is read from HBM once (128-bit loads) and kept in registers for
+// the three uses (sum, squared deviations, normalise); the block's absmax of the stored values
+// goes to workspace[row], and a second one-block launch folds the rows and divides.
+#include "ofq_device.h"
+
+namespace ofq {
+namespace {
+
+constexpr int kLnBlock = 256;
+
+template<typename T>
+struct Pack8 {
+  typename TT<T>::storage v[8];
+};
+
+template<typename T>
+__device__ __forceinline__ void load8(const typename TT<T>::storage* p, float* f) {
+  typedef typename TT<T>::storage S;
+  S tmp[8];
+  if (sizeof(S) == 2) {
+    *reinterpret_cast<u32x4*>(tmp) = *reinterpret_cast<const u32x4*>(p);
+  } else {
+    reinterpret_cast<u32x4*>(tmp)[0] = reinterpret_cast<const u32x4*>(p)[0];
+    reinterpret_cast<u32x4*>(tmp)[1] = reinterpret_cast<const u32x4*>(p)[1];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = TT<T>::load(&tmp[e]);
+}
+
+template<typename T>
+__device__ __forceinline__ void store8(typename TT<T>::storage* p, const float* f) {
+  typedef typename TT<T>::storage S;
+  S tmp[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) TT<T>::store(&tmp[e], f[e]);
+  if (sizeof(S) == 2) {
+    *reinterpret_cast<u32x4*>(p) = *reinterpret_cast<const u32x4*>(tmp);
+  } else {
+    reinterpret_cast<u32x4*>(p)[0] = reinterpret_cast<const u32x4*>(tmp)[0];
+    reinterpret_cast<u32x4*>(p)[1] = reinterpret_cast<const u32x4*>(tmp)[1];
+  }
+}
+
+// NP = packs of 8 elements each lane caches; cols <= kLnBlock * 8 * NP and 8 | cols.
+template<typename T, int NP>
+__global__ void __launch_bounds__(kLnBlock)
+ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
+                 const typename TT<T>::storage* __restrict__ gamma,
+                 const typename TT<T>::storage* __restrict__ beta,
+                 typename TT<T>::storage* __restrict__ y, float* __restrict__ row_absmax,
+                 int64_t cols, float eps) {
+  __shared__ float smem[kLnBlock / kWave];
+  const int64_t row = blockIdx.x;
+  const typename TT<T>::storage* xr = x + row * cols;
+  typename TT<T>::storage* yr = y + row * cols;
+  const int npacks = (int)(cols / 8);
+  float v[NP][8];
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int p = threadIdx.x + i * kLnBlock;
+    if (p < npacks) {
+      load8<T>(xr + (int64_t)p * 8, v[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += v[i][e];
+    }
+  }
+  sum = block_reduce(sum, OpSum(), smem);
+  const float mean = sum / (float)cols;
+  float m2 = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int p = threadIdx.x + i * kLnBlock;
+    if (p < npacks) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = v[i][e] - mean;
+        m2 = __builtin_fmaf(d, d, m2);
+      }
+    }
+  }
+  m2 = block_reduce(m2, OpSum(), smem);
+  const float var = fmaxf(m2 / (float)cols, 0.0f);
+  const float inv = 1.0f / __builtin_sqrtf(var + eps);
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int p = threadIdx.x + i * kLnBlock;
+    if (p < npacks) {
+      float g[8], b[8], o[8];
+      if (gamma) load8<T>(gamma + (int64_t)p * 8, g);
+      if (beta) load8<T>(beta + (int64_t)p * 8, b);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float t = TT<T>::round((v[i][e] - mean) * inv);
+        if (gamma) t = TT<T>::round(t * g[e]);
+        if (beta) t = TT<T>::round(t + b[e]);
+        o[e] = t;
+        amax = fmaxf(amax, fabsf(t));
+      }
+      store8<T>(yr + (int64_t)p * 8, o);
+    }
+  }
+  amax = block_reduce(amax, OpMax(), smem);
+  if (threadIdx.x == 0) row_absmax[row] = amax;
+}
+
+// any cols: three passes over the row through L2 (the row was just read, so only the first
+// pass touches HBM), scalar accesses.
+template<typename T>
+__global__ void __launch_bounds__(kLnBlock)
+ln_observer_rows_generic(const typename TT<T>::storage* __restrict__ x,
+                         const typename TT<T>::storage* __restrict__ gamma,
+                         const typename TT<T>::storage* __restrict__ beta,
+                         typename TT<T>::storage* __restrict__ y, float* __restrict__ row_absmax,
+                         int64_t cols, float eps) {
+  __shared__ float smem[kLnBlock / kWave];
+  const int64_t row = blockIdx.x;
+  const typename TT<T>::storage* xr = x + row * cols;
+  typename TT<T>::storage* yr = y + row * cols;
+  float sum = 0.0f;
+  for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) sum += TT<T>::load(xr + c);
+  sum = block_reduce(sum, OpSum(), smem);
+  const float mean = sum / (float)cols;
+  float m2 = 0.0f;
+  for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
+    const float d = TT<T>::load(xr + c) - mean;
+    m2 = __builtin_fmaf(d, d, m2);
+  }
+  m2 = block_reduce(m2, OpSum(), smem);
+  const float var = fmaxf(m2 / (float)cols, 0.0f);
+  const float inv = 1.0f / __builtin_sqrtf(var + eps);
+  float amax = 0.0f;
+  for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
+    float t = TT<T>::round((TT<T>::load(xr + c) - mean) * inv);
+    if (gamma) t = TT<T>::round(t * TT<T>::load(gamma + c));
+    if (beta) t = TT<T>::round(t + TT<T>::load(beta + c));
+    TT<T>::store(yr + c, t);
+    amax = fmaxf(amax, fabsf(t));
+  }
+  amax = block_reduce(amax, OpMax(), smem);
+  if (threadIdx.x == 0) row_absmax[row] = amax;
+}
+
+__global__ void __launch_bounds__(kLnBlock)
+ln_observer_finalize(const float* __restrict__ row_absmax, int64_t rows, int bits,
+                     float* __restrict__ scale, float* __restrict__ zero_point) {
+  __shared__ float smem[kLnBlock / kWave];
+  float amax = 0.0f;
+  for (int64_t r = threadIdx.x; r < rows; r += kLnBlock) amax = fmaxf(amax, row_absmax[r]);
+  amax = block_reduce(amax, OpMax(), smem);
+  if (threadIdx.x == 0) {
+    const float denominator = (float)(1 << (bits - 1)) - 1.0f;
+    *scale = amax / denominator;
+    *zero_point = 0.0f;
+  }
+}
+
+template<typename T>
+int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, void* y,
+           float* scale, float* zero_point, int64_t rows, int64_t cols, float eps, int bits,
+           float* ws) {
+  typedef typename TT<T>::storage S;
+  const S* xs = static_cast<const S*>(x);
+  const S* gs = static_cast<const S*>(gamma);
+  const S* bs = static_cast<const S*>(beta);
+  S* ys = static_cast<S*>(y);
+  const bool vec_ok = cols % 8 == 0 && ofq_aligned16(x) && ofq_aligned16(y)
+                      && ofq_aligned16(gamma) && ofq_aligned16(beta)
+                      && (cols * sizeof(S)) % 16 == 0;
+  const int64_t npacks = cols / 8;
+  if (vec_ok && npacks <= kLnBlock) {
+    ln_observer_rows<T, 1><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+  } else if (vec_ok && npacks <= 2 * kLnBlock) {
+    ln_observer_rows<T, 2><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+  } else if (vec_ok && npacks <= 4 * kLnBlock) {
+    ln_observer_rows<T, 4><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+  } else {
+    ln_observer_rows_generic<T><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+  }
+  ln_observer_finalize<<<1, kLnBlock, 0, st>>>(ws, rows, bits, scale, zero_point);
+  return ofq_check_launch();
+}
+
+}  // namespace
+}  // namespace ofq
+
+extern "C" size_t ofq_fused_layer_norm_min_max_observer_workspace_bytes(int, int64_t rows,
+                                                                        int64_t) {
+  return rows > 0 ? (size_t)rows * sizeof(float) : 0;
+}
+
+extern "C" int ofq_fused_layer_norm_min_max_observer(void* stream, const void* x,
+                                                     const void* gamma, const void* beta, void* y,
+                                                     float* scale, float* zero_point, int t_dtype,
+                                                     int64_t rows, int64_t cols, double epsilon,
+                                                     int quantization_bit, void* workspace,
+                                                     size_t workspace_bytes) {
+  OFQ_RETURN_IF(quantization_bit <= 1 || quantization_bit > 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(t_dtype != OFQ_F16 && t_dtype != OFQ_BF16 && t_dtype != OFQ_F32,
+                OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(rows < 1 || cols < 1 || rows > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(x == nullptr || y == nullptr || scale == nullptr || zero_point == nullptr,
+                OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(workspace == nullptr || workspace_bytes < (size_t)rows * sizeof(float),
+                OFQ_ERR_WORKSPACE);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  const float eps = (float)epsilon;
+  switch (t_dtype) {
+    case OFQ_F16:
+      return ofq::launch<ofq::f16>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps,
+                                   quantization_bit, ws);
+    case OFQ_BF16:
+      return ofq::launch<ofq::bf16>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps,
+                                    quantization_bit, ws);
+    default:
+      return ofq::launch<float>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps,
+                                quantization_bit, ws);
+  }
+}

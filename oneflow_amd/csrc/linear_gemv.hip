@@ -1,0 +1,372 @@
+// fused_linear_with_groupwise_quantized_weight, decode side (m <= 16), for gfx950, plus the
+// any-shape fallback and the op's C entry point.
+//
+// Semantics (oneflow/user/kernels/groupwise_quantization_kernels.cu:582-642, :760-839):
+//   w~[n,k] = T(T(q[n,k]) * scale[n,g]) + zero[n,g]   (both operations round to T)
+//   out[m,n] = T( sum_k x[m,k] * w~[n,k]  (fp32 accumulation)  + float(bias[n]) )
+//
+// Decode kernel.  The reference launches one 128-thread block per output element and so streams
+// the weights m times.  Here the m <= 16 rows of x ride along as the second operand of a
+// 16x16x32 MFMA whose first dimension is 16 weight rows, so the weights are read from HBM exactly
+// once whatever m is, and the k-reduction happens inside the matrix core instead of in a
+// cross-lane tree:
+//   - a block owns 16 consecutive weight rows and all of K; its waves take K in interleaved
+//     chunks of 128 (4-bit) / 64 (8-bit) elements, i.e. one 128-bit load per lane covering
+//     16 rows x 64 bytes;
+//   - lane (r = lane%16, kb = lane/16) loads 16 bytes of row r; its 32 (16) codes feed the
+//     "k-slot kb" of 4 (2) MFMAs.  The MFMA sums over k-slots, so any assignment of k to
+//     (slot, element) is valid as long as the x operand uses the same one;
+//   - int4 -> fp16 without conversions: (word & 0x000F000F) | 0x64006400 is the half2
+//     (1024+q_lo, 1024+q_hi); the nibbles 4 bits up give 1024+16q.  One packed add (or fma by
+//     1/16) recovers the codes exactly; an int8 container is first xor-ed with 0x88888888 to
+//     turn two's complement nibbles into offset binary.  The codes come out pairwise
+//     (e1,e5),(e0,e4),(e3,e7),(e2,e6) and x is permuted to match with four v_perm_b32;
+//   - w~ is then formed exactly as the reference does (packed fp16 multiply by the group scale,
+//     packed add of the zero term), which keeps the kernel bit-compatible with
+//     groupwise_dequantize;
+//   - partial sums of the waves are combined through LDS, bias is added in fp32, one rounding
+//     to T.
+#include "ofq_device.h"
+#include "ofq_internal.h"
+
+namespace ofq {
+namespace {
+
+enum { kZeroNone = 0, kZeroSymU = 1, kZeroAsym = 2 };
+
+__device__ __forceinline__ f16x2 as_h2(uint32_t u) { return __builtin_bit_cast(f16x2, u); }
+__device__ __forceinline__ uint32_t as_u32(f16x2 h) { return __builtin_bit_cast(uint32_t, h); }
+
+// eight 4-bit codes of `word` as exact fp16 values, in the pair order
+// (e1,e5) (e0,e4) (e3,e7) (e2,e6) where e_i is element i of the word (element 0 = high nibble
+// of byte 0).
+template<bool SIGNED>
+__device__ __forceinline__ void unpack4_pairs(uint32_t word, f16x2 (&o)[4]) {
+  if (SIGNED) word ^= 0x88888888u;
+  const uint32_t w8 = word >> 8;
+  const f16 off_lo = SIGNED ? (f16)(-1032.0f) : (f16)(-1024.0f);
+  const f16 off_hi = SIGNED ? (f16)(-72.0f) : (f16)(-64.0f);
+  const f16x2 ol = {off_lo, off_lo};
+  const f16x2 oh = {off_hi, off_hi};
+  const f16x2 sixteenth = {(f16)0.0625f, (f16)0.0625f};
+  o[0] = as_h2((word & 0x000F000Fu) | 0x64006400u) + ol;
+  o[1] = __builtin_elementwise_fma(as_h2((word & 0x00F000F0u) | 0x64006400u), sixteenth, oh);
+  o[2] = as_h2((w8 & 0x000F000Fu) | 0x64006400u) + ol;
+  o[3] = __builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x64006400u), sixteenth, oh);
+}
+
+// four 8-bit codes of `word` as exact fp16 values in natural order (b0,b1) (b2,b3)
+template<bool SIGNED>
+__device__ __forceinline__ void unpack8_pairs(uint32_t word, f16x2 (&o)[2]) {
+  if (SIGNED) word ^= 0x80808080u;
+  const f16 off = SIGNED ? (f16)(-1152.0f) : (f16)(-1024.0f);
+  const f16x2 o2 = {off, off};
+  o[0] = as_h2(__builtin_amdgcn_perm(word, 0x64646464u, 0x00050004u)) + o2;
+  o[1] = as_h2(__builtin_amdgcn_perm(word, 0x64646464u, 0x00070006u)) + o2;
+}
+
+// x permuted to the pair order of unpack4_pairs: [x1,x5,x0,x4,x3,x7,x2,x6]
+__device__ __forceinline__ u32x4 permute_x4(u32x4 v) {
+  u32x4 r;
+  r[0] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // (x1, x5)
+  r[1] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // (x0, x4)
+  r[2] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // (x3, x7)
+  r[3] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // (x2, x6)
+  return r;
+}
+
+template<int BITS, bool SIGNED, int ZMODE, int NWAVES, int UNROLL>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_f16_mfma(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+              const f16* __restrict__ scale, const f16* __restrict__ zero,
+              const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
+              int group_size, int gs_shift) {
+  constexpr int CH = BITS == 4 ? 128 : 64;  // k elements per chunk (64 bytes of codes per row)
+  constexpr int LK = CH / 4;                // k elements per lane per chunk
+  constexpr int NJ = LK / 8;                // MFMAs per chunk
+  __shared__ float red[NWAVES][64][4];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15;
+  const int kb = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int n_ld = (n0 + r < N) ? n0 + r : N - 1;  // clamp loads of a partial last tile
+  const int nchunks = K / CH;
+  const int G = K / group_size;
+  const uint8_t* wrow = w + (int64_t)n_ld * ((int64_t)K * BITS / 8);
+  const f16* srow = scale + (int64_t)n_ld * G;
+  const f16* zrow = ZMODE == kZeroAsym ? zero + (int64_t)n_ld * G : nullptr;
+  const bool has_x = r < M;
+  const f16* xrow = x + (int64_t)(has_x ? r : 0) * K;
+
+  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc1 = {0.f, 0.f, 0.f, 0.f};
+
+  for (int c0 = wave; c0 < nchunks; c0 += NWAVES * UNROLL) {
+    u32x4 wq[UNROLL];
+    u32x4 xv[UNROLL][NJ];
+    f16 sv[UNROLL], zv[UNROLL];
+    // issue every load of the UNROLL chunks before touching any of them
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * NWAVES;
+      const bool valid = c < nchunks;
+      const int k0 = (valid ? c : 0) * CH + kb * LK;
+      wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (int64_t)k0 * BITS / 8));
+      const int g = gs_shift >= 0 ? (k0 >> gs_shift) : (k0 / group_size);
+      sv[u] = srow[g];
+      zv[u] = ZMODE == kZeroAsym ? zrow[g] : (f16)0.0f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const u32x4 t = *reinterpret_cast<const u32x4*>(xrow + k0 + j * 8);
+        const u32x4 zero4 = {0u, 0u, 0u, 0u};
+        xv[u][j] = (has_x && valid) ? t : zero4;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const f16 s = sv[u];
+      f16 z = zv[u];
+      if (ZMODE == kZeroSymU) z = (f16)(-(float)((1 << (BITS - 1)) - 1)) * s;
+      const f16x2 s2 = {s, s};
+      const f16x2 z2 = {z, z};
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        u32x4 bop;
+        u32x4 aop;
+        if (BITS == 4) {
+          f16x2 p[4];
+          unpack4_pairs<SIGNED>(wq[u][j], p);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            f16x2 v = p[e] * s2;
+            if (ZMODE != kZeroNone) v = v + z2;
+            bop[e] = as_u32(v);
+          }
+          aop = permute_x4(xv[u][j]);
+        } else {
+          f16x2 p0[2], p1[2];
+          unpack8_pairs<SIGNED>(wq[u][2 * j], p0);
+          unpack8_pairs<SIGNED>(wq[u][2 * j + 1], p1);
+          f16x2 v[4] = {p0[0] * s2, p0[1] * s2, p1[0] * s2, p1[1] * s2};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (ZMODE != kZeroNone) v[e] = v[e] + z2;
+            bop[e] = as_u32(v[e]);
+          }
+          aop = xv[u][j];
+        }
+        const f16x8 a8 = __builtin_bit_cast(f16x8, aop);
+        const f16x8 b8 = __builtin_bit_cast(f16x8, bop);
+        if ((j & 1) == 0) {
+          acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a8, b8, acc0, 0, 0, 0);
+        } else {
+          acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a8, b8, acc1, 0, 0, 0);
+        }
+      }
+    }
+  }
+  // lane holds D[m = 4*kb + v][n = n0 + r]
+#pragma unroll
+  for (int v = 0; v < 4; ++v) red[wave][lane][v] = acc0[v] + acc1[v];
+  __syncthreads();
+  for (int t = threadIdx.x; t < 256; t += NWAVES * 64) {
+    const int l = t >> 2;
+    const int v = t & 3;
+    float sum = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < NWAVES; ++wv) sum += red[wv][l][v];
+    const int m = 4 * (l >> 4) + v;
+    const int n = n0 + (l & 15);
+    if (m < M && n < N) {
+      if (bias != nullptr) sum += (float)bias[n];
+      out[(int64_t)m * N + n] = (f16)sum;
+    }
+  }
+}
+
+// ---- any shape, any grouping: one wave per output element --------------------------------
+template<typename T, int BITS, bool SIGNED>
+__global__ void __launch_bounds__(256)
+linear_generic(const typename TT<T>::storage* __restrict__ x, const uint8_t* __restrict__ w,
+               const typename TT<T>::storage* __restrict__ scale,
+               const typename TT<T>::storage* __restrict__ zero,
+               const typename TT<T>::storage* __restrict__ bias,
+               typename TT<T>::storage* __restrict__ out, int64_t M, int64_t N, int64_t K,
+               int group_dim, int64_t group_size, int symmetric) {
+  const int lane = threadIdx.x & 63;
+  const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t m = blockIdx.y;
+  if (n >= N) return;
+  const int64_t G = group_dim == 1 ? K / group_size : 0;
+  float acc = 0.f;
+  for (int64_t k = lane; k < K; k += 64) {
+    const int64_t si = group_dim == 1 ? n * G + k / group_size : (n / group_size) * K + k;
+    const float s = TT<T>::load(scale + si);
+    float z;
+    if (!symmetric) {
+      z = TT<T>::load(zero + si);
+    } else if (SIGNED) {
+      z = 0.f;
+    } else {
+      z = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * s);
+    }
+    const float q = (float)code_at<BITS, SIGNED>(w, n * K + k);
+    const float wv = TT<T>::round(TT<T>::round(q * s) + z);
+    acc = __builtin_fmaf(TT<T>::load(x + m * K + k), wv, acc);
+  }
+  acc = wave_reduce(acc, OpSum());
+  if (lane == 0) {
+    if (bias != nullptr) acc += TT<T>::load(bias + n);
+    TT<T>::store(out + m * N + n, acc);
+  }
+}
+
+template<typename T>
+int launch_generic_t(hipStream_t st, const LinearArgs& a) {
+  typedef typename TT<T>::storage S;
+  dim3 grid((unsigned)((a.n + 3) / 4), (unsigned)a.m);
+#define OFQ_G(B, SG)                                                                         \
+  if (a.bits == B && a.w_signed == SG) {                                                     \
+    linear_generic<T, B, SG><<<grid, 256, 0, st>>>(                                          \
+        static_cast<const S*>(a.x), static_cast<const uint8_t*>(a.w),                        \
+        static_cast<const S*>(a.scale), static_cast<const S*>(a.zero),                       \
+        static_cast<const S*>(a.bias), static_cast<S*>(a.out), a.m, a.n, a.k, a.group_dim,   \
+        a.group_size, a.symmetric ? 1 : 0);                                                  \
+    return ofq_check_launch();                                                               \
+  }
+  OFQ_G(4, false) OFQ_G(4, true) OFQ_G(8, false) OFQ_G(8, true)
+#undef OFQ_G
+  return OFQ_ERR_UNSUPPORTED;
+}
+
+inline int ilog2_exact(int64_t v) {
+  if (v <= 0 || (v & (v - 1)) != 0) return -1;
+  int s = 0;
+  while ((1LL << s) < v) ++s;
+  return s;
+}
+
+template<int BITS, bool SIGNED, int ZMODE>
+int launch_gemv_variant(hipStream_t st, const LinearArgs& a) {
+  constexpr int CH = BITS == 4 ? 128 : 64;
+  const int nchunks = (int)(a.k / CH);
+  const int grid = (int)((a.n + 15) / 16);
+  const int gs_shift = ilog2_exact(a.group_size);
+  const f16* x = static_cast<const f16*>(a.x);
+  const uint8_t* w = static_cast<const uint8_t*>(a.w);
+  const f16* sc = static_cast<const f16*>(a.scale);
+  const f16* ze = static_cast<const f16*>(a.zero);
+  const f16* bi = static_cast<const f16*>(a.bias);
+  f16* out = static_cast<f16*>(a.out);
+  // waves per block: enough to spread K, few enough that every wave has >= 2 chunks
+  if (nchunks >= 64) {
+    gemv_f16_mfma<BITS, SIGNED, ZMODE, 16, 2><<<grid, 16 * 64, 0, st>>>(
+        x, w, sc, ze, bi, out, (int)a.m, (int)a.n, (int)a.k, (int)a.group_size, gs_shift);
+  } else if (nchunks >= 16) {
+    gemv_f16_mfma<BITS, SIGNED, ZMODE, 8, 4><<<grid, 8 * 64, 0, st>>>(
+        x, w, sc, ze, bi, out, (int)a.m, (int)a.n, (int)a.k, (int)a.group_size, gs_shift);
+  } else {
+    gemv_f16_mfma<BITS, SIGNED, ZMODE, 4, 2><<<grid, 4 * 64, 0, st>>>(
+        x, w, sc, ze, bi, out, (int)a.m, (int)a.n, (int)a.k, (int)a.group_size, gs_shift);
+  }
+  return ofq_check_launch();
+}
+
+}  // namespace
+
+bool gemv_wq_supported(const LinearArgs& a) {
+  if (a.t_dtype != OFQ_F16 || a.group_dim != 1 || a.m > 16 || a.m < 1) return false;
+  const int ch = a.bits == 4 ? 128 : 64;
+  const int lk = ch / 4;
+  if (a.k % ch != 0 || a.group_size % lk != 0) return false;
+  if (a.n * a.k > 0x7FFFFFFFLL * 8 || a.k > 0x7FFFFFFF || a.n > 0x7FFFFFFF - 16) return false;
+  return true;
+}
+
+int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
+  const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
+#define OFQ_V(B, SG, ZM) \
+  if (a.bits == B && a.w_signed == SG && zmode == ZM) return launch_gemv_variant<B, SG, ZM>(st, a);
+  OFQ_V(4, true, kZeroNone)
+  OFQ_V(4, false, kZeroSymU)
+  OFQ_V(4, false, kZeroAsym)
+  OFQ_V(8, true, kZeroNone)
+  OFQ_V(8, false, kZeroSymU)
+  OFQ_V(8, false, kZeroAsym)
+#undef OFQ_V
+  return OFQ_ERR_UNSUPPORTED;
+}
+
+int launch_linear_generic(hipStream_t st, const LinearArgs& a) {
+  if (a.m > 65535) return OFQ_ERR_UNSUPPORTED;
+  switch (a.t_dtype) {
+    case OFQ_F16: return launch_generic_t<f16>(st, a);
+    case OFQ_BF16: return launch_generic_t<bf16>(st, a);
+    case OFQ_F32: return launch_generic_t<float>(st, a);
+    default: return OFQ_ERR_BAD_DTYPE;
+  }
+}
+
+}  // namespace ofq
+
+using namespace ofq;
+
+extern "C" size_t ofq_fused_linear_gq_workspace_bytes(int, int, int, int, int, int64_t, int64_t,
+                                                      int64_t, int64_t) {
+  return 0;  // every path keeps its partial sums in registers / LDS
+}
+
+extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
+                                   const void* w_scale, const void* w_zero, const void* b,
+                                   void* out, int w_dtype, int t_dtype, int num_bits,
+                                   int symmetric, int group_dim, int64_t group_size, int64_t m,
+                                   int64_t n, int64_t k, void* workspace, size_t workspace_bytes) {
+  (void)workspace;
+  (void)workspace_bytes;
+  // checks of FusedLinearWithGroupwiseQuantizedWeightKernel::Compute,
+  // groupwise_quantization_kernels.cu:773-822
+  OFQ_RETURN_IF(num_bits != 4 && num_bits != 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(group_dim != 0 && group_dim != 1, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(w_dtype != OFQ_U8 && w_dtype != OFQ_I8, OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(!symmetric && w_dtype != OFQ_U8, OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(t_dtype != OFQ_F16 && t_dtype != OFQ_BF16 && t_dtype != OFQ_F32,
+                OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(m < 0 || n < 0 || k <= 0, OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(k % (8 / num_bits) != 0, OFQ_ERR_BAD_SHAPE);
+  const int64_t group_dim_size = group_dim == 0 ? n : k;
+  OFQ_RETURN_IF(group_size <= 0, OFQ_ERR_BAD_ATTR);
+  if (m == 0 || n == 0) return OFQ_OK;
+  OFQ_RETURN_IF(group_size > group_dim_size || group_dim_size % group_size != 0,
+                OFQ_ERR_BAD_SHAPE);
+  // int32 index limits of the reference launchers, :651-655
+  const int64_t i32max = 0x7FFFFFFF;
+  OFQ_RETURN_IF(m * k > i32max || n * k > i32max || m * n > i32max, OFQ_ERR_UNSUPPORTED);
+  OFQ_RETURN_IF(x == nullptr || w == nullptr || w_scale == nullptr || out == nullptr,
+                OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF((symmetric != 0) != (w_zero == nullptr), OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(!ofq_aligned16(x) || !ofq_aligned16(w) || !ofq_aligned16(w_scale)
+                    || !ofq_aligned16(w_zero) || !ofq_aligned16(b) || !ofq_aligned16(out),
+                OFQ_ERR_MISALIGNED);
+  LinearArgs a;
+  a.x = x;
+  a.w = w;
+  a.scale = w_scale;
+  a.zero = w_zero;
+  a.bias = b;
+  a.out = out;
+  a.t_dtype = t_dtype;
+  a.w_signed = w_dtype == OFQ_I8;
+  a.bits = num_bits;
+  a.symmetric = symmetric != 0;
+  a.group_dim = group_dim;
+  a.group_size = group_size;
+  a.m = m;
+  a.n = n;
+  a.k = k;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (gemv_wq_supported(a)) return launch_gemv_wq(st, a);
+  if (gemm_wq_supported(a)) return launch_gemm_wq(st, a);
+  return launch_linear_generic(st, a);
+}

@@ -1,0 +1,422 @@
+// min_max_observer, quantization, fake_quantization for gfx950.
+//
+// Arithmetic follows the reference kernels exactly so that codes are bit-identical:
+//   observer      oneflow/user/kernels/min_max_observer_kernel.cpp:22-58 (.cu:117-163)
+//   quantization  oneflow/user/kernels/quantization_kernel.cpp:22-62 (.cu:24-95)
+//   fake quant    oneflow/user/kernels/fake_quantization_kernel.cpp:22-64 (.cu:24-96)
+// i.e. one correctly rounded division, rint (round-half-even), ternary clamps that keep -0.0 and
+// NaN as the CPU code does.  hipcc's default fp32 division is the IEEE sequence.
+//
+// Observer structure: a channel (or the whole tensor) is cut into `splits` slices so that the
+// grid has enough blocks to pull full HBM bandwidth; every block reduces its slice's max and
+// min with 128-bit loads and wave shuffles and stores one (max,min) pair in the workspace; a
+// second tiny launch folds the pairs and does the scale / zero-point arithmetic.  No atomics,
+// no initialisation pass, and the result does not depend on block scheduling.
+#include "ofq_device.h"
+
+namespace ofq {
+namespace {
+
+constexpr int kObsBlock = 256;
+constexpr int64_t kObsSliceElems = 16384;  // elements one block reduces
+
+__host__ __device__ inline int64_t obs_splits(int64_t inner) {
+  int64_t s = (inner + kObsSliceElems - 1) / kObsSliceElems;
+  return s < 1 ? 1 : s;
+}
+
+template<typename T>
+__global__ void __launch_bounds__(kObsBlock)
+observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, T* __restrict__ part) {
+  __shared__ T smem[kObsBlock / kWave];
+  const int64_t c = blockIdx.x / splits;
+  const int64_t sp = blockIdx.x % splits;
+  const int64_t begin = sp * kObsSliceElems;
+  int64_t end = begin + kObsSliceElems;
+  if (end > inner) end = inner;
+  const T* p = in + c * inner;
+  T vmax = p[begin];
+  T vmin = vmax;
+  constexpr int V = 16 / sizeof(T);
+  // vector body when the slice start is 16-byte aligned
+  int64_t i = begin;
+  if (((reinterpret_cast<uintptr_t>(p + begin)) & 15u) == 0) {
+    const int64_t nvec = (end - begin) / V;
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    const vec_t* pv = reinterpret_cast<const vec_t*>(p + begin);
+    for (int64_t v = threadIdx.x; v < nvec; v += kObsBlock) {
+      const vec_t x = pv[v];
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        vmax = OpMax()(vmax, x[e]);
+        vmin = OpMin()(vmin, x[e]);
+      }
+    }
+    i = begin + nvec * V;
+  }
+  for (int64_t j = i + threadIdx.x; j < end; j += kObsBlock) {
+    vmax = OpMax()(vmax, p[j]);
+    vmin = OpMin()(vmin, p[j]);
+  }
+  vmax = block_reduce(vmax, OpMax(), smem);
+  vmin = block_reduce(vmin, OpMin(), smem);
+  if (threadIdx.x == 0) {
+    part[2 * blockIdx.x] = vmax;
+    part[2 * blockIdx.x + 1] = vmin;
+  }
+}
+
+template<typename T>
+__device__ __forceinline__ T t_rint(T v);
+template<>
+__device__ __forceinline__ float t_rint<float>(float v) {
+  return __builtin_rintf(v);
+}
+template<>
+__device__ __forceinline__ double t_rint<double>(double v) {
+  return __builtin_rint(v);
+}
+template<typename T>
+__device__ __forceinline__ T t_abs(T v) {
+  return v < 0 ? -v : (v == 0 ? (T)0 : v);
+}
+
+template<typename T>
+__global__ void __launch_bounds__(kObsBlock)
+observer_finalize(const T* __restrict__ part, int64_t channels, int64_t splits, int bits,
+                  int scheme, int formula, T* __restrict__ scale, T* __restrict__ zero_point) {
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  T vmax = part[2 * c * splits];
+  T vmin = part[2 * c * splits + 1];
+  for (int64_t s = 1; s < splits; ++s) {
+    vmax = OpMax()(vmax, part[2 * (c * splits + s)]);
+    vmin = OpMin()(vmin, part[2 * (c * splits + s) + 1]);
+  }
+  if (formula == OFQ_FORMULA_CAMBRICON) {
+    const T a = t_abs(vmax), b = t_abs(vmin);
+    const T m = a < b ? b : a;
+    // floor(log2(m)) with log2 evaluated in double and rounded to T, which is what a correctly
+    // rounded libm log2 of the CPU kernel returns (min_max_observer_kernel.cpp:55)
+    const T lg = (T)log2((double)m);
+    scale[c] = floor(lg) - (T)(bits - 2);
+    zero_point[c] = 0;
+  } else if (scheme == OFQ_SCHEME_SYMMETRIC) {
+    const T a = t_abs(vmax), b = t_abs(vmin);
+    const T m = a < b ? b : a;
+    const T denominator = (T)(1 << (bits - 1)) - 1;
+    scale[c] = m / denominator;
+    zero_point[c] = 0;
+  } else {
+    const T denominator = (T)(1 << bits) - 1;
+    const T s = (vmax - vmin) / denominator;
+    scale[c] = s;
+    zero_point[c] = -t_rint<T>(vmin / s);
+  }
+}
+
+// ---- quantization / fake quantization ---------------------------------------------------
+// IN: element type of `in`; C: type the arithmetic runs in (float for f16/bf16/f32 inputs,
+// double for f64); OUT: storage of the result (same as IN, or int8/uint8 codes).
+enum { kModeSym = 0, kModeAffineFloatZp = 1, kModeAffineU8Zp = 2 };
+
+template<typename C>
+struct QParams {
+  C upper, lower;
+};
+
+template<typename C, int MODE, bool FAKE>
+__device__ __forceinline__ C quant_one(C x, C scale, C zp, C upper, C lower) {
+  C o;
+  if (MODE == kModeSym) {
+    o = t_rint<C>(x / scale);
+  } else {
+    o = t_rint<C>(x / scale + zp);
+  }
+  o = o > upper ? upper : o;
+  o = o < lower ? lower : o;
+  if (FAKE) {
+    if (MODE == kModeSym) {
+      o = o * scale;
+    } else {
+      o = (o - zp) * scale;
+    }
+  }
+  return o;
+}
+
+template<typename S>
+struct Elem;  // load/store helpers keyed by storage type
+template<>
+struct Elem<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template<>
+struct Elem<double> {
+  static __device__ __forceinline__ double ld(const double* p) { return *p; }
+  static __device__ __forceinline__ void st(double* p, double v) { *p = v; }
+};
+template<>
+struct Elem<f16> {
+  static __device__ __forceinline__ float ld(const f16* p) { return (float)*p; }
+  static __device__ __forceinline__ void st(f16* p, float v) { *p = (f16)v; }
+};
+template<>
+struct Elem<bf16> {
+  static __device__ __forceinline__ float ld(const bf16* p) { return bf16_to_float(p->bits); }
+  static __device__ __forceinline__ void st(bf16* p, float v) { p->bits = float_to_bf16(v); }
+};
+template<>
+struct Elem<int8_t> {
+  // codes are integral and inside [-128,127] after the clamp; NaN (0/0) narrows to 0
+  static __device__ __forceinline__ void st(int8_t* p, float v) {
+    *p = (v != v) ? (int8_t)0 : (int8_t)(int)v;
+  }
+};
+template<>
+struct Elem<uint8_t> {
+  static __device__ __forceinline__ void st(uint8_t* p, float v) {
+    *p = (v != v) ? (uint8_t)0 : (uint8_t)(int)v;
+  }
+};
+
+// The zero point as the arithmetic sees it
+template<typename C, int MODE>
+__device__ __forceinline__ C effective_zp(C zp) {
+  if (MODE == kModeAffineU8Zp) {
+    // static_cast<uint8_t>(std::round(zp)): round half away from zero, then narrow
+    const C r = zp < 0 ? -floor(-zp + (C)0.5) : floor(zp + (C)0.5);
+    return (C)(uint8_t)(int)r;
+  }
+  return zp;
+}
+
+// Each lane owns V consecutive elements (V*sizeof(IN) == 16 bytes when the panel allows it).
+template<typename IN, typename C, typename OUT, int MODE, bool FAKE, int V>
+__global__ void __launch_bounds__(256)
+quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
+                const C* __restrict__ zero_point, OUT* __restrict__ out, int64_t elem_cnt,
+                int64_t panel, int64_t scale_size, C upper, C lower, int cambricon) {
+  const int64_t n_packs = elem_cnt / V;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < n_packs; p += step) {
+    const int64_t base = p * V;
+    int64_t ch = base / panel;  // V | panel, so the whole pack lies in one channel
+    if (ch > scale_size - 1) ch = scale_size - 1;
+    C s = scale[ch];
+    if (cambricon) s = (C)exp2((double)(int)s);  // scale = 2^int(shift)
+    const C zp = MODE == kModeSym ? (C)0 : effective_zp<C, MODE>(zero_point[ch]);
+    IN xin[V];
+    if (V * sizeof(IN) == 16) {
+      *reinterpret_cast<u32x4*>(xin) = *reinterpret_cast<const u32x4*>(in + base);
+    } else if (V * sizeof(IN) == 32) {
+      reinterpret_cast<u32x4*>(xin)[0] = reinterpret_cast<const u32x4*>(in + base)[0];
+      reinterpret_cast<u32x4*>(xin)[1] = reinterpret_cast<const u32x4*>(in + base)[1];
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) xin[e] = in[base + e];
+    }
+    OUT r[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const C x = (C)Elem<IN>::ld(&xin[e]);
+      Elem<OUT>::st(&r[e], quant_one<C, MODE, FAKE>(x, s, zp, upper, lower));
+    }
+    if (V * sizeof(OUT) == 16) {
+      *reinterpret_cast<u32x4*>(out + base) = *reinterpret_cast<const u32x4*>(r);
+    } else if (V * sizeof(OUT) == 32) {
+      reinterpret_cast<u32x4*>(out + base)[0] = reinterpret_cast<const u32x4*>(r)[0];
+      reinterpret_cast<u32x4*>(out + base)[1] = reinterpret_cast<const u32x4*>(r)[1];
+    } else if (V * sizeof(OUT) == 8) {
+      *reinterpret_cast<u32x2*>(out + base) = *reinterpret_cast<const u32x2*>(r);
+    } else if (V * sizeof(OUT) == 4) {
+      *reinterpret_cast<uint32_t*>(out + base) = *reinterpret_cast<const uint32_t*>(r);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[base + e] = r[e];
+    }
+  }
+}
+
+inline int grid_for(int64_t items, int block) {
+  int64_t g = (items + block - 1) / block;
+  const int64_t cap = 256 * 32;
+  if (g > cap) g = cap;
+  if (g < 1) g = 1;
+  return (int)g;
+}
+
+template<typename IN, typename C, typename OUT, int MODE, bool FAKE>
+int launch_quant(hipStream_t st, const void* in, const void* scale, const void* zp, void* out,
+                 int64_t elem_cnt, int64_t panel, int64_t scale_size, C upper, C lower,
+                 int cambricon) {
+  constexpr int V = 16 / sizeof(IN);  // 4 floats, 2 doubles, 8 halves
+  const IN* i = static_cast<const IN*>(in);
+  OUT* o = static_cast<OUT*>(out);
+  const C* s = static_cast<const C*>(scale);
+  const C* z = static_cast<const C*>(zp);
+  if (panel % V == 0 && elem_cnt % V == 0) {
+    quantize_kernel<IN, C, OUT, MODE, FAKE, V><<<grid_for(elem_cnt / V, 256), 256, 0, st>>>(
+        i, s, z, o, elem_cnt, panel, scale_size, upper, lower, cambricon);
+  } else {
+    quantize_kernel<IN, C, OUT, MODE, FAKE, 1><<<grid_for(elem_cnt, 256), 256, 0, st>>>(
+        i, s, z, o, elem_cnt, panel, scale_size, upper, lower, cambricon);
+  }
+  return ofq_check_launch();
+}
+
+template<typename IN, typename C, typename OUT, bool FAKE>
+int dispatch_mode(hipStream_t st, const void* in, const void* scale, const void* zp, void* out,
+                  int64_t elem_cnt, int64_t panel, int64_t scale_size, int bits, int scheme,
+                  int formula, int zp_mode) {
+  const bool cambricon = formula == OFQ_FORMULA_CAMBRICON;
+  if (cambricon || scheme == OFQ_SCHEME_SYMMETRIC) {
+    const C upper = (C)(1 << (bits - 1)) - 1;
+    const C lower = -upper - 1;
+    return launch_quant<IN, C, OUT, kModeSym, FAKE>(st, in, scale, zp, out, elem_cnt, panel,
+                                                    scale_size, upper, lower, cambricon);
+  }
+  const C upper = (C)(1 << bits) - 1;
+  const C lower = 0;
+  if (zp_mode == OFQ_ZP_UINT8) {
+    return launch_quant<IN, C, OUT, kModeAffineU8Zp, FAKE>(st, in, scale, zp, out, elem_cnt,
+                                                           panel, scale_size, upper, lower, 0);
+  }
+  return launch_quant<IN, C, OUT, kModeAffineFloatZp, FAKE>(st, in, scale, zp, out, elem_cnt,
+                                                            panel, scale_size, upper, lower, 0);
+}
+
+int check_quant_args(const void* in, const void* scale, const void* zero_point, const void* out,
+                     int64_t elem_cnt, int64_t scale_size, int bits, int scheme, int formula,
+                     int zp_mode) {
+  // attribute domain: oneflow/user/ops/quantization_op.cpp:92-104
+  OFQ_RETURN_IF(bits <= 1 || bits > 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(scheme != OFQ_SCHEME_SYMMETRIC && scheme != OFQ_SCHEME_AFFINE, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(formula != OFQ_FORMULA_GOOGLE && formula != OFQ_FORMULA_CAMBRICON,
+                OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(zp_mode != OFQ_ZP_FLOAT && zp_mode != OFQ_ZP_UINT8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(elem_cnt < 0 || scale_size < 1, OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(scale_size > 1 && (elem_cnt % scale_size) != 0, OFQ_ERR_BAD_SHAPE);
+  if (elem_cnt == 0) return OFQ_OK;
+  OFQ_RETURN_IF(in == nullptr || scale == nullptr || out == nullptr, OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(formula == OFQ_FORMULA_GOOGLE && scheme == OFQ_SCHEME_AFFINE
+                    && zero_point == nullptr,
+                OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(!ofq_aligned16(in) || !ofq_aligned16(out), OFQ_ERR_MISALIGNED);
+  return OFQ_OK;
+}
+
+}  // namespace
+}  // namespace ofq
+
+using namespace ofq;
+
+extern "C" size_t ofq_min_max_observer_workspace_bytes(int in_dtype, int64_t elem_cnt,
+                                                       int64_t channels) {
+  if (channels <= 0 || elem_cnt <= 0) return 0;
+  const size_t es = in_dtype == OFQ_F64 ? 8 : 4;
+  const int64_t inner = elem_cnt / channels;
+  return (size_t)(channels * obs_splits(inner)) * 2 * es;
+}
+
+extern "C" int ofq_min_max_observer(void* stream, const void* in, void* scale, void* zero_point,
+                                    int in_dtype, int64_t elem_cnt, int64_t channels,
+                                    int quantization_bit, int scheme, int formula,
+                                    void* workspace, size_t workspace_bytes) {
+  // attribute domain: oneflow/user/ops/min_max_observer_op.cpp:58-70
+  OFQ_RETURN_IF(quantization_bit <= 1 || quantization_bit > 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(scheme != OFQ_SCHEME_SYMMETRIC && scheme != OFQ_SCHEME_AFFINE, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(formula != OFQ_FORMULA_GOOGLE && formula != OFQ_FORMULA_CAMBRICON,
+                OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(in_dtype != OFQ_F32 && in_dtype != OFQ_F64, OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(channels < 1 || elem_cnt < 1 || elem_cnt % channels != 0, OFQ_ERR_BAD_SHAPE);
+  // per-channel mode is not supported in cambricon scheme: min_max_observer_kernel.cpp:105-108
+  OFQ_RETURN_IF(formula == OFQ_FORMULA_CAMBRICON && channels != 1, OFQ_ERR_UNSUPPORTED);
+  OFQ_RETURN_IF(in == nullptr || scale == nullptr || zero_point == nullptr, OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(!ofq_aligned16(in), OFQ_ERR_MISALIGNED);
+  const size_t need = ofq_min_max_observer_workspace_bytes(in_dtype, elem_cnt, channels);
+  OFQ_RETURN_IF(workspace == nullptr || workspace_bytes < need, OFQ_ERR_WORKSPACE);
+  const int64_t inner = elem_cnt / channels;
+  const int64_t splits = obs_splits(inner);
+  OFQ_RETURN_IF(channels * splits > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int fin_grid = (int)((channels + kObsBlock - 1) / kObsBlock);
+  if (in_dtype == OFQ_F32) {
+    observer_partial<float><<<(int)(channels * splits), kObsBlock, 0, st>>>(
+        static_cast<const float*>(in), inner, splits, static_cast<float*>(workspace));
+    observer_finalize<float><<<fin_grid, kObsBlock, 0, st>>>(
+        static_cast<const float*>(workspace), channels, splits, quantization_bit, scheme, formula,
+        static_cast<float*>(scale), static_cast<float*>(zero_point));
+  } else {
+    observer_partial<double><<<(int)(channels * splits), kObsBlock, 0, st>>>(
+        static_cast<const double*>(in), inner, splits, static_cast<double*>(workspace));
+    observer_finalize<double><<<fin_grid, kObsBlock, 0, st>>>(
+        static_cast<const double*>(workspace), channels, splits, quantization_bit, scheme, formula,
+        static_cast<double*>(scale), static_cast<double*>(zero_point));
+  }
+  return ofq_check_launch();
+}
+
+extern "C" int ofq_quantization(void* stream, const void* in, const void* scale,
+                                const void* zero_point, void* out, int in_dtype, int out_dtype,
+                                int64_t elem_cnt, int64_t scale_size, int quantization_bit,
+                                int scheme, int formula, int zp_mode) {
+  int rc = check_quant_args(in, scale, zero_point, out, elem_cnt, scale_size, quantization_bit,
+                            scheme, formula, zp_mode);
+  if (rc != OFQ_OK || elem_cnt == 0) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t panel = scale_size > 1 ? elem_cnt / scale_size : elem_cnt;
+  const bool integer_out = out_dtype == OFQ_I8 || out_dtype == OFQ_U8;
+  if (integer_out) {
+    // signed codes for the symmetric range [-2^(b-1), 2^(b-1)-1], unsigned for [0, 2^b-1]
+    const bool sym = scheme == OFQ_SCHEME_SYMMETRIC || formula == OFQ_FORMULA_CAMBRICON;
+    OFQ_RETURN_IF(sym != (out_dtype == OFQ_I8), OFQ_ERR_BAD_DTYPE);
+  } else {
+    OFQ_RETURN_IF(out_dtype != in_dtype, OFQ_ERR_BAD_DTYPE);
+  }
+#define OFQ_Q(IN, C, OUT)                                                                       \
+  return dispatch_mode<IN, C, OUT, false>(st, in, scale, zero_point, out, elem_cnt, panel,      \
+                                          scale_size, quantization_bit, scheme, formula, zp_mode)
+  switch (in_dtype) {
+    case OFQ_F32:
+      if (out_dtype == OFQ_I8) OFQ_Q(float, float, int8_t);
+      if (out_dtype == OFQ_U8) OFQ_Q(float, float, uint8_t);
+      OFQ_Q(float, float, float);
+    case OFQ_F64:
+      OFQ_RETURN_IF(integer_out, OFQ_ERR_UNSUPPORTED);
+      OFQ_Q(double, double, double);
+    case OFQ_F16:
+      if (out_dtype == OFQ_I8) OFQ_Q(f16, float, int8_t);
+      if (out_dtype == OFQ_U8) OFQ_Q(f16, float, uint8_t);
+      OFQ_Q(f16, float, f16);
+    case OFQ_BF16:
+      if (out_dtype == OFQ_I8) OFQ_Q(bf16, float, int8_t);
+      if (out_dtype == OFQ_U8) OFQ_Q(bf16, float, uint8_t);
+      OFQ_Q(bf16, float, bf16);
+    default: return OFQ_ERR_BAD_DTYPE;
+  }
+#undef OFQ_Q
+}
+
+extern "C" int ofq_fake_quantization(void* stream, const void* in, const void* scale,
+                                     const void* zero_point, void* out, int in_dtype,
+                                     int64_t elem_cnt, int64_t scale_size, int quantization_bit,
+                                     int scheme, int formula, int zp_mode) {
+  int rc = check_quant_args(in, scale, zero_point, out, elem_cnt, scale_size, quantization_bit,
+                            scheme, formula, zp_mode);
+  if (rc != OFQ_OK || elem_cnt == 0) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t panel = scale_size > 1 ? elem_cnt / scale_size : elem_cnt;
+#define OFQ_FQ(IN, C)                                                                          \
+  return dispatch_mode<IN, C, IN, true>(st, in, scale, zero_point, out, elem_cnt, panel,       \
+                                        scale_size, quantization_bit, scheme, formula, zp_mode)
+  switch (in_dtype) {
+    case OFQ_F32: OFQ_FQ(float, float);
+    case OFQ_F64: OFQ_FQ(double, double);
+    case OFQ_F16: OFQ_FQ(f16, float);
+    case OFQ_BF16: OFQ_FQ(bf16, float);
+    default: return OFQ_ERR_BAD_DTYPE;
+  }
+#undef OFQ_FQ
+}

@@ -1,0 +1,131 @@
+// Shared device-side helpers for the gfx950 kernels: element types, rounding to T, wave and
+// block reductions.  HIP only; compiled with -ffp-contract=off so that `a * b + c` written in
+// source rounds twice -- fused multiply-adds are always spelled out with a builtin.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ofq.h"
+
+namespace ofq {
+
+typedef _Float16 f16;
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kWave = 64;
+
+// bf16 is carried as its bit pattern; arithmetic is fp32 followed by one rounding.
+struct bf16 {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_float(uint16_t b) {
+  return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+// round-to-nearest-even; lowers to v_cvt_pk_bf16_f32 on gfx950
+__device__ __forceinline__ uint16_t float_to_bf16(float f) {
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+
+// Element-type traits: T <-> float, and "arithmetic in T" (one rounding per operation).
+template<typename T>
+struct TT;
+
+template<>
+struct TT<float> {
+  typedef float storage;
+  static constexpr int dtype = OFQ_F32;
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+template<>
+struct TT<f16> {
+  typedef f16 storage;
+  static constexpr int dtype = OFQ_F16;
+  static __device__ __forceinline__ float load(const f16* p) { return (float)*p; }
+  static __device__ __forceinline__ void store(f16* p, float v) { *p = (f16)v; }
+  static __device__ __forceinline__ float round(float v) { return (float)(f16)v; }
+};
+template<>
+struct TT<bf16> {
+  typedef uint16_t storage;
+  static constexpr int dtype = OFQ_BF16;
+  static __device__ __forceinline__ float load(const uint16_t* p) { return bf16_to_float(*p); }
+  static __device__ __forceinline__ void store(uint16_t* p, float v) { *p = float_to_bf16(v); }
+  static __device__ __forceinline__ float round(float v) {
+    return bf16_to_float(float_to_bf16(v));
+  }
+};
+
+// ---- wave64 reductions through DPP-free cross-lane shuffles (ds_bpermute / permlane) ----
+template<typename V, typename Op>
+__device__ __forceinline__ V wave_reduce(V v, Op op) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) { v = op(v, __shfl_xor(v, off, kWave)); }
+  return v;
+}
+
+struct OpSum {
+  template<typename V>
+  __device__ __forceinline__ V operator()(V a, V b) const {
+    return a + b;
+  }
+};
+struct OpMax {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+  __device__ __forceinline__ double operator()(double a, double b) const { return fmax(a, b); }
+};
+struct OpMin {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); }
+  __device__ __forceinline__ double operator()(double a, double b) const { return fmin(a, b); }
+};
+
+// Block-wide reduction; `smem` needs blockDim.x/64 elements; every thread gets the result.
+template<typename V, typename Op>
+__device__ __forceinline__ V block_reduce(V v, Op op, V* smem) {
+  v = wave_reduce(v, op);
+  const int wave = threadIdx.x / kWave;
+  const int nwaves = blockDim.x / kWave;
+  __syncthreads();  // smem may still be read from a previous reduction
+  if ((threadIdx.x & (kWave - 1)) == 0) smem[wave] = v;
+  __syncthreads();
+  V r = smem[0];
+  for (int i = 1; i < nwaves; ++i) r = op(r, smem[i]);
+  return r;
+}
+
+// integer code of element `idx` of a packed tensor (flat index over the UNPACKED shape):
+// 4-bit: element 2i is the high nibble of byte i; an int8 container sign-extends the nibble.
+template<int BITS, bool SIGNED>
+__device__ __forceinline__ int code_at(const uint8_t* q, int64_t idx) {
+  if (BITS == 8) { return SIGNED ? (int)(int8_t)q[idx] : (int)q[idx]; }
+  const uint8_t byte = q[idx >> 1];
+  const int nib = (idx & 1) ? (byte & 0xF) : (byte >> 4);
+  return SIGNED ? ((nib ^ 8) - 8) : nib;
+}
+
+}  // namespace ofq
+
+// host-side launch helpers -------------------------------------------------------------------
+#define OFQ_RETURN_IF(cond, status) \
+  do {                              \
+    if (cond) return (status);      \
+  } while (0)
+
+static inline int ofq_check_launch() {
+  return hipGetLastError() == hipSuccess ? OFQ_OK : OFQ_ERR_LAUNCH;
+}
+static inline bool ofq_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

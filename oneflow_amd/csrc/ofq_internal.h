@@ -1,0 +1,37 @@
+// Launchers shared between translation units of the library (not part of the C ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ofq {
+
+struct LinearArgs {
+  const void* x;        // [m,k] T
+  const void* w;        // [n, k*bits/8] bytes
+  const void* scale;    // [n, k/group_size] T
+  const void* zero;     // same or nullptr
+  const void* bias;     // [n] T or nullptr
+  void* out;            // [m,n] T
+  int t_dtype;          // OFQ_F16 | OFQ_BF16 | OFQ_F32
+  bool w_signed;        // int8 container
+  int bits;             // 4 | 8
+  bool symmetric;
+  int group_dim;        // 0 | 1
+  int64_t group_size;
+  int64_t m, n, k;
+};
+
+// MFMA GEMM with in-tile dequantisation; groups along K.  Returns OFQ_ERR_UNSUPPORTED when the
+// shape does not meet the kernel's tiling constraints (caller falls back).
+bool gemm_wq_supported(const LinearArgs& a);
+int launch_gemm_wq(hipStream_t st, const LinearArgs& a);
+
+// Skinny-M (m <= 16) MFMA GEMV that streams the weights once.
+bool gemv_wq_supported(const LinearArgs& a);
+int launch_gemv_wq(hipStream_t st, const LinearArgs& a);
+
+// Any shape / grouping; one wave per output element.
+int launch_linear_generic(hipStream_t st, const LinearArgs& a);
+
+}  // namespace ofq

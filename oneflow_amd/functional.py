@@ -1,0 +1,350 @@
+"""Host-side mirror of OneFlow's ``flow._C`` entry points for the quantized-inference ops.
+
+Signatures, keyword names, defaults and argument checks follow
+``oneflow/core/functional/functional_api.yaml:1061-1093`` and the functors in
+``oneflow/core/functional/impl/quantization.cpp`` (same messages), so a test written against
+``flow._C.groupwise_dequantize`` / ``flow._C.fused_linear_with_groupwise_quantized_weight`` /
+``flow._C.min_max_observer`` / ``flow._C.quantization`` / ``flow._C.fake_quantization`` reads the
+same against this module.  Tensors are ``torch`` tensors on the GPU; torch is used only to own
+device memory and to name the current stream -- all arithmetic happens in the HIP library behind
+the C ABI of ``include/ofq.h``.
+
+One deliberate difference: the reference functor routes ``m > 8`` of the fused linear through
+``groupwise_dequantize`` + matmul (quantization.cpp:341-350); here every ``m`` goes to the fused
+op, whose kernels cover both regimes.
+"""
+import torch
+
+from . import _lib
+from ._lib import BF16, F16, F32, F64, I8, U8
+
+
+class CheckFailedError(RuntimeError):
+    """Raised where the reference functor's CHECK_OR_RETURN would fail."""
+
+
+def _check(cond, msg):
+    if not cond:
+        raise CheckFailedError(msg)
+
+
+_DT = {
+    torch.float32: F32,
+    torch.float16: F16,
+    torch.bfloat16: BF16,
+    torch.float64: F64,
+    torch.int8: I8,
+    torch.uint8: U8,
+}
+
+
+def _dt(t):
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise CheckFailedError(f"unsupported dtype {t.dtype}") from None
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise CheckFailedError("tensors must live on the GPU: this build has no CPU kernels")
+
+
+def _contig(t):
+    # the runtime hands kernels contiguous inputs (op_interpreter_util.cpp:156)
+    return None if t is None else t.contiguous()
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
+# --------------------------------------------------------------------------------------------
+# groupwise_dequantize: GroupwiseDequantizeFunctor, quantization.cpp:155-220
+# --------------------------------------------------------------------------------------------
+def groupwise_dequantize(in_, scale, *, zero=None, num_bits=8, symmetric=True, group_dim=-1,
+                         group_size=-1):
+    _check(num_bits in (4, 8), "num_bits should be 4 or 8.")
+    nd = in_.dim()
+    _check(nd >= 1, "The number of dimensions for tensor in should be greater than or equal to 1.")
+    gd = nd + group_dim if group_dim < 0 else group_dim
+    _check(0 <= gd < nd, f"group_dim should be in range [-{nd},{nd}).")
+    per = 8 // num_bits
+    group_dim_size = in_.shape[gd] * (per if gd == nd - 1 else 1)
+    gs = group_dim_size if group_size < 0 else group_size
+    _check(0 < gs <= group_dim_size, f"group_size should be in range (0,{group_dim_size}].")
+    _check(group_dim_size % gs == 0, f"group_size should be a divisor of {group_dim_size}.")
+    num_groups = group_dim_size // gs
+    if symmetric:
+        _check(in_.dtype in (torch.uint8, torch.int8),
+               "The dtype of tensor in should be int8 or uint8.")
+    else:
+        _check(in_.dtype == torch.uint8, "The dtype of tensor in should be uint8.")
+    _check(scale.dim() == nd,
+           "The number of dimensions of tensor scale should be equal to tensor in.")
+    for i in range(nd):
+        if i == gd:
+            _check(scale.shape[i] == num_groups,
+                   f"The size of the {i}-th dimension of tensor scale should be equal to {num_groups}")
+        elif i == nd - 1:
+            _check(scale.shape[i] == in_.shape[i] * per,
+                   f"The size of the {i}-th dimension of tensor scale should be equal to "
+                   f"{in_.shape[i] * per}.")
+        else:
+            _check(scale.shape[i] == in_.shape[i],
+                   f"The size of the {i}-th dimension of tensor scale should be equal to tensor in.")
+    if not symmetric:
+        _check(zero is not None, "When symmetric is False, tensor zero should be specified.")
+        _check(zero.dtype == scale.dtype,
+               "The dtype of the zero tensor should be the same as the scale tensor.")
+        _check(zero.shape == scale.shape,
+               "The shape of zero tensor should be equal to tensor scale.")
+    else:
+        _check(zero is None, "When symmetric is True, tensor zero should be None.")
+    # kernels are registered on the dtype of scale (groupwise_quantization_kernels.cu:456-463);
+    # bf16 is added here
+    _check(scale.dtype in (torch.float16, torch.float32, torch.bfloat16),
+           f"no groupwise_dequantize kernel for scale dtype {scale.dtype}")
+    _require_gpu(in_, scale, zero)
+    in_, scale, zero = _contig(in_), _contig(scale), _contig(zero)
+    out_shape = list(in_.shape)
+    out_shape[-1] *= per
+    out = torch.empty(out_shape, dtype=scale.dtype, device=in_.device)
+    outer = 1
+    for d in out_shape[:gd]:
+        outer *= d
+    outer *= num_groups
+    inner = 1
+    for d in out_shape[gd + 1:]:
+        inner *= d
+    st = _lib.lib().ofq_groupwise_dequantize(
+        _stream(in_), _ptr(in_), _ptr(scale), _ptr(zero), _ptr(out), _dt(in_), _dt(scale),
+        num_bits, int(symmetric), outer, gs, inner)
+    _lib.check("ofq_groupwise_dequantize", st)
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# fused_linear_with_groupwise_quantized_weight:
+# FusedLinearWithGroupwiseQuantizedWeightFunctor, quantization.cpp:264-372
+# --------------------------------------------------------------------------------------------
+def fused_linear_with_groupwise_quantized_weight(x, w, w_scale, *, w_zero=None, b=None,
+                                                 num_bits=8, symmetric=True, group_dim=-1,
+                                                 group_size=-1):
+    _check(x.dim() >= 2,
+           "The number of dimensions for tensor x should be greater than or equal to 2.")
+    k = x.shape[-1]
+    m = x.numel() // k if k else 0
+    _check(num_bits in (4, 8), "num_bits should be 4 or 8.")
+    _check(w.dim() == 2, "The number of dimensions for tensor w should be equal to 2.")
+    per = 8 // num_bits
+    _check(k % per == 0,
+           "The size of the last dimension of x should be a multiple of (8/num_bits).")
+    _check(w.shape[1] == k // per,
+           f"The size of second dimension of tensor w should be equal to {k // per}")
+    n = w.shape[0]
+    gd = 2 + group_dim if group_dim < 0 else group_dim
+    _check(gd in (0, 1), "group_dim should be in range [-2,2).")
+    group_dim_size = n if gd == 0 else k
+    gs = group_dim_size if group_size < 0 else group_size
+    _check(0 < gs <= group_dim_size, f"group_size should be in range (0,{group_dim_size}].")
+    _check(group_dim_size % gs == 0, f"group_size should be a divisor of {group_dim_size}.")
+    num_groups = group_dim_size // gs
+    if symmetric:
+        _check(w.dtype in (torch.uint8, torch.int8),
+               "The dtype of tensor w should be int8 or uint8.")
+    else:
+        _check(w.dtype == torch.uint8, "The dtype of tensor w should be uint8.")
+    _check(w_scale.dim() == 2,
+           "The number of dimensions of tensor w_scale should be equal to 2.")
+    for i in range(2):
+        if i == gd:
+            _check(w_scale.shape[i] == num_groups,
+                   f"The size of the {i}-th dimension of tensor w_scale should be equal to "
+                   f"{num_groups}")
+        elif i == 1:
+            _check(w_scale.shape[i] == k,
+                   f"The size of the {i}-th dimension of tensor w_scale should be equal to {k}.")
+        else:
+            _check(w_scale.shape[i] == w.shape[i],
+                   f"The size of the {i}-th dimension of tensor w_scale should be equal to tensor w.")
+    _check(w_scale.dtype == x.dtype,
+           "The dtype of the w_scale tensor should be the same as the x tensor.")
+    if not symmetric:
+        _check(w_zero is not None, "When symmetric is False, tensor w_zero should be specified.")
+        _check(w_zero.dtype == w_scale.dtype,
+               "The dtype of the w_zero tensor should be the same as the w_scale tensor.")
+        _check(w_zero.shape == w_scale.shape,
+               "The shape of w_zero tensor should be equal to tensor w_scale.")
+    else:
+        _check(w_zero is None, "When symmetric is True, tensor w_zero should be None.")
+    if b is not None:
+        _check(b.dtype == x.dtype, "The dtype of the b tensor should be the same as the x tensor.")
+        _check(b.dim() == 1, "The number of dimensions for tensor b should be equal to 1.")
+        _check(b.shape[0] == n,
+               "The size of first dimension of tensor b should be equal to the size of first "
+               "dimension of tensor w")
+    _check(x.dtype in (torch.float16, torch.float32, torch.bfloat16),
+           f"no fused_linear_with_groupwise_quantized_weight kernel for dtype {x.dtype}")
+    _require_gpu(x, w, w_scale, w_zero, b)
+    x, w, w_scale, w_zero, b = map(_contig, (x, w, w_scale, w_zero, b))
+    out = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=x.dtype, device=x.device)
+    L = _lib.lib()
+    ws_bytes = L.ofq_fused_linear_gq_workspace_bytes(_dt(w), _dt(x), num_bits, int(symmetric), gd,
+                                                     gs, m, n, k)
+    ws = _workspace(ws_bytes, x.device) if ws_bytes else None
+    st = L.ofq_fused_linear_gq(_stream(x), _ptr(x), _ptr(w), _ptr(w_scale), _ptr(w_zero), _ptr(b),
+                               _ptr(out), _dt(w), _dt(x), num_bits, int(symmetric), gd, gs, m, n,
+                               k, _ptr(ws), ws_bytes)
+    _lib.check("ofq_fused_linear_gq", st)
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# min_max_observer / quantization / fake_quantization
+# functors quantization.cpp:34-153; attribute checks oneflow/user/ops/min_max_observer_op.cpp:58-70,
+# quantization_op.cpp:92-104
+# --------------------------------------------------------------------------------------------
+def _check_quant_attrs(quantization_formula, quantization_bit, quantization_scheme):
+    _check(1 < quantization_bit <= 8, "quantization_bit should be in range (1, 8].")
+    _check(quantization_scheme in ("symmetric", "affine"),
+           "quantization_scheme should be symmetric or affine.")
+    _check(quantization_formula in ("google", "cambricon"),
+           "quantization_formula should be google or cambricon.")
+
+
+def min_max_observer(in_, quantization_formula="google", quantization_bit=8,
+                     quantization_scheme="symmetric", per_layer_quantization=True):
+    """Returns ``(scale, zero_point)``; shape ``[1]`` per layer or ``[in.shape[0]]`` per channel
+    (min_max_observer_op.cpp:21-38)."""
+    _check_quant_attrs(quantization_formula, quantization_bit, quantization_scheme)
+    _check(in_.dtype in (torch.float32, torch.float64),
+           f"no min_max_observer kernel for dtype {in_.dtype}")
+    if quantization_formula == "cambricon":
+        _check(per_layer_quantization, " per-channel mode is not supported in cambricon scheme")
+    _require_gpu(in_)
+    in_ = _contig(in_)
+    channels = 1 if per_layer_quantization else in_.shape[0]
+    scale = torch.empty(channels, dtype=in_.dtype, device=in_.device)
+    zero_point = torch.empty(channels, dtype=in_.dtype, device=in_.device)
+    L = _lib.lib()
+    ws_bytes = L.ofq_min_max_observer_workspace_bytes(_dt(in_), in_.numel(), channels)
+    ws = _workspace(ws_bytes, in_.device)
+    st = L.ofq_min_max_observer(_stream(in_), _ptr(in_), _ptr(scale), _ptr(zero_point), _dt(in_),
+                                in_.numel(), channels, quantization_bit,
+                                _lib.SCHEME[quantization_scheme],
+                                _lib.FORMULA[quantization_formula], _ptr(ws), ws_bytes)
+    _lib.check("ofq_min_max_observer", st)
+    return scale, zero_point
+
+
+def _quant_common(fn_name, in_, scale, zero_point, quantization_formula, quantization_bit,
+                  quantization_scheme, out_dtype, zp_mode):
+    _check_quant_attrs(quantization_formula, quantization_bit, quantization_scheme)
+    _check(in_.dtype in (torch.float32, torch.float64, torch.float16, torch.bfloat16),
+           f"no {fn_name} kernel for dtype {in_.dtype}")
+    param_dtype = in_.dtype if in_.dtype in (torch.float32, torch.float64) else torch.float32
+    _check(scale.dtype == param_dtype, f"scale should have dtype {param_dtype}")
+    _check(zero_point is None or zero_point.dtype == param_dtype,
+           f"zero_point should have dtype {param_dtype}")
+    # per-channel iff scale has more than one element (quantization_op.cpp:66-69)
+    if scale.numel() > 1:
+        _check(scale.numel() == in_.shape[0], "scale.elem_cnt() should equal in.shape[0]")
+        _check(zero_point is None or zero_point.numel() == in_.shape[0],
+               "zero_point.elem_cnt() should equal in.shape[0]")
+    _require_gpu(in_, scale, zero_point)
+    return _contig(in_), _contig(scale), _contig(zero_point)
+
+
+def quantization(in_, scale, zero_point, quantization_formula="google", quantization_bit=8,
+                 quantization_scheme="symmetric", *, out_dtype=None, zp_mode="float"):
+    """``out_dtype`` (extension): ``torch.int8`` / ``torch.uint8`` to get integer codes instead
+    of codes stored in the input dtype.  ``zp_mode`` selects how an affine zero point is read:
+    ``"float"`` (the CUDA kernel's rule) or ``"uint8"`` (the CPU kernel's rule)."""
+    in_, scale, zero_point = _quant_common("quantization", in_, scale, zero_point,
+                                           quantization_formula, quantization_bit,
+                                           quantization_scheme, out_dtype, zp_mode)
+    out = torch.empty(in_.shape, dtype=out_dtype or in_.dtype, device=in_.device)
+    st = _lib.lib().ofq_quantization(
+        _stream(in_), _ptr(in_), _ptr(scale), _ptr(zero_point), _ptr(out), _dt(in_), _dt(out),
+        in_.numel(), scale.numel(), quantization_bit, _lib.SCHEME[quantization_scheme],
+        _lib.FORMULA[quantization_formula], _lib.ZP_MODE[zp_mode])
+    _lib.check("ofq_quantization", st)
+    return out
+
+
+def fake_quantization(in_, scale, zero_point, quantization_formula="google", quantization_bit=8,
+                      quantization_scheme="symmetric", *, zp_mode="float"):
+    in_, scale, zero_point = _quant_common("fake_quantization", in_, scale, zero_point,
+                                           quantization_formula, quantization_bit,
+                                           quantization_scheme, None, zp_mode)
+    out = torch.empty_like(in_)
+    st = _lib.lib().ofq_fake_quantization(
+        _stream(in_), _ptr(in_), _ptr(scale), _ptr(zero_point), _ptr(out), _dt(in_), in_.numel(),
+        scale.numel(), quantization_bit, _lib.SCHEME[quantization_scheme],
+        _lib.FORMULA[quantization_formula], _lib.ZP_MODE[zp_mode])
+    _lib.check("ofq_fake_quantization", st)
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# Ops named by the task but absent from the reference tree
+# --------------------------------------------------------------------------------------------
+def fused_layer_norm_min_max_observer(x, gamma=None, beta=None, epsilon=1e-5, quantization_bit=8):
+    """LayerNorm over the last axis + per-tensor symmetric observer of the result.
+    Returns ``(y, scale, zero_point)`` with fp32 ``scale`` / ``zero_point`` of shape ``[1]``."""
+    _check(1 < quantization_bit <= 8, "quantization_bit should be in range (1, 8].")
+    _check(x.dtype in (torch.float16, torch.bfloat16, torch.float32),
+           f"no fused_layer_norm_min_max_observer kernel for dtype {x.dtype}")
+    cols = x.shape[-1]
+    for name, p in (("gamma", gamma), ("beta", beta)):
+        if p is not None:
+            _check(p.dtype == x.dtype and p.numel() == cols,
+                   f"{name} should have the dtype of x and x.shape[-1] elements")
+    _require_gpu(x, gamma, beta)
+    x, gamma, beta = _contig(x), _contig(gamma), _contig(beta)
+    rows = x.numel() // cols
+    y = torch.empty_like(x)
+    scale = torch.empty(1, dtype=torch.float32, device=x.device)
+    zero_point = torch.empty(1, dtype=torch.float32, device=x.device)
+    L = _lib.lib()
+    ws_bytes = L.ofq_fused_layer_norm_min_max_observer_workspace_bytes(_dt(x), rows, cols)
+    ws = _workspace(ws_bytes, x.device)
+    st = L.ofq_fused_layer_norm_min_max_observer(
+        _stream(x), _ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(scale), _ptr(zero_point),
+        _dt(x), rows, cols, float(epsilon), quantization_bit, _ptr(ws), ws_bytes)
+    _lib.check("ofq_fused_layer_norm_min_max_observer", st)
+    return y, scale, zero_point
+
+
+def matmul_quant(a, b, a_scale, b_scale, bias=None, out_dtype=torch.float16):
+    """int8 ``a[m,k]`` x int8 ``b[n,k]`` -> ``out_dtype[m,n]``; exact int32 accumulation, then
+    ``acc * (a_scale * b_scale[n]) + bias[n]``."""
+    _check(a.dtype == torch.int8 and b.dtype == torch.int8, "a and b should be int8")
+    _check(a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1],
+           "a should be [m,k] and b [n,k]")
+    _check(a_scale.dtype == torch.float32 and a_scale.numel() == 1,
+           "a_scale should be one float32")
+    _check(b_scale.dtype == torch.float32 and b_scale.numel() == b.shape[0],
+           "b_scale should be float32 with b.shape[0] elements")
+    if bias is not None:
+        _check(bias.dtype == out_dtype and bias.numel() == b.shape[0],
+               "bias should have the output dtype and b.shape[0] elements")
+    _require_gpu(a, b, a_scale, b_scale, bias)
+    a, b, a_scale, b_scale, bias = map(_contig, (a, b, a_scale, b_scale, bias))
+    m, k = a.shape
+    n = b.shape[0]
+    out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    st = _lib.lib().ofq_matmul_quant(_stream(a), _ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale),
+                                     _ptr(bias), _ptr(out), _dt(out), m, n, k)
+    _lib.check("ofq_matmul_quant", st)
+    return out

@@ -1,0 +1,99 @@
+"""Dynamic int8 activation path: fused_layer_norm_min_max_observer -> quantization (int8 codes)
+-> matmul_quant.  These two ops are absent from the reference tree; the oracle composes them
+from reference rules, so parity with the reference itself is unpinned (see oracle/ofq_oracle.c).
+Bars used here: LayerNorm output within 1 ulp of T of the oracle (mean/variance are accumulated
+in fp32 on the GPU and in fp64 in the oracle), codes bit-exact GIVEN the same y and scale, int32
+accumulation exact, scaled output within 1 ulp of T."""
+import numpy as np
+import pytest
+
+import helpers as H
+from oracle import ofq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg5_inputs(rows=2048, cols=4096, t="f16"):
+    x = H.as_T(H.rng_for(5, 0).standard_normal((rows, cols)).astype(np.float32), t)
+    gamma = H.as_T((1 + 0.1 * H.rng_for(5, 1).standard_normal(cols)).astype(np.float32), t)
+    beta = H.as_T((0.1 * H.rng_for(5, 2).standard_normal(cols)).astype(np.float32), t)
+    return x, gamma, beta
+
+
+@pytest.mark.parametrize("t,rows,cols", [("f16", 2048, 4096), ("bf16", 64, 4096), ("f32", 33, 1000),
+                                         ("f16", 7, 8200), ("f16", 5, 24)])
+def test_layer_norm_observer(t, rows, cols):
+    import oneflow_amd as flow
+    x, gamma, beta = _cfg5_inputs(rows, cols, t)
+    y_ref, s_ref, z_ref = O.layer_norm_min_max_observer(x, gamma, beta, 1e-5, 8)
+    y, s, z = flow._C.fused_layer_norm_min_max_observer(H.to_torch(x), H.to_torch(gamma),
+                                                        H.to_torch(beta), 1e-5, 8)
+    y_np = H.to_numpy(y)
+    yf, yr = O.to_f32(y_np).astype(np.float64), O.to_f32(y_ref).astype(np.float64)
+    # within one ulp of T everywhere; almost all elements identical
+    assert (np.abs(yf - yr) <= H.ulp_of(yr, t) * 1.0001).all()
+    assert (yf != yr).mean() < 0.02
+    # scale is exactly absmax(y_gpu)/127 in fp32, zero_point 0
+    expect = np.float32(np.abs(O.to_f32(y_np)).max()) / np.float32(127.0)
+    assert H.to_numpy(s)[0] == expect and H.to_numpy(z)[0] == 0.0
+    assert abs(float(H.to_numpy(s)[0]) - float(s_ref[0])) <= 2e-3 * float(s_ref[0])
+
+
+def test_layer_norm_closed_form():
+    """Rows of +-c have mean 0 and variance c^2: y = +-c/sqrt(c^2+eps) * gamma + beta."""
+    import oneflow_amd as flow
+    cols = 512
+    x = np.tile(np.array([1.5, -1.5], np.float32), cols // 2)[None, :].repeat(3, 0)
+    y, s, z = flow._C.fused_layer_norm_min_max_observer(H.to_torch(x), None, None, 1e-5, 8)
+    expect = np.float32(1.5) * (np.float32(1.0) / np.sqrt(np.float32(2.25) + np.float32(1e-5)))
+    y = H.to_numpy(y)
+    assert np.allclose(np.abs(y), expect, rtol=2e-7, atol=0) and np.array_equal(np.sign(y), np.sign(x))
+    assert np.isclose(H.to_numpy(s)[0], expect / 127.0, rtol=3e-7)
+
+
+def test_dynamic_quantize_and_matmul_quant():
+    import oneflow_amd as flow
+    import torch
+    m, n, k = 2048, 11008, 4096
+    x, gamma, beta = _cfg5_inputs(m, k, "f16")
+    y, s, z = flow._C.fused_layer_norm_min_max_observer(H.to_torch(x), H.to_torch(gamma),
+                                                        H.to_torch(beta), 1e-5, 8)
+    a = flow._C.quantization(y, s, z, "google", 8, "symmetric", out_dtype=torch.int8)
+    a_np = H.to_numpy(a)
+    # codes: bit-exact against the oracle GIVEN the same y and scale
+    a_ref = O.quantize_to_int8(H.to_numpy(y), H.to_numpy(s), 8)
+    assert np.array_equal(a_np, a_ref)
+    assert np.abs(a_np.astype(np.int32)).max() == 127
+    w = H.rng_for(5, 3).integers(-127, 128, size=(n, k)).astype(np.int8)
+    w_scale = H.rng_for(5, 4).uniform(1e-3, 1e-2, size=n).astype(np.float32)
+    out = H.to_numpy(flow._C.matmul_quant(a, H.to_torch(w), s, H.to_torch(w_scale), None,
+                                          torch.float16))
+    rows = np.array([0, 31, 32, 127, 128, 1000, 2047])
+    cols = np.concatenate([np.arange(0, 64), np.arange(6000, 6064), np.arange(n - 64, n)])
+    # exact integer accumulation (int64 brute force) then the fp32 epilogue, rounded once
+    acc = a_np[rows].astype(np.int64) @ w[cols].astype(np.int64).T
+    sc = (H.to_numpy(s)[0] * w_scale[cols]).astype(np.float32)
+    expect = (acc.astype(np.float32) * sc[None, :]).astype(np.float16)
+    got = out[np.ix_(rows, cols)]
+    assert np.array_equal(got.view(np.uint16), expect.view(np.uint16))
+    ref = O.matmul_quant(a_np[rows], w[cols], H.to_numpy(s), w_scale[cols], None, np.float16)
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("m,n,k,t", [(1, 16, 128, "f32"), (100, 200, 256, "f16"), (130, 33, 384, "bf16")])
+def test_matmul_quant_small_exact(m, n, k, t):
+    import oneflow_amd as flow
+    import torch
+    rng = np.random.Generator(np.random.PCG64(m * 1000 + n))
+    a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, size=(n, k)).astype(np.int8)
+    a_scale = np.array([0.0123], np.float32)
+    b_scale = rng.uniform(1e-3, 1e-2, size=n).astype(np.float32)
+    bias = H.as_T(rng.standard_normal(n).astype(np.float32), t)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[t]
+    got = H.to_numpy(flow._C.matmul_quant(H.to_torch(a), H.to_torch(b), H.to_torch(a_scale),
+                                          H.to_torch(b_scale), H.to_torch(bias), tdt))
+    ref = O.matmul_quant(a, b, a_scale, b_scale, bias, {"f32": np.float32, "f16": np.float16,
+                                                        "bf16": np.uint16}[t])
+    assert np.array_equal(got.view(np.uint16 if t != "f32" else np.uint32),
+                          ref.view(np.uint16 if t != "f32" else np.uint32))

@@ -1,0 +1,125 @@
+"""fused_linear_with_groupwise_quantized_weight on the GPU against the oracle composition
+(dequantize in T -> matmul with fp32 accumulation -> + bias -> round to T).
+Tolerance (stated contract): rel-L2 <= 1e-3 and max-abs <= 2e-2 (see helpers.assert_linear_parity
+for how the absolute bound is read when one ulp of T is larger than 2e-2)."""
+import numpy as np
+import pytest
+
+import helpers as H
+from oracle import ofq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# (num_bits, m, k, n, group_dim, group_size): test_groupwise_quantization.py:209-220
+REFERENCE_CASES = [
+    (8, 1, 64, 128, 0, 128), (8, 1, 64, 128, 1, 64), (8, 16, 64, 128, 0, 128),
+    (8, 16, 64, 128, 1, 64), (8, 1, 63, 127, 0, 127), (8, 1, 63, 127, 1, 63),
+    (8, 1, 256, 512, 0, 64), (8, 1, 256, 512, 1, 64), (4, 1, 256, 512, 0, 512),
+    (4, 1, 256, 512, 1, 256), (4, 1, 256, 512, 0, 64), (4, 1, 256, 512, 1, 64),
+]
+VARIANTS = [(True, np.int8), (True, np.uint8), (False, np.uint8)]
+
+
+def _run(x, w, scale, zero, b, num_bits, symmetric, group_dim, group_size):
+    import oneflow_amd as flow
+    out = flow._C.fused_linear_with_groupwise_quantized_weight(
+        H.to_torch(x), H.to_torch(w), H.to_torch(scale), w_zero=H.to_torch(zero), b=H.to_torch(b),
+        num_bits=num_bits, symmetric=symmetric, group_dim=group_dim, group_size=group_size)
+    return H.to_numpy(out)
+
+
+@pytest.mark.parametrize("num_bits,m,k,n,group_dim,group_size", REFERENCE_CASES)
+@pytest.mark.parametrize("t", ["f16", "f32", "bf16"])
+def test_reference_cases(num_bits, m, k, n, group_dim, group_size, t):
+    rng = np.random.Generator(np.random.PCG64(hash((num_bits, m, k, n, group_dim, group_size)) % 2**32))
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32) / 10, t)
+    wf = rng.standard_normal((n, k)).astype(np.float32) / 10
+    b = H.as_T(rng.standard_normal(n).astype(np.float32) / 10, t)
+    for symmetric, qdt in VARIANTS:
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, group_dim, group_size, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, group_dim, group_size)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, group_dim, group_size)
+        H.assert_linear_parity(got, ref, t, f"{symmetric} {qdt}")
+        # the reference test's own criterion
+        assert np.allclose(O.to_f32(got), O.to_f32(ref), atol=1e-2, rtol=1e-2)
+
+
+def _decode_inputs(m, n, k, container):
+    x = H.as_T(H.rng_for(3, 0).standard_normal((m, k)).astype(np.float32), "f16")
+    if container == np.int8:
+        codes = H.rng_for(3, 1).integers(-7, 8, size=(n, k)).astype(np.int8)
+    else:
+        codes = H.rng_for(3, 1).integers(0, 15, size=(n, k)).astype(np.uint8)
+    w = H.pack_int4(codes)
+    scale = H.as_T(H.rng_for(3, 2).uniform(1e-3, 1e-2, size=(n, k // 128)).astype(np.float32), "f16")
+    b = H.as_T((H.rng_for(3, 3).standard_normal(n) * 0.01).astype(np.float32), "f16")
+    return x, w, scale, b
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008)])
+@pytest.mark.parametrize("m", [1, 4, 8])
+@pytest.mark.parametrize("container", [np.int8, np.uint8])
+def test_decode_w4a16_llama_shapes(m, n, k, container):
+    """Symmetric int4, g=128 along K, fp16, Llama-7B q/o, gate/up and down shapes."""
+    x, w, scale, b = _decode_inputs(m, n, k, container)
+    ref = O.fused_linear(x, w, scale, None, b, 4, True, 1, 128)
+    got = _run(x, w, scale, None, b, 4, True, 1, 128)
+    r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k}")
+    assert r < 2e-4  # the kernel forms w~ exactly as the oracle does; only the sum order differs
+
+
+def test_decode_m_invariance_and_integer_case():
+    """Row i of an m=8 call equals the m=1 call on that row (same kernel arithmetic per row), and
+    with all scales 1 the op is an exact integer dot product (closed form, no oracle)."""
+    x8, w, scale, b = _decode_inputs(8, 4096, 4096, np.int8)
+    out8 = _run(x8, w, scale, None, b, 4, True, 1, 128)
+    for i in (0, 5):
+        out1 = _run(x8[i:i + 1], w, scale, None, b, 4, True, 1, 128)
+        assert np.array_equal(out1[0].view(np.uint16), out8[i].view(np.uint16))
+    # integer case: x small integers, scale 1, |sum| < 2048 is exact in fp16
+    rng = np.random.Generator(np.random.PCG64(7))
+    k, n = 256, 64
+    xi = rng.integers(-2, 3, size=(3, k)).astype(np.float16)
+    codes = rng.integers(-7, 8, size=(n, k)).astype(np.int8)
+    ones = np.ones((n, k // 128), dtype=np.float16)
+    got = _run(xi, H.pack_int4(codes), ones, None, None, 4, True, 1, 128)
+    exact = xi.astype(np.int64) @ codes.astype(np.int64).T
+    assert np.array_equal(got.astype(np.int64), exact)
+
+
+@pytest.mark.parametrize("t", ["bf16", "f16"])
+def test_prefill_w8a16_sampled(t):
+    """x [2048,4096], W uint8 asymmetric [11008,4096], g=64; the GPU computes the full output, the
+    oracle a sample of rows and columns (the scalar composition on the full shape takes minutes)."""
+    m, n, k, g = 2048, 11008, 4096, 64
+    x = H.as_T(H.rng_for(4, 0).standard_normal((m, k)).astype(np.float32), t)
+    w = H.rng_for(4, 1).integers(0, 256, size=(n, k), dtype=np.uint8)
+    scale = H.as_T(H.rng_for(4, 2).uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float32), t)
+    zero = H.as_T(H.rng_for(4, 3).uniform(120, 136, size=(n, k // g)).astype(np.float32), t)
+    got = _run(x, w, scale, zero, None, 8, False, 1, g)
+    assert got.shape == (m, n)
+    rows = np.array([0, 1, 127, 128, 255, 256, 1000, 1023, 1024, 2047])
+    cols = np.concatenate([np.arange(0, 40), np.arange(5000, 5040), np.arange(n - 40, n)])
+    ref = O.fused_linear(x[rows], w[cols], scale[cols], zero[cols], None, 8, False, 1, g)
+    H.assert_linear_parity(got[np.ix_(rows, cols)], ref, t, f"prefill {t}")
+    # linearity in x: doubling x doubles every output exactly (power-of-two scaling is exact)
+    x2 = H.as_T(O.to_f32(x) * 2.0, t)
+    got2 = _run(x2, w, scale, zero, None, 8, False, 1, g)
+    assert np.array_equal(O.to_f32(got2), O.to_f32(got) * 2.0)
+
+
+@pytest.mark.parametrize("m", [17, 100, 130])
+@pytest.mark.parametrize("num_bits,symmetric,qdt", [(4, True, np.int8), (4, False, np.uint8),
+                                                    (8, True, np.uint8)])
+def test_prefill_ragged_m_and_n(m, num_bits, symmetric, qdt):
+    """m and n that are not multiples of the tile sizes."""
+    rng = np.random.Generator(np.random.PCG64(m * 31 + num_bits))
+    n, k, g = 200, 256, 64
+    for t in ("f16", "bf16"):
+        x = H.as_T(rng.standard_normal((m, k)).astype(np.float32) / 10, t)
+        wf = rng.standard_normal((n, k)).astype(np.float32) / 10
+        b = H.as_T(rng.standard_normal(n).astype(np.float32) / 10, t)
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, g, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        H.assert_linear_parity(got, ref, t, f"m={m} {t}")
