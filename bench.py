@@ -1,0 +1,358 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference hot path on one MI355X.
+
+Headline workload (what `value` measures): one decode step (m = 1) through every quantized
+linear layer of a Llama-7B-shaped model -- per decoder layer four 4096x4096, two 11008x4096 and one
+4096x11008 `fused_linear_with_groupwise_quantized_weight` calls, symmetric int4 weights packed two
+per byte, group_size 128 along K, fp16 scales, fp16 bias -- over `--layers` layers with DISTINCT
+weights (32 layers = 3.3 GB of packed weights, far beyond L2 + Infinity Cache, so every launch
+streams its weights from HBM).  value = algorithmic bytes of all launches / wall time of the step.
+
+The same JSON line carries
+  roofline      for the dominant kernel (the K=4096 instance of the MFMA GEMV): algorithmic bytes
+                per launch / average launch duration, timed live with events on the launch stream
+                over a region that contains only that kernel's launches;
+  cpu_baseline  the CPU oracle (scalar C port of the reference composition dequantize -> matmul)
+                on one decoder layer's seven GEMVs, single thread;
+  secondary     the other BASELINE configurations (prefill W8A16 GEMM at m=2048, dequantize,
+                LayerNorm+observer / quantize, int8 matmul_quant, observer/quantize of a
+                4096x4096 fp32 weight), each with its own roofline fraction.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "i8": 5000.0}
+
+LLAMA7B_LAYER = [  # (name, n, k, count per decoder layer)
+    ("qkvo", 4096, 4096, 4),
+    ("gate_up", 11008, 4096, 2),
+    ("down", 4096, 11008, 1),
+]
+
+
+def gemv_bytes(m, n, k, g=128, bits=4, tsize=2, asym=False):
+    """Algorithmic bytes of one fused linear: each tensor once, packed sizes."""
+    b = n * k * bits // 8 + n * (k // g) * tsize * (2 if asym else 1)
+    return b + m * k * tsize + n * tsize + m * n * tsize
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--m", type=int, default=1, help="decode batch (rows of x), 1..16")
+    ap.add_argument("--no-graph", action="store_true", help="launch directly instead of replaying a HIP graph")
+    ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build is single-GPU by design (the path has no collectives); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import oneflow_amd
+    from oneflow_amd import _lib
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    torch.manual_seed(1234)
+    M = args.m
+
+    # ---- synthetic Llama-7B-shaped int4 weights, distinct per layer ----------------------------
+    layers = []
+    for _ in range(args.layers):
+        mats = []
+        for name, n, k, cnt in LLAMA7B_LAYER:
+            for _c in range(cnt):
+                w = torch.randint(-128, 128, (n, k // 2), dtype=torch.int8, device=dev)
+                scale = torch.empty((n, k // 128), dtype=torch.float16, device=dev).uniform_(1e-3, 1e-2)
+                bias = (torch.randn(n, device=dev) * 0.01).to(torch.float16)
+                out = torch.empty((M, n), dtype=torch.float16, device=dev)
+                mats.append((name, n, k, w, scale, bias, out))
+        layers.append(mats)
+    x_by_k = {k: torch.randn((M, k), device=dev).to(torch.float16) for k in (4096, 11008)}
+
+    def launch(mat):
+        name, n, k, w, scale, bias, out = mat
+        st = L.ofq_fused_linear_gq(torch.cuda.current_stream().cuda_stream, x_by_k[k].data_ptr(),
+                                   w.data_ptr(), scale.data_ptr(), None, bias.data_ptr(),
+                                   out.data_ptr(), _lib.I8, _lib.F16, 4, 1, 1, 128, M, n, k, None, 0)
+        if st != 0:
+            raise RuntimeError(f"ofq_fused_linear_gq status {st}")
+
+    def step_all():
+        for mats in layers:
+            for mat in mats:
+                launch(mat)
+
+    def step_k4096():
+        for mats in layers:
+            for mat in mats:
+                if mat[2] == 4096:
+                    launch(mat)
+
+    def make_runner(fn):
+        if args.no_graph:
+            return fn
+        # warm up outside capture, then capture the launches into one HIP graph
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g.replay
+
+    def time_region(run, steps, warmup):
+        for _ in range(warmup):
+            run()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return e0.elapsed_time(e1), wall_ms
+
+    bytes_step = sum(gemv_bytes(M, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER) * args.layers
+    launches_step = sum(cnt for *_, cnt in LLAMA7B_LAYER) * args.layers
+    run_all = make_runner(step_all)
+    ev_ms, wall_ms = time_region(run_all, args.steps, args.warmup)
+    ms_per_step = wall_ms / args.steps
+    value = bytes_step / (ms_per_step * 1e-3) / 1e9
+
+    # ---- roofline of the dominant kernel: only the K=4096 GEMV launches ------------------------
+    bytes_k4096 = sum(gemv_bytes(M, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER if k == 4096) * args.layers
+    launches_k4096 = sum(cnt for _, n, k, cnt in LLAMA7B_LAYER if k == 4096) * args.layers
+    run_k = make_runner(step_k4096)
+    ev_k_ms, _ = time_region(run_k, args.steps, args.warmup)
+    avg_launch_us = ev_k_ms * 1e3 / (args.steps * launches_k4096)
+    achieved = (bytes_k4096 / launches_k4096) / (avg_launch_us * 1e-6) / 1e9
+    roofline = {
+        "kernel": "gemv_f16_mfma<4,int8,sym,8 waves> (K=4096 shapes: 4096x4096 x4, 11008x4096 x2 per layer)",
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "bytes_per_launch": bytes_k4096 // launches_k4096, "avg_launch_us": round(avg_launch_us, 3),
+    }
+
+    result = {
+        "metric": "w4a16_gemv_hbm_gbps_m1" if M == 1 else f"w4a16_gemv_hbm_gbps_m{M}",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"llama7b_decode_linears_w4a16_sym_g128_m{M}", "layers": args.layers,
+                   "launches_per_step": launches_step, "bytes_per_step": bytes_step,
+                   "hip_graph": not args.no_graph, "event_ms_per_step": round(ev_ms / args.steps, 4),
+                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2)},
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(M)
+    if not args.no_secondary:
+        del layers
+        torch.cuda.empty_cache()
+        result["secondary"] = secondary(L, _lib, torch, dev, args)
+    print(json.dumps(result))
+
+
+def cpu_baseline(M):
+    """The CPU oracle (scalar C: dequantize in fp16 arithmetic, fp32-accumulated matmul) on one
+    decoder layer's seven GEMVs; single thread, like the reference's CPU kernels."""
+    from oracle import ofq_oracle as O
+    rng = np.random.default_rng(0)
+    total_bytes = 0
+    t_total = 0.0
+    for name, n, k, cnt in LLAMA7B_LAYER:
+        w = rng.integers(-128, 128, size=(n, k // 2), dtype=np.int8)
+        scale = rng.uniform(1e-3, 1e-2, size=(n, k // 128)).astype(np.float16)
+        bias = (rng.standard_normal(n) * 0.01).astype(np.float16)
+        x = rng.standard_normal((M, k)).astype(np.float16)
+        t0 = time.perf_counter()
+        for _ in range(cnt):
+            O.fused_linear(x, w, scale, None, bias, 4, True, 1, 128)
+        t_total += time.perf_counter() - t0
+        total_bytes += gemv_bytes(M, n, k) * cnt
+    return {"value": round(total_bytes / t_total / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"one Llama-7B decoder layer (7 GEMVs, {total_bytes} algorithmic bytes, m={M}) "
+                      f"through oracle/ofq_oracle.c in {t_total:.2f} s; host has {os.cpu_count()} cpus"}
+
+
+def secondary(L, _lib, torch, dev, args):
+    """The other BASELINE configurations, each timed over back-to-back launches with events."""
+    out = {}
+    cs = lambda: torch.cuda.current_stream().cuda_stream
+
+    def timeit(fn, iters=20, warmup=3):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / iters  # us
+
+    def chk(st, what):
+        if st != 0:
+            raise RuntimeError(f"{what} status {st}")
+
+    # ---- config 4: prefill W8A16 bf16, asymmetric uint8, g=64, m=2048 -------------------------
+    m, n, k, g = 2048, 11008, 4096, 64
+    x = torch.randn((m, k), device=dev).to(torch.bfloat16)
+    w = torch.randint(0, 256, (n, k), dtype=torch.uint8, device=dev)
+    sc = torch.empty((n, k // g), device=dev).uniform_(1e-3, 1e-2).to(torch.bfloat16)
+    ze = torch.empty((n, k // g), device=dev).uniform_(120, 136).to(torch.bfloat16)
+    o = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    us = timeit(lambda: chk(L.ofq_fused_linear_gq(cs(), x.data_ptr(), w.data_ptr(), sc.data_ptr(),
+                                                  ze.data_ptr(), None, o.data_ptr(), _lib.U8,
+                                                  _lib.BF16, 8, 0, 1, g, m, n, k, None, 0), "prefill"))
+    flops = 2.0 * m * n * k
+    tf = flops / (us * 1e-6) / 1e12
+    out["prefill_w8a16_bf16_m2048"] = {
+        "us": round(us, 2), "tflops": round(tf, 1),
+        "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS["bf16"],
+                     "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS["bf16"], 4)}}
+    del x, w, sc, ze, o
+
+    # ---- config 2: groupwise_dequantize 11008x4096 uint8 asym g=128 -> fp16 ---------------------
+    n, k, g = 11008, 4096, 128
+    reps = 8  # rotate buffers: 8 x 137 MB > caches
+    qs = [torch.randint(0, 256, (n, k), dtype=torch.uint8, device=dev) for _ in range(reps)]
+    sc = torch.empty((n, k // g), device=dev).uniform_(1e-3, 1e-2).to(torch.float16)
+    ze = torch.empty((n, k // g), device=dev).uniform_(100, 156).to(torch.float16)
+    os_ = [torch.empty((n, k), dtype=torch.float16, device=dev) for _ in range(reps)]
+    it = [0]
+
+    def deq():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_groupwise_dequantize(cs(), qs[i].data_ptr(), sc.data_ptr(), ze.data_ptr(),
+                                       os_[i].data_ptr(), _lib.U8, _lib.F16, 8, 0, n * (k // g), g, 1),
+            "dequantize")
+    us = timeit(deq, iters=40)
+    nbytes = n * k + 2 * n * (k // g) * 2 + n * k * 2
+    gb = nbytes / (us * 1e-6) / 1e9
+    out["dequantize_u8_f16_11008x4096"] = {
+        "us": round(us, 2), "gbps": round(gb, 1),
+        "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+    del qs, os_
+
+    # ---- config 5: LayerNorm+observer, quantize to int8, int8 matmul_quant ----------------------
+    m, n, k = 2048, 11008, 4096
+    reps = 8
+    xs = [torch.randn((m, k), device=dev).to(torch.float16) for _ in range(reps)]
+    gamma = (1 + 0.1 * torch.randn(k, device=dev)).to(torch.float16)
+    beta = (0.1 * torch.randn(k, device=dev)).to(torch.float16)
+    ys = [torch.empty((m, k), dtype=torch.float16, device=dev) for _ in range(reps)]
+    a8 = [torch.empty((m, k), dtype=torch.int8, device=dev) for _ in range(reps)]
+    s = torch.empty(1, dtype=torch.float32, device=dev)
+    z = torch.empty(1, dtype=torch.float32, device=dev)
+    ws = torch.empty(m * 4, dtype=torch.uint8, device=dev)
+    it[0] = 0
+
+    def ln():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_fused_layer_norm_min_max_observer(cs(), xs[i].data_ptr(), gamma.data_ptr(),
+                                                    beta.data_ptr(), ys[i].data_ptr(), s.data_ptr(),
+                                                    z.data_ptr(), _lib.F16, m, k, 1e-5, 8,
+                                                    ws.data_ptr(), m * 4), "ln_observer")
+    us = timeit(ln, iters=40)
+    gb = (2 * m * k * 2) / (us * 1e-6) / 1e9
+    out["layer_norm_observer_f16_2048x4096"] = {
+        "us": round(us, 2), "gbps": round(gb, 1),
+        "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+
+    def qz():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_quantization(cs(), ys[i].data_ptr(), s.data_ptr(), z.data_ptr(), a8[i].data_ptr(),
+                               _lib.F16, _lib.I8, m * k, 1, 8, 0, 0, 0), "quantization")
+    us = timeit(qz, iters=40)
+    gb = (m * k * 3) / (us * 1e-6) / 1e9
+    out["quantize_f16_to_i8_2048x4096"] = {
+        "us": round(us, 2), "gbps": round(gb, 1),
+        "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+
+    wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev)
+    wsc = torch.empty(n, device=dev).uniform_(1e-3, 1e-2)
+    o = torch.empty((m, n), dtype=torch.float16, device=dev)
+    us = timeit(lambda: chk(L.ofq_matmul_quant(cs(), a8[0].data_ptr(), wq.data_ptr(), s.data_ptr(),
+                                               wsc.data_ptr(), None, o.data_ptr(), _lib.F16, m, n, k),
+                            "matmul_quant"))
+    tops = 2.0 * m * n * k / (us * 1e-6) / 1e12
+    out["matmul_quant_i8_m2048"] = {
+        "us": round(us, 2), "tops": round(tops, 1),
+        "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": MFMA_PEAK_TFLOPS["i8"],
+                     "unit": "TOP/s", "frac": round(tops / MFMA_PEAK_TFLOPS["i8"], 4)}}
+    del xs, ys, a8, wq, o
+
+    # ---- config 1: observer / quantization / fake_quantization of a 4096x4096 fp32 weight --------
+    reps = 6
+    wsrc = [(torch.randn((4096, 4096), device=dev) * 0.02) for _ in range(reps)]
+    qo = [torch.empty((4096, 4096), device=dev) for _ in range(reps)]
+    sc = torch.empty(4096, device=dev)
+    zp = torch.empty(4096, device=dev)
+    wsb = L.ofq_min_max_observer_workspace_bytes(_lib.F32, 4096 * 4096, 4096)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
+    it[0] = 0
+
+    def obs():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_min_max_observer(cs(), wsrc[i].data_ptr(), sc.data_ptr(), zp.data_ptr(), _lib.F32,
+                                   4096 * 4096, 4096, 8, 0, 0, ws.data_ptr(), wsb), "observer")
+
+    def qf32():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_quantization(cs(), wsrc[i].data_ptr(), sc.data_ptr(), zp.data_ptr(),
+                               qo[i].data_ptr(), _lib.F32, _lib.F32, 4096 * 4096, 4096, 8, 0, 0, 0),
+            "quantization f32")
+
+    def fq32():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_fake_quantization(cs(), wsrc[i].data_ptr(), sc.data_ptr(), zp.data_ptr(),
+                                    qo[i].data_ptr(), _lib.F32, 4096 * 4096, 4096, 8, 0, 0, 0),
+            "fake_quantization f32")
+    for name, fn, nbytes in (("min_max_observer_f32_4096x4096", obs, 4096 * 4096 * 4),
+                             ("quantization_f32_4096x4096", qf32, 4096 * 4096 * 8),
+                             ("fake_quantization_f32_4096x4096", fq32, 4096 * 4096 * 8)):
+        us = timeit(fn, iters=30)
+        gb = nbytes / (us * 1e-6) / 1e9
+        out[name] = {"us": round(us, 2), "gbps": round(gb, 1),
+                     "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS,
+                                  "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+    return out
+
+
+if __name__ == "__main__":
+    main()
