@@ -1,0 +1,450 @@
+// Device code of the skinny-M (decode) kernels of fused_linear_with_groupwise_quantized_weight.
+// Kept in a header so that experiments can instantiate the kernels directly.
+#pragma once
+
+#include "ofq_device.h"
+
+namespace ofq {
+namespace {
+
+enum { kZeroNone = 0, kZeroSymU = 1, kZeroAsym = 2 };
+
+__device__ __forceinline__ f16x2 as_h2(uint32_t u) { return __builtin_bit_cast(f16x2, u); }
+__device__ __forceinline__ uint32_t as_u32(f16x2 h) { return __builtin_bit_cast(uint32_t, h); }
+
+// eight 4-bit codes of `word` as exact fp16 values, in the pair order
+// (e1,e5) (e0,e4) (e3,e7) (e2,e6) where e_i is element i of the word (element 0 = high nibble
+// of byte 0).
+template<bool SIGNED>
+__device__ __forceinline__ void unpack4_pairs(uint32_t word, f16x2 (&o)[4]) {
+  if (SIGNED) word ^= 0x88888888u;
+  const uint32_t w8 = word >> 8;
+  const f16 off_lo = SIGNED ? (f16)(-1032.0f) : (f16)(-1024.0f);
+  const f16 off_hi = SIGNED ? (f16)(-72.0f) : (f16)(-64.0f);
+  const f16x2 ol = {off_lo, off_lo};
+  const f16x2 oh = {off_hi, off_hi};
+  const f16x2 sixteenth = {(f16)0.0625f, (f16)0.0625f};
+  o[0] = as_h2((word & 0x000F000Fu) | 0x64006400u) + ol;
+  o[1] = __builtin_elementwise_fma(as_h2((word & 0x00F000F0u) | 0x64006400u), sixteenth, oh);
+  o[2] = as_h2((w8 & 0x000F000Fu) | 0x64006400u) + ol;
+  o[3] = __builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x64006400u), sixteenth, oh);
+}
+
+// four 8-bit codes of `word` as exact fp16 values in natural order (b0,b1) (b2,b3)
+template<bool SIGNED>
+__device__ __forceinline__ void unpack8_pairs(uint32_t word, f16x2 (&o)[2]) {
+  if (SIGNED) word ^= 0x80808080u;
+  const f16 off = SIGNED ? (f16)(-1152.0f) : (f16)(-1024.0f);
+  const f16x2 o2 = {off, off};
+  o[0] = as_h2(__builtin_amdgcn_perm(word, 0x64646464u, 0x00050004u)) + o2;
+  o[1] = as_h2(__builtin_amdgcn_perm(word, 0x64646464u, 0x00070006u)) + o2;
+}
+
+// x permuted to the pair order of unpack4_pairs: [x1,x5,x0,x4,x3,x7,x2,x6]
+__device__ __forceinline__ u32x4 permute_x4(u32x4 v) {
+  u32x4 r;
+  r[0] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // (x1, x5)
+  r[1] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // (x0, x4)
+  r[2] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // (x3, x7)
+  r[3] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // (x2, x6)
+  return r;
+}
+
+template<int BITS, bool SIGNED, int ZMODE, int NWAVES, int UNROLL>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_f16_mfma(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+              const f16* __restrict__ scale, const f16* __restrict__ zero,
+              const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
+              int group_size, int gs_shift) {
+  constexpr int CH = BITS == 4 ? 128 : 64;  // k elements per chunk (64 bytes of codes per row)
+  constexpr int LK = CH / 4;                // k elements per lane per chunk
+  constexpr int NJ = LK / 8;                // MFMAs per chunk
+  __shared__ float red[NWAVES][64][4];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15;
+  const int kb = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int n_ld = (n0 + r < N) ? n0 + r : N - 1;  // clamp loads of a partial last tile
+  const int nchunks = K / CH;
+  const int G = K / group_size;
+  const uint8_t* wrow = w + (int64_t)n_ld * ((int64_t)K * BITS / 8);
+  const f16* srow = scale + (int64_t)n_ld * G;
+  const f16* zrow = ZMODE == kZeroAsym ? zero + (int64_t)n_ld * G : nullptr;
+  const bool has_x = r < M;
+  const f16* xrow = x + (int64_t)(has_x ? r : 0) * K;
+
+  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc1 = {0.f, 0.f, 0.f, 0.f};
+
+  for (int c0 = wave; c0 < nchunks; c0 += NWAVES * UNROLL) {
+    u32x4 wq[UNROLL];
+    u32x4 xv[UNROLL][NJ];
+    f16 sv[UNROLL], zv[UNROLL];
+    // issue every load of the UNROLL chunks before touching any of them
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * NWAVES;
+      const bool valid = c < nchunks;
+      const int k0 = (valid ? c : 0) * CH + kb * LK;
+      wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (int64_t)k0 * BITS / 8));
+      const int g = gs_shift >= 0 ? (k0 >> gs_shift) : (k0 / group_size);
+      sv[u] = srow[g];
+      zv[u] = ZMODE == kZeroAsym ? zrow[g] : (f16)0.0f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const u32x4 t = *reinterpret_cast<const u32x4*>(xrow + k0 + j * 8);
+        const u32x4 zero4 = {0u, 0u, 0u, 0u};
+        xv[u][j] = (has_x && valid) ? t : zero4;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const f16 s = sv[u];
+      f16 z = zv[u];
+      if (ZMODE == kZeroSymU) z = (f16)(-(float)((1 << (BITS - 1)) - 1)) * s;
+      const f16x2 s2 = {s, s};
+      const f16x2 z2 = {z, z};
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        u32x4 bop;
+        u32x4 aop;
+        if (BITS == 4) {
+          f16x2 p[4];
+          unpack4_pairs<SIGNED>(wq[u][j], p);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            f16x2 v = p[e] * s2;
+            if (ZMODE != kZeroNone) v = v + z2;
+            bop[e] = as_u32(v);
+          }
+          aop = permute_x4(xv[u][j]);
+        } else {
+          f16x2 p0[2], p1[2];
+          unpack8_pairs<SIGNED>(wq[u][2 * j], p0);
+          unpack8_pairs<SIGNED>(wq[u][2 * j + 1], p1);
+          f16x2 v[4] = {p0[0] * s2, p0[1] * s2, p1[0] * s2, p1[1] * s2};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (ZMODE != kZeroNone) v[e] = v[e] + z2;
+            bop[e] = as_u32(v[e]);
+          }
+          aop = xv[u][j];
+        }
+        const f16x8 a8 = __builtin_bit_cast(f16x8, aop);
+        const f16x8 b8 = __builtin_bit_cast(f16x8, bop);
+        if ((j & 1) == 0) {
+          acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a8, b8, acc0, 0, 0, 0);
+        } else {
+          acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a8, b8, acc1, 0, 0, 0);
+        }
+      }
+    }
+  }
+  // lane holds D[m = 4*kb + v][n = n0 + r]
+#pragma unroll
+  for (int v = 0; v < 4; ++v) red[wave][lane][v] = acc0[v] + acc1[v];
+  __syncthreads();
+  for (int t = threadIdx.x; t < 256; t += NWAVES * 64) {
+    const int l = t >> 2;
+    const int v = t & 3;
+    float sum = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < NWAVES; ++wv) sum += red[wv][l][v];
+    const int m = 4 * (l >> 4) + v;
+    const int n = n0 + (l & 15);
+    if (m < M && n < N) {
+      if (bias != nullptr) sum += (float)bias[n];
+      out[(int64_t)m * N + n] = (f16)sum;
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Fast path: 4-bit symmetric codes in an int8 container (zero term 0), fp16, groups along K with
+// 128 | group_size.  A one-shot kernel cannot overlap its arithmetic with the HBM latency it has
+// just waited for, and at 8 TB/s the whole chip has only ~20 vector instructions per 32-bit word
+// of codes, so the instruction count per word is what this kernel is built around (5, against
+// ~17 for gemv_f16_mfma):
+//
+//  (1) x is permuted into MFMA operand order ONCE per block while the weight loads are in
+//      flight, and kept in LDS; the waves then fetch ready-made operands with ds_read_b128
+//      (only the lanes of rows m < M read at all).  When M*K is too large for LDS (STAGED =
+//      false) each lane loads and permutes the x of its own k-slot instead.
+//  (2) The codes are never converted to their integer value.  The halves 0x6400|nibble are
+//      1024+u (low nibbles) and 1024+16u (high nibbles), u = q+8 after the xor that turns two's
+//      complement into offset binary (the xor is folded into the mask-and-merge, one v_bitop3).
+//      The x that meets high nibbles is pre-divided by 16 (exact in fp16 unless subnormal), so
+//      one MFMA accumulator collects
+//        acc = sum_k x q + 1032 * sum_lo x + 72 * sum_hi x
+//      and the constant part `corr` depends on (m, chunk) only: it is computed once per block
+//      when x is staged (or with two MFMAs against constant operands when x is not staged).
+//      All products are exact in fp32; the cancellation is done per chunk of 128 k, where the
+//      partial sums are ~1e4 and fp32 resolves 1e-3 of a code unit.  The group scale multiplies
+//      the chunk result once (fp32), i.e. w~ = q*s is not rounded to fp16 first: the result is
+//      closer to exact arithmetic than the reference kernel's and differs from the
+//      dequantize->matmul composition by the rounding of w~ (~3e-4 relative).
+//  (3) The 16 x G scales of the block's rows are one contiguous piece of memory: they are
+//      fetched with a single coalesced load per block into LDS instead of one 2-byte gather per
+//      lane and chunk (which costs as many memory requests as the weights themselves).
+//  (4) A wave takes chunks in adjacent pairs, so that both halves of every 128-byte line are
+//      requested by the same wave back to back.
+//
+// LDS layout of x: record (m, chunk) = 256 bytes = [kb 0..3][t 0..3][8 halves], where for the
+// 32 k-values of lane-slot kb, t=0/1 hold the k of the low/high nibbles of code words 0,1 and
+// t=2/3 those of words 2,3, in the order the nibble masks deliver them: {1,5,3,7,9,13,11,15} and
+// {0,4,2,6,8,12,10,14} (+16 for t=2,3).
+// ---------------------------------------------------------------------------------------------
+constexpr int kGemvMaxUnits = 4;  // 32-byte x units a thread may stage
+
+// x of one 16-k unit (two 128-bit words, natural order) -> low-nibble operand and high-nibble
+// operand, the latter divided by 16
+__device__ __forceinline__ void permute_unit(const u32x4 a, const u32x4 b, u32x4& lo, u32x4& hi) {
+  lo[0] = __builtin_amdgcn_perm(a[2], a[0], 0x07060302u);  // (x1, x5)
+  lo[1] = __builtin_amdgcn_perm(a[3], a[1], 0x07060302u);  // (x3, x7)
+  lo[2] = __builtin_amdgcn_perm(b[2], b[0], 0x07060302u);  // (x9, x13)
+  lo[3] = __builtin_amdgcn_perm(b[3], b[1], 0x07060302u);  // (x11, x15)
+  hi[0] = __builtin_amdgcn_perm(a[2], a[0], 0x05040100u);  // (x0, x4)
+  hi[1] = __builtin_amdgcn_perm(a[3], a[1], 0x05040100u);  // (x2, x6)
+  hi[2] = __builtin_amdgcn_perm(b[2], b[0], 0x05040100u);  // (x8, x12)
+  hi[3] = __builtin_amdgcn_perm(b[3], b[1], 0x05040100u);  // (x10, x14)
+  const f16x2 sixteenth = {(f16)0.0625f, (f16)0.0625f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) hi[i] = as_u32(as_h2(hi[i]) * sixteenth);
+}
+
+// 1032 * (sum of the low-nibble x) + 72 * (sum of the high-nibble x) of one permuted unit
+__device__ __forceinline__ float unit_corr(const u32x4 lo, const u32x4 hi) {
+  float sl = 0.f, sh = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f16x2 l = as_h2(lo[i]), h = as_h2(hi[i]);
+    sl += (float)l[0] + (float)l[1];
+    sh += (float)h[0] + (float)h[1];
+  }
+  return 1032.0f * sl + 1152.0f * sh;  // hi carries x/16: 72 * 16 = 1152
+}
+
+__device__ __forceinline__ float unit_corr_of(const u32x4 a, const u32x4 b) {
+  u32x4 lo, hi;
+  permute_unit(a, b, lo, hi);
+  return unit_corr(lo, hi);
+}
+
+template<int NWAVES, int UNROLL, bool STAGED>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+             const f16* __restrict__ scale, const f16* __restrict__ bias,
+             f16* __restrict__ out, int M, int N, int K, int group_size, int cpg_shift) {
+  // cpg_shift: log2(group_size / 128) when that is a power of two, else -1 (division per chunk)
+  static_assert(UNROLL % 2 == 0, "chunks are taken in pairs");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NT = NWAVES * 64;
+  const int nchunks = K >> 7;
+  const int npairs = (nchunks + 1) >> 1;
+  const int G = K / group_size;
+  // LDS: [reduction NWAVES*64*4 f32][scale tile 16*G halves, padded to 16 B]
+  //      [corr: nchunks x 16 f32][x records]
+  float* red = reinterpret_cast<float*>(smem);
+  f16* sl = reinterpret_cast<f16*>(smem + NWAVES * 64 * 16);
+  float* corr_l = reinterpret_cast<float*>(smem + NWAVES * 64 * 16 + ((16 * G * 2 + 15) & ~15));
+  uint8_t* zrec = reinterpret_cast<uint8_t*>(corr_l) + (STAGED ? nchunks * 64 : 0);  // 64 zero bytes
+  uint8_t* xs = zrec + 64;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
+  const int r = lane & 15;
+  const int kb = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int n_ld = (n0 + r < N) ? n0 + r : N - 1;
+  const uint8_t* wrow = w + (int64_t)n_ld * (K >> 1) + kb * 16;
+  const bool has_x = r < M;
+
+  // ---- loads that feed LDS are issued first so that they return before the weights ---------
+  const int nunits = STAGED ? (M * K) >> 4 : 0;
+  u32x4 xu[kGemvMaxUnits][2];
+  if (STAGED) {
+#pragma unroll
+    for (int i = 0; i < kGemvMaxUnits; ++i) {
+      const int u = tid + i * NT;
+      if (u < nunits) {
+        const u32x4* src = reinterpret_cast<const u32x4*>(x + (int64_t)u * 16);
+        xu[i][0] = src[0];
+        xu[i][1] = src[1];
+      }
+    }
+  }
+  // scale tile: rows n0 .. n0+15 are contiguous; a partial last tile is read element-wise
+  const int rows_valid = (N - n0) < 16 ? (N - n0) : 16;
+  const int tile_halves = rows_valid * G;
+  const f16* stile = scale + (int64_t)n0 * G;
+  u32x4 sreg[2];
+  bool s_vec[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int e = (tid + i * NT) * 8;  // first half-element of this 16-byte piece
+    s_vec[i] = e + 8 <= tile_halves;
+    if (s_vec[i]) sreg[i] = *reinterpret_cast<const u32x4*>(stile + e);
+  }
+
+  auto chunk_of = [&](int p0, int u) { return 2 * (p0 + (u >> 1) * NWAVES) + (u & 1); };
+  u32x4 wq[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int c = chunk_of(wave, u);
+    wq[u] = __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4*>(wrow + (c < nchunks ? c : 0) * 64));
+  }
+
+  // ---- fill LDS -------------------------------------------------------------------------------
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int e = (tid + i * NT) * 8;
+    if (s_vec[i]) {
+      *reinterpret_cast<u32x4*>(sl + e) = sreg[i];
+    } else if (e < tile_halves) {
+      for (int j = e; j < tile_halves && j < e + 8; ++j) sl[j] = stile[j];
+    }
+  }
+  // pieces beyond 2*NT*8 halves (G > NT) are rare; copy them plainly
+  for (int e = 2 * NT * 8 + tid; e < tile_halves; e += NT) sl[e] = stile[e];
+  if (tid < 16) reinterpret_cast<uint32_t*>(zrec)[tid] = 0u;
+  if (STAGED) {
+#pragma unroll
+    for (int i = 0; i < kGemvMaxUnits; ++i) {
+      const int u = tid + i * NT;
+      if (u < nunits) {
+        u32x4 lo, hi;
+        permute_unit(xu[i][0], xu[i][1], lo, hi);
+        // unit u = (m, chunk, j): j -> kb = j/2, t = 2*(j%2) + {0: lo, 1: hi}; 32 bytes per unit
+        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32);
+        dst[0] = lo;
+        dst[1] = hi;
+      }
+      // the 8 units of a chunk sit in 8 consecutive lanes (K/16 is a multiple of 8): fold
+      float cpart = u < nunits ? unit_corr_of(xu[i][0], xu[i][1]) : 0.f;
+      cpart += __shfl_xor(cpart, 1, 64);
+      cpart += __shfl_xor(cpart, 2, 64);
+      cpart += __shfl_xor(cpart, 4, 64);
+      if (u < nunits && (u & 7) == 0) {
+        const int m = (u >> 3) / nchunks;
+        const int c = (u >> 3) - m * nchunks;
+        corr_l[c * 16 + m] = -cpart;  // negated: it seeds the MFMA accumulator
+      }
+    }
+  }
+  __syncthreads();
+
+  const uint8_t* xrec = has_x ? xs + ((size_t)r * nchunks) * 256 + kb * 64 : zrec;
+  const int xrec_stride = has_x ? 256 : 0;
+  const f16* xrow = x + (int64_t)(has_x ? r : 0) * K + kb * 32;
+  const f16* slr = sl + r * G;
+  const f16 c_lo = (f16)1032.0f, c_hi = (f16)1152.0f;
+  const f16x8 k1032 = {c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo};
+  const f16x8 k1152 = {c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi};
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  f32x4 total = {0.f, 0.f, 0.f, 0.f};
+
+  for (int p0 = wave; p0 < npairs; p0 += NWAVES * (UNROLL / 2)) {
+    // prefetch the next group while this one is consumed
+    u32x4 wq_next[UNROLL];
+    const int pn = p0 + NWAVES * (UNROLL / 2);
+    if (pn < npairs) {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int c = chunk_of(pn, u);
+        wq_next[u] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4*>(wrow + (c < nchunks ? c : 0) * 64));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = chunk_of(p0, u);
+      if (c < nchunks) {
+        u32x4 xa[4];
+        if (STAGED) {
+          const u32x4* xp = reinterpret_cast<const u32x4*>(xrec + c * xrec_stride);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) xa[t] = xp[t];
+        } else {
+          const u32x4* xp = reinterpret_cast<const u32x4*>(xrow + c * 128);
+          u32x4 raw[4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) raw[t] = has_x ? xp[t] : zero4;
+          permute_unit(raw[0], raw[1], xa[0], xa[1]);
+          permute_unit(raw[2], raw[3], xa[2], xa[3]);
+        }
+        const float s = (float)slr[cpg_shift >= 0 ? (c >> cpg_shift) : (c * 128 / group_size)];
+        // the accumulator starts at -corr (staged), or corr is built alongside (not staged)
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        f32x4 corr = {0.f, 0.f, 0.f, 0.f};
+        if (STAGED) acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const uint32_t w0 = wq[u][2 * h];
+          const uint32_t w1 = wq[u][2 * h + 1];
+          const uint32_t w0s = w0 >> 8, w1s = w1 >> 8;
+          // (w & mask) ^ (magic | sign bit of the nibble): xor 8 and merge 0x6400 in one op
+          u32x4 blo, bhi;
+          blo[0] = (w0 & 0x000F000Fu) ^ 0x64086408u;
+          blo[1] = (w0s & 0x000F000Fu) ^ 0x64086408u;
+          blo[2] = (w1 & 0x000F000Fu) ^ 0x64086408u;
+          blo[3] = (w1s & 0x000F000Fu) ^ 0x64086408u;
+          bhi[0] = (w0 & 0x00F000F0u) ^ 0x64806480u;
+          bhi[1] = (w0s & 0x00F000F0u) ^ 0x64806480u;
+          bhi[2] = (w1 & 0x00F000F0u) ^ 0x64806480u;
+          bhi[3] = (w1s & 0x00F000F0u) ^ 0x64806480u;
+          const f16x8 a_lo = __builtin_bit_cast(f16x8, xa[2 * h]);
+          const f16x8 a_hi = __builtin_bit_cast(f16x8, xa[2 * h + 1]);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, __builtin_bit_cast(f16x8, blo), acc,
+                                                       0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, __builtin_bit_cast(f16x8, bhi), acc,
+                                                       0, 0, 0);
+          if (!STAGED) {
+            corr = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, k1032, corr, 0, 0, 0);
+            corr = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, k1152, corr, 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float q = STAGED ? acc[v] : acc[v] - corr[v];
+          total[v] = __builtin_fmaf(q, s, total[v]);
+        }
+      }
+    }
+    if (pn < npairs) {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) wq[u] = wq_next[u];
+    }
+  }
+  // lane holds D[m = 4*kb + v][n = n0 + r]
+#pragma unroll
+  for (int v = 0; v < 4; ++v) red[(wave * 64 + lane) * 4 + v] = total[v];
+  __syncthreads();
+  for (int t = tid; t < 256; t += NT) {
+    const int l = t >> 2;
+    const int v = t & 3;
+    float sum = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < NWAVES; ++wv) sum += red[(wv * 64 + l) * 4 + v];
+    const int m = 4 * (l >> 4) + v;
+    const int n = n0 + (l & 15);
+    if (m < M && n < N) {
+      if (bias != nullptr) sum += (float)bias[n];
+      out[(int64_t)m * N + n] = (f16)sum;
+    }
+  }
+}
+
+// dynamic LDS bytes of gemv_w4s_f16
+inline size_t gemv_w4s_lds_bytes(int nwaves, bool staged, int M, int K, int group_size) {
+  const int G = K / group_size;
+  return (size_t)nwaves * 64 * 16 + ((16 * G * 2 + 15) & ~15) + 64
+         + (staged ? (size_t)(K >> 7) * 64 + (size_t)M * K * 2 : 0);
+}
+
+}  // namespace
+}  // namespace ofq

@@ -26,165 +26,12 @@
 //     groupwise_dequantize;
 //   - partial sums of the waves are combined through LDS, bias is added in fp32, one rounding
 //     to T.
+#include "gemv_kernels.h"
 #include "ofq_device.h"
 #include "ofq_internal.h"
 
 namespace ofq {
 namespace {
-
-enum { kZeroNone = 0, kZeroSymU = 1, kZeroAsym = 2 };
-
-__device__ __forceinline__ f16x2 as_h2(uint32_t u) { return __builtin_bit_cast(f16x2, u); }
-__device__ __forceinline__ uint32_t as_u32(f16x2 h) { return __builtin_bit_cast(uint32_t, h); }
-
-// eight 4-bit codes of `word` as exact fp16 values, in the pair order
-// (e1,e5) (e0,e4) (e3,e7) (e2,e6) where e_i is element i of the word (element 0 = high nibble
-// of byte 0).
-template<bool SIGNED>
-__device__ __forceinline__ void unpack4_pairs(uint32_t word, f16x2 (&o)[4]) {
-  if (SIGNED) word ^= 0x88888888u;
-  const uint32_t w8 = word >> 8;
-  const f16 off_lo = SIGNED ? (f16)(-1032.0f) : (f16)(-1024.0f);
-  const f16 off_hi = SIGNED ? (f16)(-72.0f) : (f16)(-64.0f);
-  const f16x2 ol = {off_lo, off_lo};
-  const f16x2 oh = {off_hi, off_hi};
-  const f16x2 sixteenth = {(f16)0.0625f, (f16)0.0625f};
-  o[0] = as_h2((word & 0x000F000Fu) | 0x64006400u) + ol;
-  o[1] = __builtin_elementwise_fma(as_h2((word & 0x00F000F0u) | 0x64006400u), sixteenth, oh);
-  o[2] = as_h2((w8 & 0x000F000Fu) | 0x64006400u) + ol;
-  o[3] = __builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x64006400u), sixteenth, oh);
-}
-
-// four 8-bit codes of `word` as exact fp16 values in natural order (b0,b1) (b2,b3)
-template<bool SIGNED>
-__device__ __forceinline__ void unpack8_pairs(uint32_t word, f16x2 (&o)[2]) {
-  if (SIGNED) word ^= 0x80808080u;
-  const f16 off = SIGNED ? (f16)(-1152.0f) : (f16)(-1024.0f);
-  const f16x2 o2 = {off, off};
-  o[0] = as_h2(__builtin_amdgcn_perm(word, 0x64646464u, 0x00050004u)) + o2;
-  o[1] = as_h2(__builtin_amdgcn_perm(word, 0x64646464u, 0x00070006u)) + o2;
-}
-
-// x permuted to the pair order of unpack4_pairs: [x1,x5,x0,x4,x3,x7,x2,x6]
-__device__ __forceinline__ u32x4 permute_x4(u32x4 v) {
-  u32x4 r;
-  r[0] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // (x1, x5)
-  r[1] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // (x0, x4)
-  r[2] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // (x3, x7)
-  r[3] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // (x2, x6)
-  return r;
-}
-
-template<int BITS, bool SIGNED, int ZMODE, int NWAVES, int UNROLL>
-__global__ void __launch_bounds__(NWAVES * 64)
-gemv_f16_mfma(const f16* __restrict__ x, const uint8_t* __restrict__ w,
-              const f16* __restrict__ scale, const f16* __restrict__ zero,
-              const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
-              int group_size, int gs_shift) {
-  constexpr int CH = BITS == 4 ? 128 : 64;  // k elements per chunk (64 bytes of codes per row)
-  constexpr int LK = CH / 4;                // k elements per lane per chunk
-  constexpr int NJ = LK / 8;                // MFMAs per chunk
-  __shared__ float red[NWAVES][64][4];
-
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int r = lane & 15;
-  const int kb = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int n_ld = (n0 + r < N) ? n0 + r : N - 1;  // clamp loads of a partial last tile
-  const int nchunks = K / CH;
-  const int G = K / group_size;
-  const uint8_t* wrow = w + (int64_t)n_ld * ((int64_t)K * BITS / 8);
-  const f16* srow = scale + (int64_t)n_ld * G;
-  const f16* zrow = ZMODE == kZeroAsym ? zero + (int64_t)n_ld * G : nullptr;
-  const bool has_x = r < M;
-  const f16* xrow = x + (int64_t)(has_x ? r : 0) * K;
-
-  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f};
-  f32x4 acc1 = {0.f, 0.f, 0.f, 0.f};
-
-  for (int c0 = wave; c0 < nchunks; c0 += NWAVES * UNROLL) {
-    u32x4 wq[UNROLL];
-    u32x4 xv[UNROLL][NJ];
-    f16 sv[UNROLL], zv[UNROLL];
-    // issue every load of the UNROLL chunks before touching any of them
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * NWAVES;
-      const bool valid = c < nchunks;
-      const int k0 = (valid ? c : 0) * CH + kb * LK;
-      wq[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + (int64_t)k0 * BITS / 8));
-      const int g = gs_shift >= 0 ? (k0 >> gs_shift) : (k0 / group_size);
-      sv[u] = srow[g];
-      zv[u] = ZMODE == kZeroAsym ? zrow[g] : (f16)0.0f;
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const u32x4 t = *reinterpret_cast<const u32x4*>(xrow + k0 + j * 8);
-        const u32x4 zero4 = {0u, 0u, 0u, 0u};
-        xv[u][j] = (has_x && valid) ? t : zero4;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const f16 s = sv[u];
-      f16 z = zv[u];
-      if (ZMODE == kZeroSymU) z = (f16)(-(float)((1 << (BITS - 1)) - 1)) * s;
-      const f16x2 s2 = {s, s};
-      const f16x2 z2 = {z, z};
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        u32x4 bop;
-        u32x4 aop;
-        if (BITS == 4) {
-          f16x2 p[4];
-          unpack4_pairs<SIGNED>(wq[u][j], p);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            f16x2 v = p[e] * s2;
-            if (ZMODE != kZeroNone) v = v + z2;
-            bop[e] = as_u32(v);
-          }
-          aop = permute_x4(xv[u][j]);
-        } else {
-          f16x2 p0[2], p1[2];
-          unpack8_pairs<SIGNED>(wq[u][2 * j], p0);
-          unpack8_pairs<SIGNED>(wq[u][2 * j + 1], p1);
-          f16x2 v[4] = {p0[0] * s2, p0[1] * s2, p1[0] * s2, p1[1] * s2};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (ZMODE != kZeroNone) v[e] = v[e] + z2;
-            bop[e] = as_u32(v[e]);
-          }
-          aop = xv[u][j];
-        }
-        const f16x8 a8 = __builtin_bit_cast(f16x8, aop);
-        const f16x8 b8 = __builtin_bit_cast(f16x8, bop);
-        if ((j & 1) == 0) {
-          acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a8, b8, acc0, 0, 0, 0);
-        } else {
-          acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a8, b8, acc1, 0, 0, 0);
-        }
-      }
-    }
-  }
-  // lane holds D[m = 4*kb + v][n = n0 + r]
-#pragma unroll
-  for (int v = 0; v < 4; ++v) red[wave][lane][v] = acc0[v] + acc1[v];
-  __syncthreads();
-  for (int t = threadIdx.x; t < 256; t += NWAVES * 64) {
-    const int l = t >> 2;
-    const int v = t & 3;
-    float sum = 0.f;
-#pragma unroll
-    for (int wv = 0; wv < NWAVES; ++wv) sum += red[wv][l][v];
-    const int m = 4 * (l >> 4) + v;
-    const int n = n0 + (l & 15);
-    if (m < M && n < N) {
-      if (bias != nullptr) sum += (float)bias[n];
-      out[(int64_t)m * N + n] = (f16)sum;
-    }
-  }
-}
 
 // ---- any shape, any grouping: one wave per output element --------------------------------
 template<typename T, int BITS, bool SIGNED>
@@ -248,6 +95,50 @@ inline int ilog2_exact(int64_t v) {
   return s;
 }
 
+// ---- fast path launcher (gemv_w4s_f16) ------------------------------------------------------
+template<int NW, bool STAGED>
+int launch_w4s_inst(hipStream_t st, const LinearArgs& a, size_t lds, int cpg_shift) {
+  auto kern = gemv_w4s_f16<NW, 2, STAGED>;
+  if (lds > 64 * 1024) return OFQ_ERR_UNSUPPORTED;
+  const int grid = (int)((a.n + 15) / 16);
+  kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
+                                  static_cast<const f16*>(a.scale),
+                                  static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
+                                  (int)a.m, (int)a.n, (int)a.k, (int)a.group_size, cpg_shift);
+  return ofq_check_launch();
+}
+
+bool w4s_supported(const LinearArgs& a) {
+  return a.t_dtype == OFQ_F16 && a.bits == 4 && a.w_signed && a.symmetric && a.group_dim == 1
+         && a.m >= 1 && a.m <= 16 && a.k % 128 == 0 && a.group_size % 128 == 0
+         && a.k <= (1 << 20) && a.n <= 0x7FFFFFFF - 16;
+}
+
+int launch_w4s(hipStream_t st, const LinearArgs& a) {
+  const int64_t tiles = (a.n + 15) / 16;
+  const int npairs = (int)((a.k / 128 + 1) / 2);
+  // waves per block: as many as still let every block be resident at once (<= 24 waves per CU on
+  // 256 CUs), so the kernel runs as a single round of blocks; never more than there are pairs
+  int nw = 16;
+  while (nw > 2 && (tiles * nw > 6144 || nw > npairs)) nw >>= 1;
+  const int nt = nw * 64;
+  const int64_t nunits = a.m * a.k / 16;
+  bool staged = nunits <= (int64_t)kGemvMaxUnits * nt;
+  size_t lds = gemv_w4s_lds_bytes(nw, staged, (int)a.m, (int)a.k, (int)a.group_size);
+  if (staged && lds > 48 * 1024) {
+    staged = false;
+    lds = gemv_w4s_lds_bytes(nw, false, (int)a.m, (int)a.k, (int)a.group_size);
+  }
+  const int cpg_shift = ilog2_exact(a.group_size / 128);
+#define OFQ_W4S(NWV)                                                                   \
+  if (nw == NWV)                                                                       \
+    return staged ? launch_w4s_inst<NWV, true>(st, a, lds, cpg_shift)                  \
+                  : launch_w4s_inst<NWV, false>(st, a, lds, cpg_shift);
+  OFQ_W4S(16) OFQ_W4S(8) OFQ_W4S(4) OFQ_W4S(2)
+#undef OFQ_W4S
+  return OFQ_ERR_UNSUPPORTED;
+}
+
 template<int BITS, bool SIGNED, int ZMODE>
 int launch_gemv_variant(hipStream_t st, const LinearArgs& a) {
   constexpr int CH = BITS == 4 ? 128 : 64;
@@ -286,6 +177,10 @@ bool gemv_wq_supported(const LinearArgs& a) {
 }
 
 int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
+  if (w4s_supported(a)) {
+    const int rc = launch_w4s(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
 #define OFQ_V(B, SG, ZM) \
   if (a.bits == B && a.w_signed == SG && zmode == ZM) return launch_gemv_variant<B, SG, ZM>(st, a);
