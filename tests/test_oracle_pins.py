@@ -1,0 +1,327 @@
+"""Pins of the CPU oracle (oracle/ofq_oracle.c) against evidence that does not come from the
+oracle itself: the known-answer table of the reference's CPU kernels, IEEE conversions of numpy /
+torch, exact rational or integer arithmetic, closed forms and invariants.  CPU only."""
+import json
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+import helpers as H
+from oracle import ofq_oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_cpu_known_answers.json")
+
+
+def _f32_from_hex(h):
+    return np.float32(float.fromhex(h))
+
+
+def _bits32(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def _codes(strs):
+    return np.array([-0.0 if s == "-0" else float(s) for s in strs], dtype=np.float32)
+
+
+# ------------------------------------------------------------------------------------------------
+# observer / quantization / fake quantization: the reference CPU kernels' own outputs
+# ------------------------------------------------------------------------------------------------
+def test_known_answers_of_reference_cpu_kernels():
+    g = json.load(open(GOLDEN))
+    x = np.array(g["input"], dtype=np.float32)
+    for row in g["rows"]:
+        s, z = O.min_max_observer(x, g["formula"], row["bits"], row["scheme"], row["per_layer"])
+        exp_s = np.array([_f32_from_hex(h) for h in row["scale"]], dtype=np.float32)
+        assert np.array_equal(_bits32(s), _bits32(exp_s)), row
+        assert np.array_equal(z, np.array(row["zero_point"], dtype=np.float32)), row
+        q = O.quantization(x, s, z, g["formula"], row["bits"], row["scheme"], zp_mode="cpu")
+        # bit comparison: the sign of zero is part of the reference's output
+        assert np.array_equal(_bits32(q.ravel()), _bits32(_codes(row["codes"]))), row
+    s, z = O.min_max_observer(x, "google", 8, "symmetric", False)
+    f = O.fake_quantization(x, s, z, "google", 8, "symmetric")
+    exp = np.array([_f32_from_hex(h) for h in g["fake_quantization_symmetric_8bit_per_channel"]],
+                   dtype=np.float32)
+    assert np.array_equal(_bits32(f.ravel()), _bits32(exp))
+    rhe = g["round_half_even"]
+    q = O.quantization(np.array(rhe["input"], np.float32), np.array(rhe["scale"], np.float32),
+                       np.zeros(1, np.float32))
+    assert np.array_equal(_bits32(q), _bits32(_codes(rhe["codes"])))
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("per_layer", [True, False])
+def test_symmetric_quantization_invariants(bits, per_layer):
+    """What the mathematics fixes without restating the kernel: codes are integers in
+    [-2^(b-1), 2^(b-1)-1], each is a nearest integer of x/s, the (channel) absmax maps to
+    +-(2^(b-1)-1), and the scale is the correctly rounded quotient absmax / (2^(b-1)-1)."""
+    rng = np.random.default_rng(bits * 10 + per_layer)
+    x = (rng.standard_normal((9, 40, 20)) * 0.3).astype(np.float32)
+    s, z = O.min_max_observer(x, "google", bits, "symmetric", per_layer)
+    qmax = 2 ** (bits - 1) - 1
+    absmax = np.abs(x).max() if per_layer else np.abs(x).reshape(9, -1).max(axis=1)
+    # correctly rounded quotient: compare with exact rational division rounded to fp32
+    exact = [Fraction(float(a)) / qmax for a in np.atleast_1d(absmax)]
+    assert np.array_equal(s, np.array([np.float32(float(e)) for e in exact], np.float32))
+    assert np.all(z == 0)
+    q = O.quantization(x, s, z, "google", bits, "symmetric")
+    assert np.array_equal(q, np.rint(q)) and q.min() >= -qmax - 1 and q.max() <= qmax
+    sb = s.reshape((-1,) + (1,) * (x.ndim - 1)).astype(np.float64)
+    assert np.abs(x.astype(np.float64) / sb - q).max() <= 0.5 + qmax * 2.0 ** -23
+    per_ch = np.abs(q).reshape(1 if per_layer else 9, -1).max(axis=1)
+    assert np.all(per_ch == qmax)
+    # fake quantization is one fp32 multiply of the code by the scale
+    f = O.fake_quantization(x, s, z, "google", bits, "symmetric")
+    assert np.array_equal(f, (q * s.reshape(sb.shape)).astype(np.float32))
+
+
+def test_ties_round_to_even_and_clamp():
+    x = np.array([0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, 126.5, 127.5, 1e9, -128.5, -1e9], np.float32)
+    q = O.quantization(x, np.ones(1, np.float32), np.zeros(1, np.float32))
+    expect = np.array([0, 2, 2, 4, -0.0, -2, -2, 126, 127, 127, -128, -128], np.float32)
+    assert np.array_equal(_bits32(q), _bits32(expect))
+    # affine range is [0, 2^b - 1]; the two zero-point rules agree on integral zero points
+    xa = np.array([-3.0, -0.4, 0.4, 0.5, 1.5, 300.0], np.float32)
+    for mode in ("cpu", "cuda"):
+        qa = O.quantization(xa, np.ones(1, np.float32), np.array([2.0], np.float32), "google", 8,
+                            "affine", zp_mode=mode)
+        assert qa.tolist() == [0.0, 2.0, 2.0, 2.0, 4.0, 255.0]
+    # and differ on a fractional one: CPU rounds it to uint8 first (2.6 -> 3), CUDA does not
+    zp = np.array([2.6], np.float32)
+    cpu = O.quantization(np.array([0.0], np.float32), np.ones(1, np.float32), zp, "google", 8, "affine", zp_mode="cpu")
+    gpu = O.quantization(np.array([0.3], np.float32), np.ones(1, np.float32), zp, "google", 8, "affine", zp_mode="cuda")
+    assert cpu[0] == 3.0 and gpu[0] == 3.0  # rint(0.3 + 2.6 = 2.9)
+    gpu2 = O.quantization(np.array([-0.2], np.float32), np.ones(1, np.float32), zp, "google", 8, "affine", zp_mode="cuda")
+    cpu2 = O.quantization(np.array([-0.2], np.float32), np.ones(1, np.float32), zp, "google", 8, "affine", zp_mode="cpu")
+    assert gpu2[0] == 2.0 and cpu2[0] == 3.0
+
+
+def test_affine_observer_closed_form():
+    x = np.array([[-1.0, 0.0, 3.0, 2.0]], np.float32)
+    s, z = O.min_max_observer(x, "google", 8, "affine", True)
+    assert s[0] == np.float32(4.0) / np.float32(255.0)
+    assert z[0] == -np.rint(np.float32(-1.0) / s[0])
+    s, z = O.min_max_observer(x, "cambricon", 8, "symmetric", True)
+    assert s[0] == np.floor(np.log2(3.0)) - 6 and z[0] == 0  # 2^(1-6) steps
+
+
+def test_double_precision_paths_follow_the_same_rules():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((6, 50))
+    s, z = O.min_max_observer(x, "google", 8, "symmetric", False)
+    assert np.array_equal(s, np.abs(x).max(axis=1) / 127.0)
+    q = O.quantization(x, s, z)
+    assert np.array_equal(q, np.clip(np.rint(x / s[:, None]), -128, 127))
+
+
+# ------------------------------------------------------------------------------------------------
+# fp16 / bf16 conversions of the oracle against numpy / torch
+# ------------------------------------------------------------------------------------------------
+def test_half_and_bf16_conversions():
+    import torch
+    L = O.lib()
+    h = np.arange(65536, dtype=np.uint16)
+    f = np.array([L.ofq_ref_half_to_float(int(v)) for v in h], dtype=np.float32)
+    ref = h.view(np.float16).astype(np.float32)
+    assert np.array_equal(_bits32(f)[~np.isnan(ref)], _bits32(ref)[~np.isnan(ref)])
+    assert np.array_equal(np.isnan(f), np.isnan(ref))
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(20000) * 10.0 ** rng.integers(-9, 6, 20000)).astype(np.float32)
+    hv = rng.integers(0, 0x7BFF, 4000).astype(np.uint16)
+    mid = (hv.view(np.float16).astype(np.float32) + (hv + 1).astype(np.uint16).view(np.float16).astype(np.float32)) / 2
+    edge = np.array([65504, 65519.996, 65520, 65536, 1e-8, 2.0 ** -25, 2.0 ** -24, 6.1e-5, 0, -0.0,
+                     np.inf, -np.inf], dtype=np.float32)
+    x = np.concatenate([x, mid, -mid, edge]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        expect = x.astype(np.float16).view(np.uint16)
+    got = np.array([L.ofq_ref_float_to_half(float(v)) for v in x], dtype=np.uint16)
+    assert np.array_equal(got, expect)
+    got_b = np.array([L.ofq_ref_float_to_bf16(float(v)) for v in x], dtype=np.uint16)
+    exp_b = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got_b, exp_b)
+    assert np.array_equal(O.f32_to_bf16_bits(x), exp_b)
+    assert L.ofq_ref_float_to_bf16(float("nan")) == 0x7FC0
+
+
+# ------------------------------------------------------------------------------------------------
+# groupwise_dequantize
+# ------------------------------------------------------------------------------------------------
+def _round_T(v, t):
+    """Correctly rounded double -> T -> double through numpy (fp16) or torch (bf16)."""
+    import torch
+    if t == "f16":
+        return float(np.float16(v))
+    if t == "bf16":
+        # double -> bf16 in one rounding: go through exact Fraction comparison on fp32 neighbours
+        f = np.float32(v)
+        if float(f) == v:
+            return float(torch.tensor([f]).to(torch.bfloat16).float()[0])
+        # v not representable in fp32: products q*s of an 8-bit code and an 8-bit significand and
+        # sums of two bf16 values always are, so this does not occur here
+        raise AssertionError("unexpected")
+    return float(np.float32(v))
+
+
+@pytest.mark.parametrize("t", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("bits,signed", [(8, False), (8, True), (4, False), (4, True)])
+def test_dequantize_brute_force_all_codes(t, bits, signed):
+    """Every code value x sampled (scale, zero): out = round_T(round_T(q*s) + z) evaluated with
+    Python floats (exact for these operands) and numpy/torch conversions."""
+    rng = np.random.default_rng(bits + signed)
+    lo, hi = (-(1 << (bits - 1)), (1 << (bits - 1))) if signed else (0, 1 << bits)
+    vals = np.arange(lo, hi)
+    group = 256
+    codes = np.resize(vals, group).astype(np.int8 if signed else np.uint8)
+    packed = codes if bits == 8 else H.pack_int4(codes)
+    n_groups = 24
+    q = np.tile(packed, (n_groups, 1))
+    scales = H.as_T(rng.uniform(1e-3, 2.0, size=(n_groups, 1)).astype(np.float32), t)
+    zeros = H.as_T(rng.uniform(-150, 150, size=(n_groups, 1)).astype(np.float32), t)
+    for symmetric in ((True, False) if not signed else (True,)):
+        out = O.groupwise_dequantize(q, scales, None if symmetric else zeros, bits, symmetric, 1, group)
+        outf = O.to_f32(out).astype(np.float64)
+        sf = O.to_f32(scales).astype(np.float64)
+        zf = O.to_f32(zeros).astype(np.float64)
+        for g in range(n_groups):
+            s = float(sf[g, 0])
+            if not symmetric:
+                z = float(zf[g, 0])
+            elif signed:
+                z = 0.0
+            else:
+                z = _round_T(-float((1 << (bits - 1)) - 1) * s, t)
+            for i in range(group):
+                expect = _round_T(_round_T(float(codes[i]) * s, t) + z, t)
+                assert outf[g, i] == expect, (g, i, codes[i], s, z)
+
+
+def test_dequantize_identity_and_nibble_order():
+    codes = np.arange(-128, 128).astype(np.int8).reshape(2, 128)
+    out = O.groupwise_dequantize(codes, np.ones((2, 1), np.float16), None, 8, True, 1, 128)
+    assert np.array_equal(out.astype(np.int32), codes.astype(np.int32))
+    # int4: element 2i is the HIGH nibble (the reference test's packer), both containers
+    v = np.array([[-8, 7, -1, 0, 3, -4, 5, 6]], np.int8)
+    packed = H.pack_int4(v)
+    assert packed.view(np.uint8).tolist() == [[0x87, 0xF0, 0x3C, 0x56]]
+    assert np.array_equal(H.unpack_int4(packed), v)
+    out = O.groupwise_dequantize(packed, np.ones((1, 1), np.float32), None, 4, True, 1, 8)
+    assert out.tolist() == v.astype(np.float32).tolist()
+    u = np.array([[15, 0, 9, 8, 1, 2, 3, 4]], np.uint8)
+    out = O.groupwise_dequantize(H.pack_int4(u), np.ones((1, 1), np.float32),
+                                 np.zeros((1, 1), np.float32), 4, False, 1, 8)
+    assert out.tolist() == u.astype(np.float32).tolist()
+    # symmetric uint8 container: codes are offset by 2^(b-1)-1
+    out = O.groupwise_dequantize(H.pack_int4(u), np.full((1, 1), 0.5, np.float32), None, 4, True, 1, 8)
+    assert out.tolist() == ((u.astype(np.float32) - 7) * 0.5).tolist()
+
+
+@pytest.mark.parametrize("shape,group_dim,group_size", [((6, 8, 16), 0, 3), ((6, 8, 16), 1, 4),
+                                                        ((6, 8, 16), 2, 8), ((5, 7, 6), 1, 7)])
+def test_dequantize_group_axis_layout(shape, group_dim, group_size):
+    """Group axis anywhere: compare with a numpy broadcast of scale/zero over the group axis
+    (fp32, where the two roundings are plain fp32 operations)."""
+    rng = np.random.default_rng(1)
+    q = rng.integers(0, 256, size=shape, dtype=np.uint8)
+    sshape = list(shape)
+    sshape[group_dim] //= group_size
+    scale = rng.uniform(0.01, 1, size=sshape).astype(np.float32)
+    zero = rng.uniform(-5, 5, size=sshape).astype(np.float32)
+    out = O.groupwise_dequantize(q, scale, zero, 8, False, group_dim, group_size)
+    expect = (q.astype(np.float32) * np.repeat(scale, group_size, axis=group_dim)).astype(np.float32) \
+        + np.repeat(zero, group_size, axis=group_dim)
+    assert np.array_equal(out, expect.astype(np.float32))
+
+
+# ------------------------------------------------------------------------------------------------
+# fused linear
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("group_dim", [0, 1])
+def test_fused_linear_integer_case_is_exact(bits, group_dim):
+    """All scales 1, no zero: the op is an integer matrix product, exact in fp32."""
+    rng = np.random.default_rng(bits + group_dim)
+    m, n, k = 3, 32, 64
+    x = rng.integers(-4, 5, size=(m, k)).astype(np.float32)
+    lim = 1 << (bits - 1)
+    codes = rng.integers(-lim, lim, size=(n, k)).astype(np.int8)
+    w = codes if bits == 8 else H.pack_int4(codes)
+    gs = 16
+    scale = np.ones((n, k // gs) if group_dim == 1 else (n // gs, k), np.float32)
+    b = rng.integers(-3, 4, size=n).astype(np.float32)
+    out = O.fused_linear(x, w, scale, None, b, bits, True, group_dim, gs)
+    exact = x.astype(np.int64) @ codes.astype(np.int64).T + b.astype(np.int64)
+    assert np.array_equal(out.astype(np.int64), exact)
+
+
+@pytest.mark.parametrize("t", ["f16", "bf16"])
+def test_fused_linear_is_dequantize_then_matmul(t):
+    """out == round_T(x @ dequantize(w).T + b) with the product taken in float64 by numpy: the
+    oracle's fp32 (and fp64) accumulation must agree to accumulation error, and m-invariance
+    holds bitwise."""
+    rng = np.random.default_rng(3)
+    m, n, k, g = 5, 48, 256, 64
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), t)
+    wf = rng.standard_normal((n, k)).astype(np.float32)
+    b = H.as_T(rng.standard_normal(n).astype(np.float32), t)
+    for bits, sym, qdt in ((4, True, np.int8), (4, False, np.uint8), (8, True, np.uint8)):
+        w, scale, zero = H.quantize_groupwise(wf, bits, sym, 1, g, qdt, t)
+        wd = O.to_f32(O.groupwise_dequantize(w, scale, zero, bits, sym, 1, g)).astype(np.float64)
+        exact = O.to_f32(x).astype(np.float64) @ wd.T + O.to_f32(b).astype(np.float64)
+        for acc in ("f32", "f64"):
+            out = O.to_f32(O.fused_linear(x, w, scale, zero, b, bits, sym, 1, g, acc=acc)).astype(np.float64)
+            assert (np.abs(out - exact) <= H.ulp_of(exact, t) * 0.51 + 1e-4).all()
+        full = O.fused_linear(x, w, scale, zero, b, bits, sym, 1, g)
+        one = O.fused_linear(x[2:3], w, scale, zero, b, bits, sym, 1, g)
+        assert np.array_equal(full[2], one[0])
+
+
+# ------------------------------------------------------------------------------------------------
+# ops absent from the reference (parity with the reference unpinned): closed forms
+# ------------------------------------------------------------------------------------------------
+def test_layer_norm_observer_closed_forms():
+    cols = 64
+    x = np.tile(np.array([2.0, -2.0], np.float32), cols // 2)[None, :].repeat(2, 0)
+    gamma = np.full(cols, 0.5, np.float32)
+    beta = np.full(cols, 0.25, np.float32)
+    y, s, z = O.layer_norm_min_max_observer(x, gamma, beta, 1e-5, 8)
+    inv = np.float32(1.0 / np.sqrt(4.0 + 1e-5))
+    n = (x * inv).astype(np.float32)
+    assert np.array_equal(y, (n * np.float32(0.5)).astype(np.float32) + np.float32(0.25))
+    assert s[0] == np.abs(y).max() / np.float32(127.0) and z[0] == 0
+    # constant rows: variance 0, y = beta
+    y, s, z = O.layer_norm_min_max_observer(np.full((1, 8), 3.0, np.float16), None,
+                                            np.full(8, 0.5, np.float16), 1e-5, 8)
+    assert np.all(y == np.float16(0.5))
+    # against a float64 LayerNorm on random data, to fp16 resolution
+    rng = np.random.default_rng(2)
+    xr = rng.standard_normal((4, 512)).astype(np.float16)
+    g = (1 + 0.1 * rng.standard_normal(512)).astype(np.float16)
+    b = (0.1 * rng.standard_normal(512)).astype(np.float16)
+    y, s, z = O.layer_norm_min_max_observer(xr, g, b, 1e-5, 8)
+    xd = xr.astype(np.float64)
+    ref = (xd - xd.mean(1, keepdims=True)) / np.sqrt(xd.var(1, keepdims=True) + 1e-5) * g + b
+    assert np.abs(y.astype(np.float64) - ref).max() < 4e-3
+    q = O.quantize_to_int8(y, s, 8)
+    assert np.abs(q.astype(np.int32)).max() == 127
+    assert np.array_equal(q, np.clip(np.rint(y.astype(np.float32) / s[0]), -128, 127).astype(np.int8))
+
+
+def test_matmul_quant_exact_integer_accumulation():
+    rng = np.random.default_rng(4)
+    m, n, k = 7, 19, 4096
+    a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, size=(n, k)).astype(np.int8)
+    a[0, :] = -128
+    b[0, :] = -128  # largest accumulator: 4096 * 16384 = 2^26
+    out = O.matmul_quant(a, b, np.ones(1, np.float32), np.ones(n, np.float32), None, np.float32)
+    acc = a.astype(np.int64) @ b.astype(np.int64).T
+    assert np.array_equal(out, acc.astype(np.float32))
+    sa = np.array([0.02], np.float32)
+    sb = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float16)
+    out = O.matmul_quant(a, b, sa, sb, bias, np.float16)
+    expect = (acc.astype(np.float32) * (sa[0] * sb)[None, :] + bias.astype(np.float32)).astype(np.float16)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(out.view(np.uint16), expect.view(np.uint16))
