@@ -9,7 +9,8 @@ weights (32 layers = 3.3 GB of packed weights, far beyond L2 + Infinity Cache, s
 streams its weights from HBM).  value = algorithmic bytes of all launches / wall time of the step.
 
 The same JSON line carries
-  roofline      for the dominant kernel (the K=4096 instance of the MFMA GEMV): algorithmic bytes
+  roofline      for the dominant kernel (the 16-wave instance of the MFMA GEMV, which serves the
+                4096-row shapes: four 4096x4096 and one 4096x11008 per layer): algorithmic bytes
                 per launch / average launch duration, timed live with events on the launch stream
                 over a region that contains only that kernel's launches;
   cpu_baseline  the CPU oracle (scalar C port of the reference composition dequantize -> matmul)
@@ -102,10 +103,10 @@ def main():
             for mat in mats:
                 launch(mat)
 
-    def step_k4096():
+    def step_dominant():
         for mats in layers:
             for mat in mats:
-                if mat[2] == 4096:
+                if mat[1] == 4096:
                     launch(mat)
 
     def make_runner(fn):
@@ -141,15 +142,15 @@ def main():
     ms_per_step = wall_ms / args.steps
     value = bytes_step / (ms_per_step * 1e-3) / 1e9
 
-    # ---- roofline of the dominant kernel: only the K=4096 GEMV launches ------------------------
-    bytes_k4096 = sum(gemv_bytes(M, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER if k == 4096) * args.layers
-    launches_k4096 = sum(cnt for _, n, k, cnt in LLAMA7B_LAYER if k == 4096) * args.layers
-    run_k = make_runner(step_k4096)
+    # ---- roofline of the dominant kernel: only the launches with n = 4096 (16-wave instance) -----
+    bytes_k4096 = sum(gemv_bytes(M, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER if n == 4096) * args.layers
+    launches_k4096 = sum(cnt for _, n, k, cnt in LLAMA7B_LAYER if n == 4096) * args.layers
+    run_k = make_runner(step_dominant)
     ev_k_ms, _ = time_region(run_k, args.steps, args.warmup)
     avg_launch_us = ev_k_ms * 1e3 / (args.steps * launches_k4096)
     achieved = (bytes_k4096 / launches_k4096) / (avg_launch_us * 1e-6) / 1e9
     roofline = {
-        "kernel": "gemv_f16_mfma<4,int8,sym,8 waves> (K=4096 shapes: 4096x4096 x4, 11008x4096 x2 per layer)",
+        "kernel": "gemv_w4s_f16<16 waves, staged x> (n=4096 shapes: 4096x4096 x4, 4096x11008 x1 per layer)",
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
         "bytes_per_launch": bytes_k4096 // launches_k4096, "avg_launch_us": round(avg_launch_us, 3),

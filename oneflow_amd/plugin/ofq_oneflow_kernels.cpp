@@ -1,0 +1,359 @@
+// OneFlow user-op kernels for the quantized-inference family, backed by the HIP library behind
+// include/ofq.h.  This file is the C++ host side of the drop-in: it registers kernels under the
+// reference's op names and argument names and forwards to the C ABI.  It is written against
+// OneFlow's user-op API (oneflow/core/framework/framework.h); with -DOFQ_PLUGIN_STANDALONE it
+// compiles against the minimal restatement in standalone/ so that the registrations can be
+// exercised without a OneFlow build.
+//
+// Replaced registrations (device kCUDA, the only accelerator value of DeviceType,
+// oneflow/core/common/device_type.proto:4-13):
+//   groupwise_dequantize                          groupwise_quantization_kernels.cu:456-463
+//   fused_linear_with_groupwise_quantized_weight  groupwise_quantization_kernels.cu:844-851
+//   min_max_observer                              min_max_observer_kernel.cu:240-258
+//   quantization                                  quantization_kernel.cu:149-156
+//   fake_quantization                             fake_quantization_kernel.cu:150-157
+// bf16 variants are added; kernels carry kKernelPriorityOptimized so that they win over stock
+// kernels registered for the same (op, device, dtype)
+// (oneflow/core/framework/user_op_registry_manager.cpp:95-114).
+#include "oneflow/core/framework/framework.h"
+
+#include "ofq.h"
+
+namespace oneflow {
+
+namespace {
+
+// How the raw stream is obtained is the one place that differs between a real OneFlow build and
+// the standalone build: OneFlow hands out ep::CudaStream::cuda_stream()
+// (oneflow/core/ep/cuda/cuda_stream.h:91); on a ROCm build of the EP layer that handle IS the
+// hipStream_t.
+inline void* RawStream(user_op::KernelComputeContext* ctx) {
+#ifdef OFQ_PLUGIN_STANDALONE
+  return ctx->stream() ? ctx->stream()->raw_stream() : nullptr;
+#else
+  return ctx->stream()->As<ep::CudaStream>()->cuda_stream();
+#endif
+}
+
+inline int ToOfq(DataType dt) {
+  switch (dt) {
+    case DataType::kFloat: return OFQ_F32;
+    case DataType::kFloat16: return OFQ_F16;
+    case DataType::kBFloat16: return OFQ_BF16;
+    case DataType::kDouble: return OFQ_F64;
+    case DataType::kInt8: return OFQ_I8;
+    case DataType::kUInt8: return OFQ_U8;
+    default: UNIMPLEMENTED(); return -1;
+  }
+}
+
+inline void CheckOk(int status, const char* what) {
+  if (status != OFQ_OK) {
+    std::cerr << what << ": " << ofq_status_string(status) << "\n";
+    CHECK_EQ(status, OFQ_OK);
+  }
+}
+
+inline int Scheme(const std::string& s) {
+  return s == "symmetric" ? OFQ_SCHEME_SYMMETRIC : OFQ_SCHEME_AFFINE;
+}
+inline int Formula(const std::string& s) {
+  return s == "google" ? OFQ_FORMULA_GOOGLE : OFQ_FORMULA_CAMBRICON;
+}
+
+}  // namespace
+
+// ---- groupwise_dequantize: args in, scale, [zero] -> out; attrs num_bits, symmetric,
+//      group_dim, group_size (OneFlowUserOps.td:8343-8362) ------------------------------------
+class OfqGroupwiseDequantizeKernel final : public user_op::OpKernel,
+                                           public user_op::CudaGraphSupport {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx) const override {
+    const user_op::Tensor* in = ctx->Tensor4ArgNameAndIndex("in", 0);
+    const user_op::Tensor* scale = ctx->Tensor4ArgNameAndIndex("scale", 0);
+    const user_op::Tensor* zero =
+        ctx->has_input("zero", 0) ? ctx->Tensor4ArgNameAndIndex("zero", 0) : nullptr;
+    user_op::Tensor* out = ctx->Tensor4ArgNameAndIndex("out", 0);
+    const int64_t group_size = ctx->Attr<int64_t>("group_size");
+    const int64_t group_dim = ctx->Attr<int64_t>("group_dim");
+    const int32_t num_bits = ctx->Attr<int32_t>("num_bits");
+    const bool symmetric = ctx->Attr<bool>("symmetric");
+    // shape rules of GroupwiseDequantizeKernel::Compute, groupwise_quantization_kernels.cu:409-437
+    const int64_t axes = in->shape_view().NumAxes();
+    CHECK_GE(axes, 1);
+    CHECK_EQ(scale->shape_view().NumAxes(), axes);
+    CHECK_EQ(out->shape_view().NumAxes(), axes);
+    CHECK_GE(group_dim, 0);
+    CHECK_LT(group_dim, axes);
+    for (int64_t i = 0; i < axes; ++i) {
+      const int64_t f = (i == axes - 1) ? 8 / num_bits : 1;
+      CHECK_EQ(out->shape_view().At(i), in->shape_view().At(i) * f);
+    }
+    const int64_t group_dim_size = out->shape_view().At(group_dim);
+    CHECK_GT(group_size, 0);
+    CHECK_LE(group_size, group_dim_size);
+    CHECK_EQ(group_dim_size % group_size, 0);
+    const int64_t num_groups = group_dim_size / group_size;
+    for (int64_t i = 0; i < axes; ++i) {
+      const int64_t expected = i == group_dim ? num_groups : out->shape_view().At(i);
+      CHECK_EQ(scale->shape_view().At(i), expected);
+      if (zero != nullptr) { CHECK_EQ(zero->shape_view().At(i), expected); }
+    }
+    const int64_t outer = out->shape_view().Count(0, group_dim) * num_groups;
+    const int64_t inner = out->shape_view().Count(group_dim + 1);
+    CheckOk(ofq_groupwise_dequantize(RawStream(ctx), in->dptr(), scale->dptr(),
+                                     zero ? zero->dptr() : nullptr, out->mut_dptr(),
+                                     ToOfq(in->data_type()), ToOfq(scale->data_type()), num_bits,
+                                     symmetric ? 1 : 0, outer, group_size, inner),
+            "groupwise_dequantize");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_DEQUANTIZE(dtype)                                       \
+  REGISTER_USER_KERNEL("groupwise_dequantize")                               \
+      .SetCreateFn<OfqGroupwiseDequantizeKernel>()                           \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)       \
+                       && (user_op::HobDataType("scale", 0) == dtype))       \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_DEQUANTIZE(DataType::kFloat16);
+REGISTER_OFQ_DEQUANTIZE(DataType::kBFloat16);
+REGISTER_OFQ_DEQUANTIZE(DataType::kFloat);
+
+// ---- fused_linear_with_groupwise_quantized_weight: x, w, w_scale, [w_zero], [b] -> out -----
+class OfqFusedLinearKernel final : public user_op::OpKernel, public user_op::CudaGraphSupport {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx, user_op::OpKernelState*,
+               const user_op::OpKernelCache*) const override {
+    const user_op::Tensor* x = ctx->Tensor4ArgNameAndIndex("x", 0);
+    const user_op::Tensor* w = ctx->Tensor4ArgNameAndIndex("w", 0);
+    const user_op::Tensor* w_scale = ctx->Tensor4ArgNameAndIndex("w_scale", 0);
+    const user_op::Tensor* b = ctx->has_input("b", 0) ? ctx->Tensor4ArgNameAndIndex("b", 0) : nullptr;
+    const user_op::Tensor* w_zero =
+        ctx->has_input("w_zero", 0) ? ctx->Tensor4ArgNameAndIndex("w_zero", 0) : nullptr;
+    user_op::Tensor* out = ctx->Tensor4ArgNameAndIndex("out", 0);
+    const DataType data_type = x->data_type();
+    CHECK_EQ(w_scale->data_type(), data_type);
+    CHECK_EQ(out->data_type(), data_type);
+    const int64_t group_size = ctx->Attr<int64_t>("group_size");
+    const int64_t group_dim = ctx->Attr<int64_t>("group_dim");
+    const int32_t num_bits = ctx->Attr<int32_t>("num_bits");
+    const bool symmetric = ctx->Attr<bool>("symmetric");
+    // shape rules of the reference kernel, groupwise_quantization_kernels.cu:778-822
+    CHECK_GE(x->shape_view().NumAxes(), 2);
+    const int64_t k = x->shape_view().At(x->shape_view().NumAxes() - 1);
+    const int64_t m = x->shape_view().elem_cnt() / k;
+    CHECK_EQ(w->shape_view().NumAxes(), 2);
+    CHECK_EQ(w->shape_view().At(1) * (8 / num_bits), k);
+    const int64_t n = w->shape_view().At(0);
+    const int64_t num_groups = (group_dim == 0 ? n : k) / group_size;
+    CHECK_EQ(w_scale->shape_view().At(0), group_dim == 0 ? num_groups : n);
+    CHECK_EQ(w_scale->shape_view().At(1), group_dim == 0 ? k : num_groups);
+    if (w_zero != nullptr) { CHECK(w_zero->shape_view() == w_scale->shape_view()); }
+    if (b != nullptr) { CHECK_EQ(b->shape_view().At(0), n); }
+    CHECK_EQ(out->shape_view().At(out->shape_view().NumAxes() - 1), n);
+    CHECK_EQ(symmetric, w_zero == nullptr);
+    CheckOk(ofq_fused_linear_gq(RawStream(ctx), x->dptr(), w->dptr(), w_scale->dptr(),
+                                w_zero ? w_zero->dptr() : nullptr, b ? b->dptr() : nullptr,
+                                out->mut_dptr(), ToOfq(w->data_type()), ToOfq(data_type), num_bits,
+                                symmetric ? 1 : 0, (int)group_dim, group_size, m, n, k, nullptr, 0),
+            "fused_linear_with_groupwise_quantized_weight");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_FUSED_LINEAR(dtype)                                     \
+  REGISTER_USER_KERNEL("fused_linear_with_groupwise_quantized_weight")       \
+      .SetCreateFn<OfqFusedLinearKernel>()                                   \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)       \
+                       && (user_op::HobDataType("out", 0) == dtype))         \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_FUSED_LINEAR(DataType::kFloat16);
+REGISTER_OFQ_FUSED_LINEAR(DataType::kBFloat16);
+REGISTER_OFQ_FUSED_LINEAR(DataType::kFloat);
+
+// ---- min_max_observer: in -> scale, zero_point (+ tmp_buffer) -------------------------------
+class OfqMinMaxObserverKernel final : public user_op::OpKernel {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx) const override {
+    const user_op::Tensor* in = ctx->Tensor4ArgNameAndIndex("in", 0);
+    user_op::Tensor* scale = ctx->Tensor4ArgNameAndIndex("scale", 0);
+    user_op::Tensor* zero_point = ctx->Tensor4ArgNameAndIndex("zero_point", 0);
+    user_op::Tensor* tmp = ctx->Tensor4ArgNameAndIndex("tmp_buffer", 0);
+    const bool per_layer = ctx->Attr<bool>("per_layer_quantization");
+    const int64_t elem_cnt = in->shape_view().elem_cnt();
+    const int64_t channels = per_layer ? 1 : in->shape_view().At(0);
+    CheckOk(ofq_min_max_observer(RawStream(ctx), in->dptr(), scale->mut_dptr(),
+                                 zero_point->mut_dptr(), ToOfq(in->data_type()), elem_cnt, channels,
+                                 ctx->Attr<int32_t>("quantization_bit"),
+                                 Scheme(ctx->Attr<std::string>("quantization_scheme")),
+                                 Formula(ctx->Attr<std::string>("quantization_formula")),
+                                 tmp->mut_dptr(), (size_t)tmp->shape_view().elem_cnt()),
+            "min_max_observer");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_OBSERVER(dtype)                                                         \
+  REGISTER_USER_KERNEL("min_max_observer")                                                   \
+      .SetCreateFn<OfqMinMaxObserverKernel>()                                                \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)                       \
+                       && (user_op::HobDataType("in", 0) == dtype))                          \
+      .SetInferTmpSizeFn([](user_op::InferContext* ctx) -> size_t {                          \
+        const ShapeView shape = ctx->InputShape("in", 0);                                    \
+        const int64_t channels = ctx->Attr<bool>("per_layer_quantization") ? 1 : shape.At(0);\
+        return ofq_min_max_observer_workspace_bytes(dtype == DataType::kDouble ? OFQ_F64     \
+                                                                               : OFQ_F32,    \
+                                                    shape.elem_cnt(), channels);             \
+      })                                                                                     \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_OBSERVER(DataType::kFloat);
+REGISTER_OFQ_OBSERVER(DataType::kDouble);
+
+// ---- quantization / fake_quantization: in, scale, zero_point -> out ---------------------------
+template<bool kFake>
+class OfqQuantizationKernel final : public user_op::OpKernel {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx) const override {
+    const user_op::Tensor* in = ctx->Tensor4ArgNameAndIndex("in", 0);
+    const user_op::Tensor* scale = ctx->Tensor4ArgNameAndIndex("scale", 0);
+    const user_op::Tensor* zero_point = ctx->Tensor4ArgNameAndIndex("zero_point", 0);
+    user_op::Tensor* out = ctx->Tensor4ArgNameAndIndex("out", 0);
+    const int64_t elem_cnt = in->shape_view().elem_cnt();
+    const int64_t scale_size = scale->shape_view().elem_cnt();
+    const int bits = ctx->Attr<int32_t>("quantization_bit");
+    const int scheme = Scheme(ctx->Attr<std::string>("quantization_scheme"));
+    const int formula = Formula(ctx->Attr<std::string>("quantization_formula"));
+    const int dt = ToOfq(in->data_type());
+    // OFQ_ZP_FLOAT: the zero-point rule of the CUDA kernels this replaces
+    if (kFake) {
+      CheckOk(ofq_fake_quantization(RawStream(ctx), in->dptr(), scale->dptr(), zero_point->dptr(),
+                                    out->mut_dptr(), dt, elem_cnt, scale_size, bits, scheme,
+                                    formula, OFQ_ZP_FLOAT),
+              "fake_quantization");
+    } else {
+      CheckOk(ofq_quantization(RawStream(ctx), in->dptr(), scale->dptr(), zero_point->dptr(),
+                               out->mut_dptr(), dt, dt, elem_cnt, scale_size, bits, scheme,
+                               formula, OFQ_ZP_FLOAT),
+              "quantization");
+    }
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_QUANTIZATION(op_name, fake, dtype)                      \
+  REGISTER_USER_KERNEL(op_name)                                              \
+      .SetCreateFn<OfqQuantizationKernel<fake>>()                            \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)       \
+                       && (user_op::HobDataType("in", 0) == dtype))          \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_QUANTIZATION("quantization", false, DataType::kFloat);
+REGISTER_OFQ_QUANTIZATION("quantization", false, DataType::kDouble);
+REGISTER_OFQ_QUANTIZATION("fake_quantization", true, DataType::kFloat);
+REGISTER_OFQ_QUANTIZATION("fake_quantization", true, DataType::kDouble);
+
+}  // namespace oneflow
+
+#ifdef OFQ_PLUGIN_STANDALONE
+// ---- test hooks of the standalone build ---------------------------------------------------------
+using namespace oneflow;
+
+namespace {
+class RawStreamHolder final : public ep::Stream {
+ public:
+  explicit RawStreamHolder(void* s) : s_(s) {}
+  void* raw_stream() const override { return s_; }
+
+ private:
+  void* s_;
+};
+
+const user_op::KernelRegistration* Lookup(const std::string& op, const user_op::KernelRegContext& c) {
+  const user_op::KernelRegistration* best = nullptr;
+  for (const auto& r : user_op::KernelRegistry()) {
+    if (r.op_type_name == op && r.matched(c) && (best == nullptr || r.priority > best->priority)) {
+      best = &r;
+    }
+  }
+  return best;
+}
+}  // namespace
+
+extern "C" int ofq_plugin_registration_count() { return (int)user_op::KernelRegistry().size(); }
+
+extern "C" int ofq_plugin_registration_info(int i, char* name, int name_cap, int* priority,
+                                            int* needs_tmp) {
+  const auto& regs = user_op::KernelRegistry();
+  if (i < 0 || i >= (int)regs.size()) return -1;
+  const std::string& n = regs[i].op_type_name;
+  int j = 0;
+  for (; j < (int)n.size() && j < name_cap - 1; ++j) name[j] = n[j];
+  name[j] = 0;
+  *priority = regs[i].priority;
+  *needs_tmp = regs[i].infer_tmp_size ? 1 : 0;
+  return 0;
+}
+
+// 1 if a kernel is registered for (op, device, dtype of `arg`)
+extern "C" int ofq_plugin_has_kernel(const char* op, int device, const char* arg, int dtype) {
+  user_op::KernelRegContext c;
+  c.device = (DeviceType)device;
+  c.arg_dtypes[arg] = (DataType)dtype;
+  return Lookup(op, c) != nullptr ? 1 : 0;
+}
+
+// tmp_buffer bytes the observer registration asks the runtime for
+extern "C" long long ofq_plugin_observer_tmp_bytes(int dtype, const long long* shape, int rank,
+                                                   int per_layer) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["in"] = (DataType)dtype;
+  const auto* r = Lookup("min_max_observer", c);
+  if (r == nullptr || !r->infer_tmp_size) return -1;
+  user_op::InferContext ic;
+  ic.shapes["in"] = std::vector<int64_t>(shape, shape + rank);
+  ic.attrs["per_layer_quantization"].b = per_layer != 0;
+  return (long long)r->infer_tmp_size(&ic);
+}
+
+// Runs the registered fused linear kernel on device pointers through a KernelComputeContext,
+// the way the runtime would (2-D x).
+extern "C" int ofq_plugin_run_fused_linear(void* stream, void* x, void* w, void* w_scale,
+                                           void* w_zero, void* b, void* out, int t_dtype,
+                                           int w_dtype, long long m, long long n, long long k,
+                                           int num_bits, int symmetric, long long group_dim,
+                                           long long group_size) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["out"] = (DataType)t_dtype;
+  const auto* r = Lookup("fused_linear_with_groupwise_quantized_weight", c);
+  if (r == nullptr) return -1;
+  RawStreamHolder st(stream);
+  user_op::KernelComputeContext ctx;
+  ctx.stream_ = &st;
+  const DataType T = (DataType)t_dtype;
+  const int64_t groups = (group_dim == 0 ? n : k) / group_size;
+  ctx.AddTensor("x", {m, k}, T, x);
+  ctx.AddTensor("w", {n, k * num_bits / 8}, (DataType)w_dtype, w);
+  if (group_dim == 0) {
+    ctx.AddTensor("w_scale", {groups, k}, T, w_scale);
+    if (w_zero) ctx.AddTensor("w_zero", {groups, k}, T, w_zero);
+  } else {
+    ctx.AddTensor("w_scale", {n, groups}, T, w_scale);
+    if (w_zero) ctx.AddTensor("w_zero", {n, groups}, T, w_zero);
+  }
+  if (b) ctx.AddTensor("b", {n}, T, b);
+  ctx.AddTensor("out", {m, n}, T, out);
+  ctx.attrs["num_bits"].i = num_bits;
+  ctx.attrs["symmetric"].b = symmetric != 0;
+  ctx.attrs["group_dim"].i = group_dim;
+  ctx.attrs["group_size"].i = group_size;
+  auto kernel = r->create();
+  kernel->Compute(&ctx, nullptr, nullptr);
+  return 0;
+}
+#endif  // OFQ_PLUGIN_STANDALONE

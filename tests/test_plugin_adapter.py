@@ -1,0 +1,76 @@
+"""The C++ OneFlow adapter (oneflow_amd/plugin): registrations carry the reference's op names,
+device/dtype predicates and tmp_buffer sizing; on the GPU, a kernel looked up from the registry and
+run through a KernelComputeContext gives the same bits as the direct C-ABI call."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PLUGIN = os.path.join(ROOT, "oneflow_amd", "plugin", "libofq_oneflow_plugin.so")
+# DataType / DeviceType values of oneflow/core/common/data_type.proto and device_type.proto
+K_FLOAT, K_DOUBLE, K_INT8, K_UINT8, K_FLOAT16, K_BFLOAT16 = 2, 3, 4, 7, 9, 11
+K_CPU, K_CUDA = 1, 2
+
+
+@pytest.fixture(scope="module")
+def plugin():
+    if not os.path.exists(PLUGIN):
+        pytest.fail(f"{PLUGIN} missing: run __graft_entry__.build()")
+    return ctypes.CDLL(PLUGIN)
+
+
+def test_registrations(plugin):
+    n = plugin.ofq_plugin_registration_count()
+    seen = {}
+    for i in range(n):
+        name = ctypes.create_string_buffer(128)
+        prio, tmp = ctypes.c_int(), ctypes.c_int()
+        assert plugin.ofq_plugin_registration_info(i, name, 128, ctypes.byref(prio), ctypes.byref(tmp)) == 0
+        seen.setdefault(name.value.decode(), []).append((prio.value, tmp.value))
+    assert set(seen) == {"groupwise_dequantize", "fused_linear_with_groupwise_quantized_weight",
+                         "min_max_observer", "quantization", "fake_quantization"}
+    assert len(seen["groupwise_dequantize"]) == 3 and len(seen["min_max_observer"]) == 2
+    # every kernel outranks a stock registration (priority 0); only the observer needs tmp_buffer
+    assert all(p == 10 for v in seen.values() for p, _ in v)
+    assert all(t == 1 for _, t in seen["min_max_observer"])
+    assert all(t == 0 for _, t in seen["quantization"] + seen["groupwise_dequantize"])
+    has = plugin.ofq_plugin_has_kernel
+    assert has(b"groupwise_dequantize", K_CUDA, b"scale", K_FLOAT16) == 1
+    assert has(b"groupwise_dequantize", K_CUDA, b"scale", K_BFLOAT16) == 1
+    assert has(b"groupwise_dequantize", K_CPU, b"scale", K_FLOAT16) == 0
+    assert has(b"groupwise_dequantize", K_CUDA, b"scale", K_DOUBLE) == 0
+    assert has(b"fused_linear_with_groupwise_quantized_weight", K_CUDA, b"out", K_FLOAT16) == 1
+    assert has(b"quantization", K_CUDA, b"in", K_DOUBLE) == 1
+    assert has(b"quantization", K_CUDA, b"in", K_FLOAT16) == 0
+    assert has(b"matmul", K_CUDA, b"out", K_FLOAT16) == 0
+    plugin.ofq_plugin_observer_tmp_bytes.restype = ctypes.c_longlong
+    shape = (ctypes.c_longlong * 2)(4096, 4096)
+    assert plugin.ofq_plugin_observer_tmp_bytes(K_FLOAT, shape, 2, 0) == 4096 * 2 * 4
+    assert plugin.ofq_plugin_observer_tmp_bytes(K_FLOAT, shape, 2, 1) == 1024 * 2 * 4
+
+
+@pytest.mark.gpu
+def test_fused_linear_through_the_adapter(plugin):
+    import torch
+    import helpers as H
+    import oneflow_amd as flow
+    rng = np.random.default_rng(11)
+    m, n, k, g = 4, 512, 1024, 128
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    w = H.pack_int4(rng.integers(-7, 8, size=(n, k)).astype(np.int8))
+    scale = rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float16)
+    b = (rng.standard_normal(n) * 0.01).astype(np.float16)
+    xt, wt, st, bt = map(H.to_torch, (x, w, scale, b))
+    direct = flow._C.fused_linear_with_groupwise_quantized_weight(
+        xt, wt, st, b=bt, num_bits=4, symmetric=True, group_dim=1, group_size=g)
+    out = torch.empty_like(direct)
+    vp, ll = ctypes.c_void_p, ctypes.c_longlong
+    plugin.ofq_plugin_run_fused_linear.argtypes = [vp] * 7 + [ctypes.c_int] * 2 + [ll] * 3 + [ctypes.c_int] * 2 + [ll] * 2
+    rc = plugin.ofq_plugin_run_fused_linear(
+        torch.cuda.current_stream().cuda_stream, xt.data_ptr(), wt.data_ptr(), st.data_ptr(), None,
+        bt.data_ptr(), out.data_ptr(), K_FLOAT16, K_INT8, m, n, k, 4, 1, 1, g)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, direct)
