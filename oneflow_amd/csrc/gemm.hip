@@ -26,10 +26,8 @@ namespace {
 template<typename T, class MF, int BITS, bool SIGNED, int ZMODE>
 int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
   typedef typename TT<T>::storage S;
-  constexpr int BM = 128, BN = 128;
-  typedef BDequant<T, BITS, SIGNED, ZMODE, BN> BP;
   typedef EpBias<T> EP;
-  typename BP::Params bp;
+  typename BDequant<T, BITS, SIGNED, ZMODE, 128>::Params bp;
   bp.w = static_cast<const uint8_t*>(a.w);
   bp.scale = static_cast<const S*>(a.scale);
   bp.zero = static_cast<const S*>(a.zero);
@@ -40,7 +38,13 @@ int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
   typename EP::Params ep;
   ep.bias = static_cast<const S*>(a.bias);
   ep.out = static_cast<S*>(a.out);
-  return launch_core<MF, BP, EP, BM, BN, 2, 2>(st, a.x, a.k * 2, bp, ep, a.m, a.n, a.k / 64);
+  // 256x128 tiles on 8 waves when there are enough rows of x to fill them, else 128x128 on 4
+  if (a.m > 128) {
+    return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 512>, EP, 256, 128, 4, 2>(
+        st, a.x, a.k * 2, bp, ep, a.m, a.n, a.k / 64);
+  }
+  return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 256>, EP, 128, 128, 2, 2>(
+      st, a.x, a.k * 2, bp, ep, a.m, a.n, a.k / 64);
 }
 
 template<typename T, class MF>
@@ -94,9 +98,7 @@ extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, cons
                 OFQ_ERR_NULL_POINTER);
   OFQ_RETURN_IF(!ofq_aligned16(a) || !ofq_aligned16(b) || !ofq_aligned16(out), OFQ_ERR_MISALIGNED);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  constexpr int BM = 128, BN = 128;
-  typedef BCopy<BN> BP;
-  BP::Params bp;
+  BCopy<128>::Params bp;
   bp.b = static_cast<const uint8_t*>(b);
   bp.ldb = k;
   bp.N = (int)n;
@@ -108,7 +110,12 @@ extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, cons
     ep.b_scale = b_scale;                                                                      \
     ep.bias = static_cast<const TT<T>::storage*>(bias);                                        \
     ep.out = static_cast<TT<T>::storage*>(out);                                                \
-    return launch_core<MfmaI8, BP, EP, BM, BN, 2, 2>(st, a, k, bp, ep, m, n, k / 128);         \
+    if (m > 128) {                                                                             \
+      return launch_core2<MfmaI8, B2Copy<128, 512>, EP, 256, 128, 4, 2>(st, a, k, bp, ep, m,   \
+                                                                        n, k / 128);           \
+    }                                                                                          \
+    return launch_core2<MfmaI8, B2Copy<128, 256>, EP, 128, 128, 2, 2>(st, a, k, bp, ep, m, n,  \
+                                                                      k / 128);                \
   }
   switch (out_dtype) {
     case OFQ_F16: OFQ_MQ(f16)

@@ -15,6 +15,7 @@ constexpr int kThreads = 256;
 // ---- MFMA policies -------------------------------------------------------------------------
 struct MfmaF16 {
   typedef f32x16 Acc;
+  typedef float Scalar;
   static __device__ __forceinline__ Acc mma(u32x4 a, u32x4 b, Acc c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -22,6 +23,7 @@ struct MfmaF16 {
 };
 struct MfmaBF16 {
   typedef f32x16 Acc;
+  typedef float Scalar;
   static __device__ __forceinline__ Acc mma(u32x4 a, u32x4 b, Acc c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -29,6 +31,7 @@ struct MfmaBF16 {
 };
 struct MfmaI8 {
   typedef i32x16 Acc;
+  typedef int Scalar;
   static __device__ __forceinline__ Acc mma(u32x4 a, u32x4 b, Acc c) {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a),
                                                  __builtin_bit_cast(i32x4, b), c, 0, 0, 0);
@@ -157,7 +160,24 @@ struct EpBias {
     if (p.bias != nullptr) acc += TT<T>::load(p.bias + n);
     TT<T>::store(p.out + (int64_t)m * N + n, acc);
   }
-  static __device__ __forceinline__ float widen(float v) { return v; }
+  // four consecutive n (n .. n+3, all < N): bias added in fp32, one rounding to T
+  static __device__ __forceinline__ void convert4(const Params& p, const float* acc, int n,
+                                                  typename TT<T>::storage* out4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = acc[e];
+      if (p.bias != nullptr) v += TT<T>::load(p.bias + n + e);
+      TT<T>::store(out4 + e, v);
+    }
+  }
+  static __device__ __forceinline__ typename TT<T>::storage convert1(const Params& p, float acc,
+                                                                     int n) {
+    typename TT<T>::storage o;
+    if (p.bias != nullptr) acc += TT<T>::load(p.bias + n);
+    TT<T>::store(&o, acc);
+    return o;
+  }
+  typedef T elem_t;
 };
 template<typename T>
 struct EpScale {
@@ -173,6 +193,26 @@ struct EpScale {
     if (p.bias != nullptr) r = r + TT<T>::load(p.bias + n);
     TT<T>::store(p.out + (int64_t)m * N + n, r);
   }
+  static __device__ __forceinline__ void convert4(const Params& p, const int* acc, int n,
+                                                  typename TT<T>::storage* out4) {
+    const float sa = p.a_scale[0];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float s = sa * p.b_scale[n + e];
+      float r = (float)acc[e] * s;
+      if (p.bias != nullptr) r = r + TT<T>::load(p.bias + n + e);
+      TT<T>::store(out4 + e, r);
+    }
+  }
+  static __device__ __forceinline__ typename TT<T>::storage convert1(const Params& p, int acc,
+                                                                     int n) {
+    typename TT<T>::storage o;
+    float r = (float)acc * (p.a_scale[0] * p.b_scale[n]);
+    if (p.bias != nullptr) r = r + TT<T>::load(p.bias + n);
+    TT<T>::store(&o, r);
+    return o;
+  }
+  typedef T elem_t;
 };
 
 // ---- the core ----------------------------------------------------------------------------------
@@ -305,6 +345,442 @@ int launch_core(hipStream_t st, const void* A, int64_t lda, const typename BP::P
   }
   kern<<<m_tiles * n_tiles, kThreads, lds_bytes, st>>>(static_cast<const uint8_t*>(A), lda, bp, ep,
                                                        (int)M, (int)N, (int)KT, m_tiles, n_tiles);
+  return ofq_check_launch();
+}
+
+
+// =================================================================================================
+// Second-generation core: asynchronous global->LDS copies (global_load_lds_dwordx4) for every tile
+// that needs no arithmetic on the way, XOR-swizzled 128-byte LDS rows instead of padding, two LDS
+// stages with the copies issued one full k-tile ahead, and (for quantised weights) the codes
+// fetched two k-tiles ahead into registers and dequantised into LDS in the shadow of the MFMAs.
+//
+// What bounds it: the path L2 -> vector L1 -> LDS delivers 64 bytes per clock per CU, and a k-tile
+// of a BM x BN block needs (BM+BN)*128 bytes for BM*BN/32 MFMA clocks per SIMD.  128x128 needs
+// exactly 64 B/clk at full MFMA rate, 256x128 needs 48, 256x256 needs 32 -- large tiles are not a
+// register-reuse nicety here but the condition for being MFMA-bound at all.
+//
+// LDS addressing.  A wave-level global_load_lds writes 64 x 16 bytes to consecutive LDS addresses,
+// i.e. 8 rows of 128 bytes.  Lane l fills slot (row = l/8, position p = l%8) and fetches the
+// global 16-byte piece c = p ^ (row & 7) of its row, so piece c of row r lives at position
+// c ^ (r & 7).  The fragment reads of 8 consecutive rows (same c) then touch 8 different
+// positions: conflict-free without padding.
+// =================================================================================================
+constexpr int kStageRow = 128;
+
+__device__ __forceinline__ void async_copy16(const uint8_t* gsrc, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(
+      (const __attribute__((address_space(1))) void*)gsrc,
+      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+// wait until at most N of this wave's vector-memory operations (incl. global->LDS copies) are
+// still outstanding; they complete in issue order, so this retires everything but the N newest
+template<int N>
+__device__ __forceinline__ void wait_vmem_le() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
+}
+__device__ __forceinline__ void wait_vmem_all() { wait_vmem_le<0>(); }
+
+// rows [0, ROWS) x 128 bytes of tile kt of a row-major byte matrix -> swizzled LDS tile
+template<int ROWS, int NWAVES>
+__device__ __forceinline__ void async_tile(const uint8_t* __restrict__ g, int64_t ld, int row0,
+                                           int row_limit, int kt, uint8_t* lds_tile, int wave,
+                                           int lane) {
+  static_assert(ROWS % (8 * NWAVES) == 0, "tile rows must split evenly over the waves");
+  const int sub = lane >> 3;                 // row within the 8-row group
+  const int piece = (lane & 7) ^ (sub & 7);  // global piece this lane fetches
+#pragma unroll
+  for (int j = 0; j < ROWS / (8 * NWAVES); ++j) {
+    const int grp = j * NWAVES + wave;  // 8-row group of the tile
+    int row = row0 + grp * 8 + sub;
+    row = row < row_limit ? row : row_limit - 1;
+    async_copy16(g + (int64_t)row * ld + (int64_t)kt * kStageRow + piece * 16,
+                 lds_tile + grp * 1024);
+  }
+}
+
+template<int BN, int NT>
+struct B2Copy {
+  typedef typename BCopy<BN>::Params Params;
+  static constexpr bool kDirect = true;
+  struct Regs {};
+  static __device__ __forceinline__ void load(const Params& p, int n0, int kt, int wave, int lane,
+                                              int, Regs&, uint8_t* lds_b) {
+    async_tile<BN, NT / 64>(p.b, p.ldb, n0, p.N, kt, lds_b, wave, lane);
+  }
+  static __device__ __forceinline__ void store_part(const Params&, const Regs&, uint8_t*, int, int) {}
+};
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// 16 values of T (two 128-bit pieces) from 16 byte codes, w~ = T(T(q)*s) + z.
+// bf16: v_cvt_f32_ubyteN, v_mul_f32, v_cvt_pk_bf16_f32, re-widen, v_add_f32, v_cvt_pk_bf16_f32
+// (5 vector instructions per element); fp16: the 0x6400 trick with packed fp16 math (2 per element).
+template<typename T, bool SIGNED, int ZMODE>
+__device__ __forceinline__ void dequant16_b8(const u32x4 codes, float s, float z, u32x4& o0,
+                                             u32x4& o1) {
+  uint32_t r[8];
+  if constexpr (TT<T>::dtype == OFQ_BF16 && !SIGNED) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t x = codes[w];
+      const f32x2 p01 = {(float)(x & 0xFFu) * s, (float)((x >> 8) & 0xFFu) * s};
+      const f32x2 p23 = {(float)((x >> 16) & 0xFFu) * s, (float)(x >> 24) * s};
+      uint32_t r01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(p01, bf16x2_t));
+      uint32_t r23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(p23, bf16x2_t));
+      if (ZMODE != 0) {
+        const f32x2 a01 = {__builtin_bit_cast(float, r01 << 16) + z,
+                           __builtin_bit_cast(float, r01 & 0xFFFF0000u) + z};
+        const f32x2 a23 = {__builtin_bit_cast(float, r23 << 16) + z,
+                           __builtin_bit_cast(float, r23 & 0xFFFF0000u) + z};
+        r01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(a01, bf16x2_t));
+        r23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(a23, bf16x2_t));
+      }
+      r[2 * w] = r01;
+      r[2 * w + 1] = r23;
+    }
+  } else if constexpr (TT<T>::dtype == OFQ_F16) {
+    const f16 sh = (f16)s, zh = (f16)z;  // s and z were widened from fp16: exact
+    const f16x2 s2 = {sh, sh}, z2 = {zh, zh};
+    const f16 off = SIGNED ? (f16)(-1152.0f) : (f16)(-1024.0f);
+    const f16x2 off2 = {off, off};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      uint32_t word = codes[w];
+      if (SIGNED) word ^= 0x80808080u;
+      f16x2 a = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(word, 0x64646464u, 0x00050004u)) + off2;
+      f16x2 b = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(word, 0x64646464u, 0x00070006u)) + off2;
+      a = a * s2;
+      b = b * s2;
+      if (ZMODE != 0) {
+        a = a + z2;
+        b = b + z2;
+      }
+      r[2 * w] = __builtin_bit_cast(uint32_t, a);
+      r[2 * w + 1] = __builtin_bit_cast(uint32_t, b);
+    }
+  } else {
+    typename TT<T>::storage vals[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const uint32_t b = (codes[e >> 2] >> ((e & 3) * 8)) & 0xFFu;
+      const int code = SIGNED ? (int)(int8_t)b : (int)b;
+      float v = TT<T>::round((float)code * s);
+      if (ZMODE != 0) v = v + z;
+      TT<T>::store(&vals[e], v);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = reinterpret_cast<const uint32_t*>(vals)[i];
+  }
+  o0 = u32x4{r[0], r[1], r[2], r[3]};
+  o1 = u32x4{r[4], r[5], r[6], r[7]};
+}
+
+// Groupwise-quantised weights for the second-generation core: codes are loaded as stored
+// ([N, K*bits/8] bytes) two k-tiles ahead, and turned into T when written to the swizzled LDS tile.
+template<typename T, int BITS, bool SIGNED, int ZMODE, int BN, int NT>
+struct B2Dequant {
+  typedef typename BDequant<T, BITS, SIGNED, ZMODE, BN>::Params Params;
+  static constexpr bool kDirect = false;
+  static constexpr int kCodeBytesPerRow = 64 * BITS / 8;
+  static constexpr int kChunksPerRow = kCodeBytesPerRow / 16;  // 4 (8-bit) or 2 (4-bit)
+  static constexpr int kElemsPerChunk = 16 * 8 / BITS;         // 16 or 32
+  static constexpr int kTotalChunks = BN * kChunksPerRow;
+  static constexpr int kChunks = (kTotalChunks + NT - 1) / NT;
+  static constexpr bool kRagged = kTotalChunks % NT != 0;  // some threads own one chunk less
+  struct Regs {
+    u32x4 v[kChunks];
+    float s[kChunks];
+    float z[kChunks];
+  };
+  static __device__ __forceinline__ void load(const Params& p, int n0, int kt, int, int, int tid,
+                                              Regs& r, uint8_t*) {
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+      const int q = tid + i * NT;
+      if (kRagged && q >= kTotalChunks) continue;
+      int row = n0 + q / kChunksPerRow;
+      row = row < p.N ? row : p.N - 1;
+      const int c = q % kChunksPerRow;
+      r.v[i] = *reinterpret_cast<const u32x4*>(p.w + (int64_t)row * p.ldw
+                                               + (int64_t)kt * kCodeBytesPerRow + c * 16);
+      const int k = kt * 64 + c * kElemsPerChunk;
+      const int64_t si = (int64_t)row * p.G + k / p.group_size;
+      const float s = TT<T>::load(p.scale + si);
+      r.s[i] = s;
+      if (ZMODE == 2) {
+        r.z[i] = TT<T>::load(p.zero + si);
+      } else if (ZMODE == 1) {
+        r.z[i] = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * s);
+      } else {
+        r.z[i] = 0.f;
+      }
+    }
+  }
+  // dequantise and store a quarter of the thread's chunks (all of them when there are fewer)
+  static __device__ __forceinline__ void store_part(const Params&, const Regs& r, uint8_t* lds,
+                                                    int tid, int part) {
+    typedef typename TT<T>::storage S;
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+      if ((kChunks >= 4 ? (i & 3) : (i * (4 / kChunks))) != part) continue;
+      const int q = tid + i * NT;
+      if (kRagged && q >= kTotalChunks) continue;
+      const int row = q / kChunksPerRow;
+      const int c = q % kChunksPerRow;
+      uint8_t* rowp = lds + row * kStageRow;
+      const int sw = row & 7;
+      if constexpr (BITS == 8) {
+        u32x4 o0, o1;
+        dequant16_b8<T, SIGNED, ZMODE>(r.v[i], r.s[i], r.z[i], o0, o1);
+        *reinterpret_cast<u32x4*>(rowp + (((2 * c) ^ sw) << 4)) = o0;
+        *reinterpret_cast<u32x4*>(rowp + (((2 * c + 1) ^ sw) << 4)) = o1;
+      } else {
+        S vals[32];
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+          const uint32_t b = (r.v[i][e >> 3] >> (((e >> 1) & 3) * 8)) & 0xFFu;
+          const int nib = (e & 1) ? (b & 0xF) : (b >> 4);
+          const int code = SIGNED ? ((nib ^ 8) - 8) : nib;
+          float v = TT<T>::round((float)code * r.s[i]);
+          if (ZMODE != 0) v = v + r.z[i];
+          TT<T>::store(&vals[e], v);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<u32x4*>(rowp + (((4 * c + j) ^ sw) << 4)) =
+              reinterpret_cast<const u32x4*>(vals)[j];
+      }
+    }
+  }
+};
+
+// NSTAGE LDS stages; the copies of tile t are issued at the top of iteration t-(NSTAGE-1).
+// DBG (experiments only): 1 = no MFMA, 2 = no global traffic after the prologue
+template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2, int DBG = 0>
+__global__ void __launch_bounds__(WM * WN * 64)
+gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
+           typename EP::Params ep, int M, int N, int KT, int m_tiles, int n_tiles) {
+  constexpr int NWAVES = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int kABytes = BM * kStageRow;
+  constexpr int kStage = (BM + BN) * kStageRow;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  const int nblocks = m_tiles * n_tiles;
+  int logical;
+  {
+    const int b = blockIdx.x;
+    const int xcd = b & 7, idx = b >> 3;
+    const int per = nblocks >> 3, rem = nblocks & 7;
+    logical = xcd < rem ? xcd * (per + 1) + idx : rem * (per + 1) + (xcd - rem) * per + idx;
+  }
+  const int m0 = (logical % m_tiles) * BM;
+  const int n0 = (logical / m_tiles) * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / WN) * WTM;
+  const int wn0 = (wave % WN) * WTN;
+
+  typename MF::Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  typename BP::Regs breg0, breg1;  // codes of even / odd tiles (never indexed dynamically)
+  constexpr int D = NSTAGE - 1;  // prefetch distance of the copies
+  // vector-memory operations a wave issues per iteration for the copies (they are issued last,
+  // so "at most this many outstanding" means: everything older has landed)
+  constexpr int kCopyOps = BM / (8 * NWAVES) + (BP::kDirect ? BN / (8 * NWAVES) : 0);
+  auto stage_of = [&](int t) { return lds + (t % NSTAGE) * kStage; };
+  auto issue_copies = [&](int t, typename BP::Regs& regs) {
+    async_tile<BM, NWAVES>(A, lda, m0, M, t, stage_of(t), wave, lane);
+    if (BP::kDirect) BP::load(bp, n0, t, wave, lane, tid, regs, stage_of(t) + kABytes);
+  };
+
+  // ---- prologue: tile 0 complete in its stage, copies of tiles 1..D-1 and the codes of tile 1
+  //      in flight --------------------------------------------------------------------------------
+  if (!BP::kDirect) {
+    BP::load(bp, n0, 0, wave, lane, tid, breg0, nullptr);
+#pragma unroll
+    for (int part = 0; part < 4; ++part) BP::store_part(bp, breg0, lds + kABytes, tid, part);
+    if (KT > 1) BP::load(bp, n0, 1, wave, lane, tid, breg1, nullptr);
+  }
+  issue_copies(0, breg0);
+  wait_vmem_all();
+#pragma unroll
+  for (int t = 1; t < D; ++t)
+    if (t < KT) issue_copies(t, breg0);
+  __syncthreads();
+
+  // fragment addressing: row = (wave tile row) + i*32 + lane%32, piece c = 2*ks + lane/32 stored
+  // at position c ^ (row & 7); row & 7 == lane & 7 because every tile origin is a multiple of 8
+  const int frag_row = lane & 31;
+  const int x7 = lane & 7;
+  const int half = lane >> 5;
+  int frag_off[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) frag_off[ks] = ((2 * ks + half) ^ x7) << 4;
+
+  // One k-tile.  On entry every wave has passed the barrier that ended iteration kt-1, tile kt is
+  // complete in its stage and the stage of tile kt-1 is free.  `st_regs` holds the codes of tile
+  // kt+1 (requested at the top of iteration kt-1); they are dequantised into that tile's stage
+  // during the MFMAs.  `ld_regs` (free since iteration kt-1) receives the codes of tile kt+2.
+  // Issue order per iteration: code loads first, copies last, so that "at most kCopyOps
+  // outstanding" at the end retires everything except the copies just issued.
+  auto iteration = [&](int kt, typename BP::Regs& st_regs, typename BP::Regs& ld_regs) {
+    const bool more_copies = DBG != 2 && kt + D < KT;
+    if (DBG != 2 && !BP::kDirect && kt + 2 < KT)
+      BP::load(bp, n0, kt + 2, wave, lane, tid, ld_regs, nullptr);
+    if (more_copies) issue_copies(kt + D, ld_regs);
+    uint8_t* cur = stage_of(kt);
+    uint8_t* nxt = stage_of(kt + 1);
+    const uint8_t* a_base = cur + (wm0 + frag_row) * kStageRow;
+    const uint8_t* b_base = cur + kABytes + (wn0 + frag_row) * kStageRow;
+    const bool store_b = !BP::kDirect && (kt + 1 < KT);
+    // fragments of k-step ks+1 are fetched before the MFMAs of k-step ks are issued
+    u32x4 af[2][TM], bf[2][TN];
+    auto fetch = [&](int ks, int set) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[set][i] = *reinterpret_cast<const u32x4*>(a_base + i * 32 * kStageRow + frag_off[ks]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bf[set][j] = *reinterpret_cast<const u32x4*>(b_base + j * 32 * kStageRow + frag_off[ks]);
+    };
+    fetch(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      if (ks < 3) fetch(ks + 1, (ks + 1) & 1);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          if (DBG == 1) {
+            acc[i][j][0] += af[ks & 1][i][0] + bf[ks & 1][j][0];
+          } else {
+            // weights as the first operand: the 32x32 result is D[n][m], so a lane ends up with
+            // 4 CONSECUTIVE n per register quad -- what the row-major output wants
+            acc[i][j] = MF::mma(bf[ks & 1][j], af[ks & 1][i], acc[i][j]);
+          }
+        }
+      // a quarter of the conversions per k-step, in the shadow of the MFMAs just issued
+      if (store_b) BP::store_part(bp, st_regs, nxt + kABytes, tid, ks);
+    }
+    // tile kt+1 must be complete: its copies are older than those issued in this iteration
+    if (D > 1 && more_copies) {
+      wait_vmem_le<kCopyOps>();
+    } else {
+      wait_vmem_all();
+    }
+    __syncthreads();  // ... for every wave, and everyone is done reading `cur`
+  };
+  for (int kt = 0; kt < KT; kt += 2) {
+    iteration(kt, breg1, breg0);
+    if (kt + 1 < KT) iteration(kt + 1, breg0, breg1);
+  }
+
+  // ---- epilogue: registers -> (wave-private, padded) LDS tile -> 128-bit row-contiguous stores --
+  // Each lane holds, per 32x32 tile and register quad g, the 4 consecutive outputs
+  // out[m = .. + lane%32][n = .. + 8g + 4*(lane/32) + 0..3]; they are converted (bias / scales,
+  // one rounding to T), packed to 8 bytes and written to LDS; rows are then read back 16 bytes
+  // per lane so that every global store instruction writes whole row segments.
+  typedef typename EP::elem_t OT;
+  typedef typename TT<OT>::storage OS;
+  static_assert(sizeof(OS) == 2 || sizeof(OS) == 4, "output element size");
+  constexpr int kRowBytesOut = WTN * (int)sizeof(OS) + 8;  // +8: conflict-free 8-byte writes
+  static_assert(NWAVES * WTM * kRowBytesOut <= 160 * 1024, "epilogue tile must fit in LDS");
+  uint8_t* ep_tile = lds + wave * (WTM * kRowBytesOut);  // all waves passed the last barrier
+  const bool vec_ok = (N % 8 == 0) && (n0 + wn0 + WTN <= N);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int nl = j * 32 + 8 * g + 4 * (lane >> 5);  // local n of the quad
+        const int n = n0 + wn0 + nl;
+        OS q[4];
+        typename MF::Acc& a = acc[i][j];
+        if (n + 3 < N) {
+          const typename MF::Scalar quad[4] = {a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+          EP::convert4(ep, quad, n, q);
+        } else {
+          // quad straddles or lies beyond N: element-wise, out-of-range slots are never stored
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            q[e] = OS();
+            if (n + e < N) q[e] = EP::convert1(ep, a[4 * g + e], n + e);
+          }
+        }
+        uint8_t* dst = ep_tile + (i * 32 + (lane & 31)) * kRowBytesOut + nl * (int)sizeof(OS);
+        if (sizeof(OS) == 2) {
+          *reinterpret_cast<u32x2*>(dst) = *reinterpret_cast<const u32x2*>(q);
+        } else {
+          *reinterpret_cast<u32x2*>(dst) = reinterpret_cast<const u32x2*>(q)[0];
+          *reinterpret_cast<u32x2*>(dst + 8) = reinterpret_cast<const u32x2*>(q)[1];
+        }
+      }
+    }
+  }
+  // a wave only reads what it wrote itself; LDS operations of one wave complete in order
+  constexpr int kLanesPerRow = WTN * (int)sizeof(OS) / 16;
+  constexpr int kRowsPerIter = 64 / kLanesPerRow;
+  const int rsub = lane / kLanesPerRow;
+  const int cpiece = lane % kLanesPerRow;
+#pragma unroll
+  for (int it = 0; it < WTM / kRowsPerIter; ++it) {
+    const int ml = it * kRowsPerIter + rsub;
+    const int m = m0 + wm0 + ml;
+    if (m >= M) continue;
+    const uint8_t* src = ep_tile + ml * kRowBytesOut + cpiece * 16;
+    const u32x2 lo = *reinterpret_cast<const u32x2*>(src);
+    const u32x2 hi = *reinterpret_cast<const u32x2*>(src + 8);
+    const int ncol = n0 + wn0 + cpiece * (16 / (int)sizeof(OS));
+    OS* gdst = ep.out + (int64_t)m * N + ncol;
+    const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+    if (vec_ok) {
+      *reinterpret_cast<u32x4*>(gdst) = v;
+    } else {
+      const OS* e = reinterpret_cast<const OS*>(&v);
+#pragma unroll
+      for (int t = 0; t < 16 / (int)sizeof(OS); ++t)
+        if (ncol + t < N) gdst[t] = e[t];
+    }
+  }
+}
+
+template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2, int DBG = 0>
+int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::Params& bp,
+                 const typename EP::Params& ep, int64_t M, int64_t N, int64_t KT) {
+  const int m_tiles = (int)((M + BM - 1) / BM);
+  const int n_tiles = (int)((N + BN - 1) / BN);
+  // two stages, or the epilogue's padded output tile if that is larger
+  constexpr size_t kOutElem = sizeof(typename TT<typename EP::elem_t>::storage);
+  constexpr size_t kEpilogue = (size_t)BM * WN * ((BN / WN) * kOutElem + 8);
+  constexpr size_t kStages = NSTAGE * (size_t)(BM + BN) * kStageRow;
+  const size_t lds_bytes = kStages > kEpilogue ? kStages : kEpilogue;
+  auto kern = gemm_core2<MF, BP, EP, BM, BN, WM, WN, NSTAGE, DBG>;
+  if (lds_bytes > 64 * 1024) {
+    static bool attr_set = false;  // idempotent; a benign race at worst repeats the call
+    if (!attr_set) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)
+          != hipSuccess) {
+        return OFQ_ERR_LAUNCH;
+      }
+      attr_set = true;
+    }
+  }
+  kern<<<m_tiles * n_tiles, WM * WN * 64, lds_bytes, st>>>(
+      static_cast<const uint8_t*>(A), lda, bp, ep, (int)M, (int)N, (int)KT, m_tiles, n_tiles);
   return ofq_check_launch();
 }
 
