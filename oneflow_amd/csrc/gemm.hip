@@ -78,6 +78,16 @@ int launch_gemm_wq(hipStream_t st, const LinearArgs& a) {
   return launch_wq_t<bf16, MfmaBF16>(st, a);
 }
 
+// The int8 GEMM is bound by the L2 -> LDS traffic per MFMA, which falls with the tile area, so a
+// 256x352 tile (one per CU, 8 waves side by side along M) beats 256x128 whenever its tiles fill
+// whole rounds of the 256 CUs reasonably well; with a poor fill the idle tail costs more than the
+// traffic saves.
+bool wide_tiles_pay(int64_t m, int64_t n) {
+  const int64_t tiles = ((m + 255) / 256) * ((n + 351) / 352);
+  const int64_t rounds = (tiles + 255) / 256;
+  return tiles * 100 >= rounds * 256 * 80;
+}
+
 }  // namespace ofq
 
 using namespace ofq;
@@ -110,6 +120,10 @@ extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, cons
     ep.b_scale = b_scale;                                                                      \
     ep.bias = static_cast<const TT<T>::storage*>(bias);                                        \
     ep.out = static_cast<TT<T>::storage*>(out);                                                \
+    if (m > 128 && wide_tiles_pay(m, n)) {                                                     \
+      return launch_core2<MfmaI8, B2Copy<352, 512>, EP, 256, 352, 8, 1>(st, a, k, bp, ep, m,   \
+                                                                        n, k / 128);           \
+    }                                                                                          \
     if (m > 128) {                                                                             \
       return launch_core2<MfmaI8, B2Copy<128, 512>, EP, 256, 128, 4, 2>(st, a, k, bp, ep, m,   \
                                                                         n, k / 128);           \

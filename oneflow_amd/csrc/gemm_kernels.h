@@ -40,13 +40,14 @@ struct MfmaI8 {
 
 // ---- B-tile producers ------------------------------------------------------------------------
 // Plain copy of 128-byte rows (int8 weights of matmul_quant).
+struct BCopyParams {
+  const uint8_t* b;
+  int64_t ldb;  // bytes per row
+  int N;
+};
 template<int BN>
 struct BCopy {
-  struct Params {
-    const uint8_t* b;
-    int64_t ldb;  // bytes per row
-    int N;
-  };
+  typedef BCopyParams Params;
   static constexpr int kChunks = BN * 8 / kThreads;
   struct Regs {
     u32x4 v[kChunks];
@@ -163,10 +164,18 @@ struct EpBias {
   // four consecutive n (n .. n+3, all < N): bias added in fp32, one rounding to T
   static __device__ __forceinline__ void convert4(const Params& p, const float* acc, int n,
                                                   typename TT<T>::storage* out4) {
+    typename TT<T>::storage bias4[4];
+    if (p.bias != nullptr) {
+      if (sizeof(typename TT<T>::storage) == 2) {
+        *reinterpret_cast<u32x2*>(bias4) = *reinterpret_cast<const u32x2*>(p.bias + n);
+      } else {
+        *reinterpret_cast<u32x4*>(bias4) = *reinterpret_cast<const u32x4*>(p.bias + n);
+      }
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       float v = acc[e];
-      if (p.bias != nullptr) v += TT<T>::load(p.bias + n + e);
+      if (p.bias != nullptr) v += TT<T>::load(bias4 + e);
       TT<T>::store(out4 + e, v);
     }
   }
@@ -193,14 +202,24 @@ struct EpScale {
     if (p.bias != nullptr) r = r + TT<T>::load(p.bias + n);
     TT<T>::store(p.out + (int64_t)m * N + n, r);
   }
+  // n is a multiple of 4: the four scales (and biases) come as one aligned vector load
   static __device__ __forceinline__ void convert4(const Params& p, const int* acc, int n,
                                                   typename TT<T>::storage* out4) {
     const float sa = p.a_scale[0];
+    const f32x4 sb = *reinterpret_cast<const f32x4*>(p.b_scale + n);
+    typename TT<T>::storage bias4[4];
+    if (p.bias != nullptr) {
+      if (sizeof(typename TT<T>::storage) == 2) {
+        *reinterpret_cast<u32x2*>(bias4) = *reinterpret_cast<const u32x2*>(p.bias + n);
+      } else {
+        *reinterpret_cast<u32x4*>(bias4) = *reinterpret_cast<const u32x4*>(p.bias + n);
+      }
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float s = sa * p.b_scale[n + e];
+      const float s = sa * sb[e];
       float r = (float)acc[e] * s;
-      if (p.bias != nullptr) r = r + TT<T>::load(p.bias + n + e);
+      if (p.bias != nullptr) r = r + TT<T>::load(bias4 + e);
       TT<T>::store(out4 + e, r);
     }
   }
@@ -387,12 +406,14 @@ template<int ROWS, int NWAVES>
 __device__ __forceinline__ void async_tile(const uint8_t* __restrict__ g, int64_t ld, int row0,
                                            int row_limit, int kt, uint8_t* lds_tile, int wave,
                                            int lane) {
-  static_assert(ROWS % (8 * NWAVES) == 0, "tile rows must split evenly over the waves");
+  static_assert(ROWS % 8 == 0, "tile rows come in groups of 8");
+  constexpr int kGroups = ROWS / 8;
   const int sub = lane >> 3;                 // row within the 8-row group
   const int piece = (lane & 7) ^ (sub & 7);  // global piece this lane fetches
 #pragma unroll
-  for (int j = 0; j < ROWS / (8 * NWAVES); ++j) {
-    const int grp = j * NWAVES + wave;  // 8-row group of the tile
+  for (int j = 0; j < (kGroups + NWAVES - 1) / NWAVES; ++j) {
+    const int grp = j * NWAVES + wave;  // 8-row group of the tile (wave-uniform)
+    if (kGroups % NWAVES != 0 && grp >= kGroups) break;
     int row = row0 + grp * 8 + sub;
     row = row < row_limit ? row : row_limit - 1;
     async_copy16(g + (int64_t)row * ld + (int64_t)kt * kStageRow + piece * 16,
@@ -489,10 +510,12 @@ struct B2Dequant {
   static constexpr int kTotalChunks = BN * kChunksPerRow;
   static constexpr int kChunks = (kTotalChunks + NT - 1) / NT;
   static constexpr bool kRagged = kTotalChunks % NT != 0;  // some threads own one chunk less
+  // scale / zero stay in their storage type until they are used: converting them at load time
+  // would put a wait for the loads right behind their issue
   struct Regs {
     u32x4 v[kChunks];
-    float s[kChunks];
-    float z[kChunks];
+    typename TT<T>::storage s[kChunks];
+    typename TT<T>::storage z[kChunks];
   };
   static __device__ __forceinline__ void load(const Params& p, int n0, int kt, int, int, int tid,
                                               Regs& r, uint8_t*) {
@@ -507,15 +530,8 @@ struct B2Dequant {
                                                + (int64_t)kt * kCodeBytesPerRow + c * 16);
       const int k = kt * 64 + c * kElemsPerChunk;
       const int64_t si = (int64_t)row * p.G + k / p.group_size;
-      const float s = TT<T>::load(p.scale + si);
-      r.s[i] = s;
-      if (ZMODE == 2) {
-        r.z[i] = TT<T>::load(p.zero + si);
-      } else if (ZMODE == 1) {
-        r.z[i] = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * s);
-      } else {
-        r.z[i] = 0.f;
-      }
+      r.s[i] = p.scale[si];
+      if (ZMODE == 2) r.z[i] = p.zero[si];
     }
   }
   // dequantise and store a quarter of the thread's chunks (all of them when there are fewer)
@@ -531,9 +547,13 @@ struct B2Dequant {
       const int c = q % kChunksPerRow;
       uint8_t* rowp = lds + row * kStageRow;
       const int sw = row & 7;
+      const float sc = TT<T>::load(&r.s[i]);
+      float zc = 0.f;
+      if (ZMODE == 2) zc = TT<T>::load(&r.z[i]);
+      if (ZMODE == 1) zc = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * sc);
       if constexpr (BITS == 8) {
         u32x4 o0, o1;
-        dequant16_b8<T, SIGNED, ZMODE>(r.v[i], r.s[i], r.z[i], o0, o1);
+        dequant16_b8<T, SIGNED, ZMODE>(r.v[i], sc, zc, o0, o1);
         *reinterpret_cast<u32x4*>(rowp + (((2 * c) ^ sw) << 4)) = o0;
         *reinterpret_cast<u32x4*>(rowp + (((2 * c + 1) ^ sw) << 4)) = o1;
       } else {
@@ -543,8 +563,8 @@ struct B2Dequant {
           const uint32_t b = (r.v[i][e >> 3] >> (((e >> 1) & 3) * 8)) & 0xFFu;
           const int nib = (e & 1) ? (b & 0xF) : (b >> 4);
           const int code = SIGNED ? ((nib ^ 8) - 8) : nib;
-          float v = TT<T>::round((float)code * r.s[i]);
-          if (ZMODE != 0) v = v + r.z[i];
+          float v = TT<T>::round((float)code * sc);
+          if (ZMODE != 0) v = v + zc;
           TT<T>::store(&vals[e], v);
         }
 #pragma unroll
@@ -557,7 +577,8 @@ struct B2Dequant {
 };
 
 // NSTAGE LDS stages; the copies of tile t are issued at the top of iteration t-(NSTAGE-1).
-// DBG (experiments only): 1 = no MFMA, 2 = no global traffic after the prologue
+// DBG (experiments only): 1 = no MFMA, 2 = no global traffic after the prologue,
+// 5 = codes are fetched but not converted
 template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2, int DBG = 0>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
@@ -598,6 +619,8 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
   constexpr int D = NSTAGE - 1;  // prefetch distance of the copies
   // vector-memory operations a wave issues per iteration for the copies (they are issued last,
   // so "at most this many outstanding" means: everything older has landed)
+  static_assert(NSTAGE == 2 || (BM % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0),
+                "deeper pipelines need the same number of copies in every wave");
   constexpr int kCopyOps = BM / (8 * NWAVES) + (BP::kDirect ? BN / (8 * NWAVES) : 0);
   auto stage_of = [&](int t) { return lds + (t % NSTAGE) * kStage; };
   auto issue_copies = [&](int t, typename BP::Regs& regs) {
@@ -645,7 +668,9 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
     const uint8_t* a_base = cur + (wm0 + frag_row) * kStageRow;
     const uint8_t* b_base = cur + kABytes + (wn0 + frag_row) * kStageRow;
     const bool store_b = !BP::kDirect && (kt + 1 < KT);
-    // fragments of k-step ks+1 are fetched before the MFMAs of k-step ks are issued
+    // fragments of k-step ks+1 are fetched before the MFMAs of k-step ks are issued (when the
+    // fragment set is small enough to keep twice in registers)
+    constexpr bool kDoubleFrag = (TM + TN) <= 6;
     u32x4 af[2][TM], bf[2][TN];
     auto fetch = [&](int ks, int set) {
 #pragma unroll
@@ -655,24 +680,29 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
       for (int j = 0; j < TN; ++j)
         bf[set][j] = *reinterpret_cast<const u32x4*>(b_base + j * 32 * kStageRow + frag_off[ks]);
     };
-    fetch(0, 0);
+    if (kDoubleFrag) fetch(0, 0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      if (ks < 3) fetch(ks + 1, (ks + 1) & 1);
+      const int set = kDoubleFrag ? (ks & 1) : 0;
+      if (kDoubleFrag) {
+        if (ks < 3) fetch(ks + 1, (ks + 1) & 1);
+      } else {
+        fetch(ks, 0);
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
           if (DBG == 1) {
-            acc[i][j][0] += af[ks & 1][i][0] + bf[ks & 1][j][0];
+            acc[i][j][0] += af[set][i][0] + bf[set][j][0];
           } else {
             // weights as the first operand: the 32x32 result is D[n][m], so a lane ends up with
             // 4 CONSECUTIVE n per register quad -- what the row-major output wants
-            acc[i][j] = MF::mma(bf[ks & 1][j], af[ks & 1][i], acc[i][j]);
+            acc[i][j] = MF::mma(bf[set][j], af[set][i], acc[i][j]);
           }
         }
       // a quarter of the conversions per k-step, in the shadow of the MFMAs just issued
-      if (store_b) BP::store_part(bp, st_regs, nxt + kABytes, tid, ks);
+      if (store_b && DBG != 5) BP::store_part(bp, st_regs, nxt + kABytes, tid, ks);
     }
     // tile kt+1 must be complete: its copies are older than those issued in this iteration
     if (D > 1 && more_copies) {
@@ -695,64 +725,75 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
   typedef typename EP::elem_t OT;
   typedef typename TT<OT>::storage OS;
   static_assert(sizeof(OS) == 2 || sizeof(OS) == 4, "output element size");
-  constexpr int kRowBytesOut = WTN * (int)sizeof(OS) + 8;  // +8: conflict-free 8-byte writes
-  static_assert(NWAVES * WTM * kRowBytesOut <= 160 * 1024, "epilogue tile must fit in LDS");
+  // The wave tile is written in panels of JP 32-column MFMA tiles so that the staging area of all
+  // waves fits in the stage memory.
+  constexpr int kLdsBudget = NSTAGE * kStage;
+  constexpr int JP0 = (kLdsBudget / (NWAVES * WTM) - 8) / (32 * (int)sizeof(OS));
+  constexpr int JP = JP0 >= TN ? TN : (JP0 >= 4 ? (JP0 / 2) * 2 : JP0);  // whole 128-byte pieces
+  static_assert(JP >= 1, "no room for the epilogue staging area");
+  constexpr int kRowBytesOut = JP * 32 * (int)sizeof(OS) + 8;  // +8: conflict-free 8-byte writes
   uint8_t* ep_tile = lds + wave * (WTM * kRowBytesOut);  // all waves passed the last barrier
-  const bool vec_ok = (N % 8 == 0) && (n0 + wn0 + WTN <= N);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int jp = 0; jp < TN; jp += JP) {
+    const int panel_cols = (TN - jp < JP ? TN - jp : JP) * 32;
+    const int ncol0 = n0 + wn0 + jp * 32;  // first column of the panel
+    const bool vec_ok = (N % 8 == 0) && (ncol0 + panel_cols <= N);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int nl = j * 32 + 8 * g + 4 * (lane >> 5);  // local n of the quad
-        const int n = n0 + wn0 + nl;
-        OS q[4];
-        typename MF::Acc& a = acc[i][j];
-        if (n + 3 < N) {
-          const typename MF::Scalar quad[4] = {a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
-          EP::convert4(ep, quad, n, q);
-        } else {
-          // quad straddles or lies beyond N: element-wise, out-of-range slots are never stored
+      for (int jj = 0; jj < JP; ++jj) {
+        const int j = jp + jj;
+        if (j >= TN) break;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            q[e] = OS();
-            if (n + e < N) q[e] = EP::convert1(ep, a[4 * g + e], n + e);
+        for (int g = 0; g < 4; ++g) {
+          const int nl = jj * 32 + 8 * g + 4 * (lane >> 5);  // column of the quad in the panel
+          const int n = ncol0 + nl;
+          OS q[4];
+          typename MF::Acc& a = acc[i][j];
+          if (n + 3 < N) {
+            const typename MF::Scalar quad[4] = {a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+            EP::convert4(ep, quad, n, q);
+          } else {
+            // quad straddles or lies beyond N: element-wise, out-of-range slots are never stored
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              q[e] = OS();
+              if (n + e < N) q[e] = EP::convert1(ep, a[4 * g + e], n + e);
+            }
           }
-        }
-        uint8_t* dst = ep_tile + (i * 32 + (lane & 31)) * kRowBytesOut + nl * (int)sizeof(OS);
-        if (sizeof(OS) == 2) {
-          *reinterpret_cast<u32x2*>(dst) = *reinterpret_cast<const u32x2*>(q);
-        } else {
-          *reinterpret_cast<u32x2*>(dst) = reinterpret_cast<const u32x2*>(q)[0];
-          *reinterpret_cast<u32x2*>(dst + 8) = reinterpret_cast<const u32x2*>(q)[1];
+          uint8_t* dst = ep_tile + (i * 32 + (lane & 31)) * kRowBytesOut + nl * (int)sizeof(OS);
+          if (sizeof(OS) == 2) {
+            *reinterpret_cast<u32x2*>(dst) = *reinterpret_cast<const u32x2*>(q);
+          } else {
+            *reinterpret_cast<u32x2*>(dst) = reinterpret_cast<const u32x2*>(q)[0];
+            *reinterpret_cast<u32x2*>(dst + 8) = reinterpret_cast<const u32x2*>(q)[1];
+          }
         }
       }
     }
-  }
-  // a wave only reads what it wrote itself; LDS operations of one wave complete in order
-  constexpr int kLanesPerRow = WTN * (int)sizeof(OS) / 16;
-  constexpr int kRowsPerIter = 64 / kLanesPerRow;
-  const int rsub = lane / kLanesPerRow;
-  const int cpiece = lane % kLanesPerRow;
+    // a wave only reads what it wrote itself; LDS operations of one wave complete in order.
+    // 16 bytes per lane: piece p of row r, pieces_per_row = panel bytes / 16.
+    const int pieces_per_row = panel_cols * (int)sizeof(OS) / 16;
+    const int total_pieces = WTM * pieces_per_row;
+    for (int t = lane; t < total_pieces; t += 64) {
+      const int ml = t / pieces_per_row;
+      const int cpiece = t - ml * pieces_per_row;
+      const int m = m0 + wm0 + ml;
+      if (m >= M) continue;
+      const uint8_t* src = ep_tile + ml * kRowBytesOut + cpiece * 16;
+      const u32x2 lo = *reinterpret_cast<const u32x2*>(src);
+      const u32x2 hi = *reinterpret_cast<const u32x2*>(src + 8);
+      const int ncol = ncol0 + cpiece * (16 / (int)sizeof(OS));
+      OS* gdst = ep.out + (int64_t)m * N + ncol;
+      const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+      if (vec_ok) {
+        *reinterpret_cast<u32x4*>(gdst) = v;
+      } else {
+        const OS* e = reinterpret_cast<const OS*>(&v);
 #pragma unroll
-  for (int it = 0; it < WTM / kRowsPerIter; ++it) {
-    const int ml = it * kRowsPerIter + rsub;
-    const int m = m0 + wm0 + ml;
-    if (m >= M) continue;
-    const uint8_t* src = ep_tile + ml * kRowBytesOut + cpiece * 16;
-    const u32x2 lo = *reinterpret_cast<const u32x2*>(src);
-    const u32x2 hi = *reinterpret_cast<const u32x2*>(src + 8);
-    const int ncol = n0 + wn0 + cpiece * (16 / (int)sizeof(OS));
-    OS* gdst = ep.out + (int64_t)m * N + ncol;
-    const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
-    if (vec_ok) {
-      *reinterpret_cast<u32x4*>(gdst) = v;
-    } else {
-      const OS* e = reinterpret_cast<const OS*>(&v);
-#pragma unroll
-      for (int t = 0; t < 16 / (int)sizeof(OS); ++t)
-        if (ncol + t < N) gdst[t] = e[t];
+        for (int t2 = 0; t2 < 16 / (int)sizeof(OS); ++t2)
+          if (ncol + t2 < N) gdst[t2] = e[t2];
+      }
     }
   }
 }
@@ -762,11 +803,8 @@ int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::
                  const typename EP::Params& ep, int64_t M, int64_t N, int64_t KT) {
   const int m_tiles = (int)((M + BM - 1) / BM);
   const int n_tiles = (int)((N + BN - 1) / BN);
-  // two stages, or the epilogue's padded output tile if that is larger
-  constexpr size_t kOutElem = sizeof(typename TT<typename EP::elem_t>::storage);
-  constexpr size_t kEpilogue = (size_t)BM * WN * ((BN / WN) * kOutElem + 8);
-  constexpr size_t kStages = NSTAGE * (size_t)(BM + BN) * kStageRow;
-  const size_t lds_bytes = kStages > kEpilogue ? kStages : kEpilogue;
+  // the stages; the epilogue stages its output panels in the same memory
+  const size_t lds_bytes = NSTAGE * (size_t)(BM + BN) * kStageRow;
   auto kern = gemm_core2<MF, BP, EP, BM, BN, WM, WN, NSTAGE, DBG>;
   if (lds_bytes > 64 * 1024) {
     static bool attr_set = false;  // idempotent; a benign race at worst repeats the call

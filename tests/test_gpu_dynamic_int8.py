@@ -105,3 +105,36 @@ def test_matmul_quant_small_exact(m, n, k, t):
                                                         "bf16": np.uint16}[t])
     assert np.array_equal(got.view(np.uint16 if t != "f32" else np.uint32),
                           ref.view(np.uint16 if t != "f32" else np.uint32))
+
+
+@pytest.mark.parametrize("t", ["f32", "bf16"])
+def test_matmul_quant_wide_tiles_full_output(t):
+    """A shape that is dispatched to the 256x352 tiles with ragged last tiles in both m and n;
+    every output is checked.  The int32 accumulators come from a float64 matmul, which is exact
+    here (|sum| <= 128*128*256 < 2^53)."""
+    import oneflow_amd as flow
+    import torch
+    m, n, k = 2053, 8196, 256
+    rng = np.random.Generator(np.random.PCG64(99))
+    a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, size=(n, k)).astype(np.int8)
+    a_scale = np.array([0.0071], np.float32)
+    b_scale = rng.uniform(1e-3, 1e-2, size=n).astype(np.float32)
+    bias = H.as_T(rng.standard_normal(n).astype(np.float32), t)
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16}[t]
+    got = H.to_numpy(flow._C.matmul_quant(H.to_torch(a), H.to_torch(b), H.to_torch(a_scale),
+                                          H.to_torch(b_scale), H.to_torch(bias), tdt))
+    acc = (a.astype(np.float64) @ b.astype(np.float64).T)
+    assert np.abs(acc).max() < 2**31
+    sc = (a_scale[0] * b_scale).astype(np.float32)
+    val = (acc.astype(np.float32) * sc[None, :]).astype(np.float32) + O.to_f32(bias)[None, :]
+    if t == "f32":
+        assert np.array_equal(got, val.astype(np.float32))
+    else:
+        assert np.array_equal(got, O.f32_to_bf16_bits(val))
+    # the oracle itself on a corner that includes the ragged edges
+    rows, cols = np.arange(m - 40, m), np.arange(n - 70, n)
+    ref = O.matmul_quant(a[rows], b[cols], a_scale, b_scale[cols], bias[cols],
+                         {"f32": np.float32, "bf16": np.uint16}[t])
+    view = np.uint32 if t == "f32" else np.uint16
+    assert np.array_equal(got[np.ix_(rows, cols)].view(view), ref.view(view))
