@@ -32,6 +32,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the dominant kernel (mean over its launches of one step) from two
+# `rocprofv3 --pmc` runs of `bench.py --pmc-calibration` (FETCH_SIZE, then WRITE_SIZE, each scaled
+# by what the same counter reads for an elementwise kernel of known size: x2.0 and x1.0); the
+# summary is profiles/gemv_w4s_f16__llama7b_decode_m1__hbm_traffic_pmc.txt.  Valid for m = 1 only.
+PMC_TRAFFIC_BYTES_PER_LAUNCH_M1 = 11819780
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "i8": 5000.0}
 
 LLAMA7B_LAYER = [  # (name, n, k, count per decoder layer)
@@ -57,6 +62,10 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch directly instead of replaying a HIP graph")
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="for a `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` run: a few direct launches of "
+                         "the hot path plus an elementwise kernel of known traffic (1 GiB read, "
+                         "1 GiB written) to scale the counters by; prints no result line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU by design (the path has no collectives); "
@@ -135,6 +144,16 @@ def main():
         wall_ms = (time.perf_counter() - t0) * 1e3
         return e0.elapsed_time(e1), wall_ms
 
+    if args.pmc_calibration:
+        src = torch.zeros(256 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)  # vectorized_elementwise_kernel: 2^30 B in, 2^30 B out
+        for _ in range(2):
+            step_all()
+        torch.cuda.synchronize()
+        return
+
     bytes_step = sum(gemv_bytes(M, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER) * args.layers
     launches_step = sum(cnt for *_, cnt in LLAMA7B_LAYER) * args.layers
     run_all = make_runner(step_all)
@@ -152,7 +171,8 @@ def main():
     roofline = {
         "kernel": "gemv_w4s_f16<16 waves, staged x> (n=4096 shapes: 4096x4096 x4, 4096x11008 x1 per layer)",
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": PMC_TRAFFIC_BYTES_PER_LAUNCH_M1 if (M == 1 and args.layers == 32) else None,
         "bytes_per_launch": bytes_k4096 // launches_k4096, "avg_launch_us": round(avg_launch_us, 3),
     }
 
@@ -184,18 +204,19 @@ def cpu_baseline(M):
     rng = np.random.default_rng(0)
     total_bytes = 0
     t_total = 0.0
+    reps = 4  # about 10 s of scalar CPU work
     for name, n, k, cnt in LLAMA7B_LAYER:
         w = rng.integers(-128, 128, size=(n, k // 2), dtype=np.int8)
         scale = rng.uniform(1e-3, 1e-2, size=(n, k // 128)).astype(np.float16)
         bias = (rng.standard_normal(n) * 0.01).astype(np.float16)
         x = rng.standard_normal((M, k)).astype(np.float16)
         t0 = time.perf_counter()
-        for _ in range(cnt):
+        for _ in range(cnt * reps):
             O.fused_linear(x, w, scale, None, bias, 4, True, 1, 128)
         t_total += time.perf_counter() - t0
-        total_bytes += gemv_bytes(M, n, k) * cnt
+        total_bytes += gemv_bytes(M, n, k) * cnt * reps
     return {"value": round(total_bytes / t_total / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"one Llama-7B decoder layer (7 GEMVs, {total_bytes} algorithmic bytes, m={M}) "
+            "sample": f"{reps} Llama-7B decoder layers ({7 * reps} GEMVs, {total_bytes} algorithmic bytes, m={M}) "
                       f"through oracle/ofq_oracle.c in {t_total:.2f} s; host has {os.cpu_count()} cpus"}
 
 
