@@ -215,14 +215,15 @@ __device__ __forceinline__ void permute_unit(const u32x4 a, const u32x4 b, u32x4
   for (int i = 0; i < 4; ++i) hi[i] = as_u32(as_h2(hi[i]) * sixteenth);
 }
 
-// 1032 * (sum of the low-nibble x) + 72 * (sum of the high-nibble x) of one permuted unit
+// 1032 * (sum of the low-nibble x) + 72 * (sum of the high-nibble x) of one permuted unit;
+// v_dot2_f32_f16 against (1, 1) adds two halves into an fp32 sum per instruction
 __device__ __forceinline__ float unit_corr(const u32x4 lo, const u32x4 hi) {
+  const f16x2 ones = {(f16)1.0f, (f16)1.0f};
   float sl = 0.f, sh = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const f16x2 l = as_h2(lo[i]), h = as_h2(hi[i]);
-    sl += (float)l[0] + (float)l[1];
-    sh += (float)h[0] + (float)h[1];
+    sl = __builtin_amdgcn_fdot2(as_h2(lo[i]), ones, sl, false);
+    sh = __builtin_amdgcn_fdot2(as_h2(hi[i]), ones, sh, false);
   }
   return 1032.0f * sl + 1152.0f * sh;  // hi carries x/16: 72 * 16 = 1152
 }
@@ -233,7 +234,17 @@ __device__ __forceinline__ float unit_corr_of(const u32x4 a, const u32x4 b) {
   return unit_corr(lo, hi);
 }
 
-template<int NWAVES, int UNROLL, bool STAGED>
+// DBG (timing experiments only, results are then wrong): 1 = no MFMA/bit work, 2 = no LDS x
+// operand reads, 4 = no cross-wave reduction, 8 = no x staging.
+// Pins the widening of a prefetched bias value to the place of use: without the empty asm the
+// compiler sinks the conversion (and the wait for every load issued so far) up to the load.
+__device__ __forceinline__ f16 bias_at_end(uint16_t raw) {
+  uint32_t v = raw;
+  asm volatile("" : "+v"(v));
+  return __builtin_bit_cast(f16, (uint16_t)v);
+}
+
+template<int NWAVES, int UNROLL, bool STAGED, int DBG = 0>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
              const f16* __restrict__ scale, const f16* __restrict__ bias,
@@ -264,11 +275,12 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const bool has_x = r < M;
 
   // ---- loads that feed LDS are issued first so that they return before the weights ---------
-  const int nunits = STAGED ? (M * K) >> 4 : 0;
+  const int nunits = (STAGED && !(DBG & 8)) ? (M * K) >> 4 : 0;
   u32x4 xu[kGemvMaxUnits][2];
   if (STAGED) {
 #pragma unroll
     for (int i = 0; i < kGemvMaxUnits; ++i) {
+      if (wave * 64 + i * NT >= nunits) break;  // wave-uniform: nothing left for this wave
       const int u = tid + i * NT;
       if (u < nunits) {
         const u32x4* src = reinterpret_cast<const u32x4*>(x + (int64_t)u * 16);
@@ -288,6 +300,13 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
     const int e = (tid + i * NT) * 8;  // first half-element of this 16-byte piece
     s_vec[i] = e + 8 <= tile_halves;
     if (s_vec[i]) sreg[i] = *reinterpret_cast<const u32x4*>(stile + e);
+  }
+
+  // the bias of the outputs this thread will write at the very end (tid = m * 16 + n)
+  // (kept as raw bits: widening it here would wait for every load issued so far)
+  uint16_t bias_raw = 0;
+  if (bias != nullptr && tid < M * 16 && n0 + (tid & 15) < N) {
+    bias_raw = reinterpret_cast<const uint16_t*>(bias)[n0 + (tid & 15)];
   }
 
   auto chunk_of = [&](int p0, int u) { return 2 * (p0 + (u >> 1) * NWAVES) + (u & 1); };
@@ -315,6 +334,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   if (STAGED) {
 #pragma unroll
     for (int i = 0; i < kGemvMaxUnits; ++i) {
+      if (wave * 64 + i * NT >= nunits) break;
       const int u = tid + i * NT;
       if (u < nunits) {
         u32x4 lo, hi;
@@ -365,7 +385,10 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
       const int c = chunk_of(p0, u);
       if (c < nchunks) {
         u32x4 xa[4];
-        if (STAGED) {
+        if (DBG & 2) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) xa[t] = u32x4{0x3c003c00u + (uint32_t)c, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+        } else if (STAGED) {
           const u32x4* xp = reinterpret_cast<const u32x4*>(xrec + c * xrec_stride);
 #pragma unroll
           for (int t = 0; t < 4; ++t) xa[t] = xp[t];
@@ -381,9 +404,13 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
         // the accumulator starts at -corr (staged), or corr is built alongside (not staged)
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         f32x4 corr = {0.f, 0.f, 0.f, 0.f};
-        if (STAGED) acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
+        if (STAGED && !(DBG & 2)) acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
+        if (DBG & 1) {
+          acc[0] += __builtin_bit_cast(float, wq[u][0] ^ wq[u][1] ^ xa[0][0]);
+          acc[1] += __builtin_bit_cast(float, wq[u][2] ^ wq[u][3] ^ xa[1][0] ^ xa[2][1] ^ xa[3][2]);
+        }
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < 2 && !(DBG & 1); ++h) {
           const uint32_t w0 = wq[u][2 * h];
           const uint32_t w1 = wq[u][2 * h + 1];
           const uint32_t w0s = w0 >> 8, w1s = w1 >> 8;
@@ -420,23 +447,291 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
       for (int u = 0; u < UNROLL; ++u) wq[u] = wq_next[u];
     }
   }
-  // lane holds D[m = 4*kb + v][n = n0 + r]
+  // lane holds D[m = 4*kb + v][n = n0 + r]; only rows m < M travel through LDS
+  if (DBG & 4) {
+    if (wave == 0 && kb == 0 && n0 + r < N) out[n0 + r] = (f16)(total[0] + total[1] + total[2] + total[3]);
+    return;
+  }
 #pragma unroll
-  for (int v = 0; v < 4; ++v) red[(wave * 64 + lane) * 4 + v] = total[v];
+  for (int v = 0; v < 4; ++v) {
+    const int m = 4 * kb + v;
+    if (m < M) red[(wave * 16 + m) * 16 + r] = total[v];
+  }
   __syncthreads();
-  for (int t = tid; t < 256; t += NT) {
-    const int l = t >> 2;
-    const int v = t & 3;
+  if (tid < M * 16) {
     float sum = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < NWAVES; ++wv) sum += red[(wv * 64 + l) * 4 + v];
-    const int m = 4 * (l >> 4) + v;
-    const int n = n0 + (l & 15);
-    if (m < M && n < N) {
-      if (bias != nullptr) sum += (float)bias[n];
+    for (int wv = 0; wv < NWAVES; ++wv) sum += red[wv * 256 + tid];
+    const int m = tid >> 4;
+    const int n = n0 + (tid & 15);
+    if (n < N) {
+      sum += (float)bias_at_end(bias_raw);
       out[(int64_t)m * N + n] = (f16)sum;
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Row-balanced variant of the fast path.  The grid is a whole number of blocks per CU and every
+// block owns `rows_per_block` CONSECUTIVE weight rows (any count up to 16 * kW4pMaxTiles), which
+// it walks as 16-row tiles with a partial last tile: all blocks stream the same number of bytes
+// whatever n is (11008 rows = 43 per block on 256 CUs, where 16-row blocks would leave a third of
+// the CUs a tile short), and x is permuted into LDS once per block, not once per 16 rows, which
+// is what makes m > 1 affordable (the staged x is m*k*2 bytes per block).  The 16 waves take the
+// (tile, chunk-pair) items of the block round-robin and keep one item in flight beyond the one
+// they work on; partial sums go to LDS per (tile, wave) and are folded after a single barrier.
+// Arithmetic is that of gemv_w4s_f16.
+// ---------------------------------------------------------------------------------------------
+constexpr int kW4pMaxTiles = 4;
+
+template<int NWAVES, int kW4pDepth = 2>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+             const f16* __restrict__ scale, const f16* __restrict__ bias,
+             f16* __restrict__ out, int M, int N, int K, int group_size, int cpg_shift,
+             int rows_per_block) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NT = NWAVES * 64;
+  const int nchunks = K >> 7;
+  const int npairs = (nchunks + 1) >> 1;
+  const int G = K / group_size;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15;
+  const int kb = lane >> 4;
+  const int row0 = blockIdx.x * rows_per_block;
+  int rows_blk = N - row0;
+  if (rows_blk > rows_per_block) rows_blk = rows_per_block;
+  if (rows_blk <= 0) return;
+  const int ntiles = (rows_blk + 15) >> 4;
+  const bool has_x = r < M;
+
+  // LDS: [red ntiles*NWAVES*M*16 f32][scales rows_per_block*G halves, padded to 16 B]
+  //      [corr nchunks*16 f32][64 zero bytes][x records M*nchunks*256 B]
+  float* red = reinterpret_cast<float*>(smem);
+  const int red_floats = kW4pMaxTiles * NWAVES * M * 16;
+  f16* sl = reinterpret_cast<f16*>(smem + (size_t)red_floats * 4);
+  float* corr_l = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(sl)
+                                           + ((rows_per_block * G * 2 + 15) & ~15));
+  uint8_t* zrec = reinterpret_cast<uint8_t*>(corr_l) + nchunks * 64;
+  uint8_t* xs = zrec + 64;
+
+  // ---- requests that feed LDS go out first ----------------------------------------------------
+  const int nunits = (M * K) >> 4;
+  u32x4 xu[kGemvMaxUnits][2];
+#pragma unroll
+  for (int i = 0; i < kGemvMaxUnits; ++i) {
+    if (wave * 64 + i * NT >= nunits) break;
+    const int u = tid + i * NT;
+    if (u < nunits) {
+      const u32x4* src = reinterpret_cast<const u32x4*>(x + (int64_t)u * 16);
+      xu[i][0] = src[0];
+      xu[i][1] = src[1];
+    }
+  }
+  // the scales of the block's rows are one contiguous piece
+  const int tile_halves = rows_blk * G;
+  const f16* stile = scale + (int64_t)row0 * G;
+  const bool s_aligned = ((reinterpret_cast<uintptr_t>(stile)) & 15u) == 0;
+  u32x4 sreg;
+  const int se = tid * 8;
+  const bool s_vec = s_aligned && se + 8 <= tile_halves;
+  if (s_vec) sreg = *reinterpret_cast<const u32x4*>(stile + se);
+  // bias of the output this thread folds at the end: tid = (tile * M + m) * 16 + n
+  // (kept as raw bits: widening it here would wait for every load issued so far)
+  uint16_t bias_raw = 0;
+  {
+    const int t = tid / (M * 16);
+    const int n = row0 + t * 16 + (tid & 15);
+    if (bias != nullptr && t < ntiles && (t * 16 + (tid & 15)) < rows_blk) {
+      bias_raw = reinterpret_cast<const uint16_t*>(bias)[n];
+    }
+  }
+
+  // ---- the wave's items: j = wave, wave + NWAVES, ... over ntiles * npairs; the first
+  // kW4pDepth of them are requested now, before anything is waited for (for the usual shapes
+  // that is all of them: the block's whole share of the weights is in flight at once)
+  const uint8_t* wbase = w + (int64_t)row0 * (K >> 1) + kb * 16;
+  // Straight-line on purpose: a load under a branch (even a uniform one) makes the compiler
+  // wait for everything in flight at the first LDS fill.  A slot without an item (live = false)
+  // reads one and the same 16 bytes in every lane, a single cached request; lanes past the
+  // block's rows re-read its first row (their outputs are never stored).
+  auto issue = [&](int tile, int pair, u32x4 (&dst)[2], bool live) {
+    const int row_l = tile * 16 + r;
+    const bool ok = row_l < rows_blk;
+    const uint8_t* p = wbase + (int64_t)(ok ? row_l : 0) * (K >> 1);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = 2 * pair + u;
+      const uint8_t* q = p + (c < nchunks ? c : 0) * 64;
+      dst[u] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4*>(live ? q : w + (int64_t)row0 * (K >> 1)));
+    }
+  };
+  auto advance = [&](int& tile, int& pair, int by) {
+    pair += by;
+    while (pair >= npairs) {
+      pair -= npairs;
+      ++tile;
+    }
+  };
+  int it_tile[kW4pDepth], it_pair[kW4pDepth];
+  u32x4 wq[kW4pDepth][2];
+#pragma unroll
+  for (int d = 0; d < kW4pDepth; ++d) {
+    it_tile[d] = 0;
+    it_pair[d] = wave + d * NWAVES;
+    advance(it_tile[d], it_pair[d], 0);
+    // unconditional, so that the wait counts stay exact: a slot without an item reads one and
+    // the same 16 bytes in every lane (a single cached request)
+    {
+      const bool live = it_tile[d] < ntiles;
+      issue(live ? it_tile[d] : 0, live ? it_pair[d] : 0, wq[d], live);
+    }
+  }
+
+  // ---- fill LDS -------------------------------------------------------------------------------
+  for (int e = tid; e < red_floats / 4; e += NT) reinterpret_cast<f32x4*>(red)[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (s_vec) {
+    *reinterpret_cast<u32x4*>(sl + se) = sreg;
+  } else if (se < tile_halves && s_aligned) {
+    for (int j = se; j < tile_halves && j < se + 8; ++j) sl[j] = stile[j];
+  }
+  for (int e = (s_aligned ? NT * 8 : 0) + tid; e < tile_halves; e += NT) sl[e] = stile[e];
+  if (tid < 16) reinterpret_cast<uint32_t*>(zrec)[tid] = 0u;
+#pragma unroll
+  for (int i = 0; i < kGemvMaxUnits; ++i) {
+    if (wave * 64 + i * NT >= nunits) break;
+    const int u = tid + i * NT;
+    if (u < nunits) {
+      u32x4 lo, hi;
+      permute_unit(xu[i][0], xu[i][1], lo, hi);
+      u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32);
+      dst[0] = lo;
+      dst[1] = hi;
+    }
+    float cpart = u < nunits ? unit_corr_of(xu[i][0], xu[i][1]) : 0.f;
+    cpart += __shfl_xor(cpart, 1, 64);
+    cpart += __shfl_xor(cpart, 2, 64);
+    cpart += __shfl_xor(cpart, 4, 64);
+    if (u < nunits && (u & 7) == 0) {
+      const int m = (u >> 3) / nchunks;
+      const int c = (u >> 3) - m * nchunks;
+      corr_l[c * 16 + m] = -cpart;
+    }
+  }
+  __syncthreads();
+
+  const uint8_t* xrec = has_x ? xs + ((size_t)r * nchunks) * 256 + kb * 64 : zrec;
+  const int xrec_stride = has_x ? 256 : 0;
+  f32x4 total = {0.f, 0.f, 0.f, 0.f};
+  auto flush = [&](int t) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int m = 4 * kb + v;
+      if (m < M) red[((t * NWAVES + wave) * M + m) * 16 + r] = total[v];
+    }
+  };
+
+  // one item = the chunk pair `pair` of tile `tile`, codes in slot d
+  auto process = [&](int d, int tile, int pair) {
+    const f16* slr = sl + (tile * 16 + r) * G;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = 2 * pair + u;
+      if (c < nchunks) {
+        const u32x4* xp = reinterpret_cast<const u32x4*>(xrec + c * xrec_stride);
+        u32x4 xa[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xa[t] = xp[t];
+        const float s = (float)slr[cpg_shift >= 0 ? (c >> cpg_shift) : (c * 128 / group_size)];
+        f32x4 acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const uint32_t w0 = wq[d][u][2 * h];
+          const uint32_t w1 = wq[d][u][2 * h + 1];
+          const uint32_t w0s = w0 >> 8, w1s = w1 >> 8;
+          u32x4 blo, bhi;
+          blo[0] = (w0 & 0x000F000Fu) ^ 0x64086408u;
+          blo[1] = (w0s & 0x000F000Fu) ^ 0x64086408u;
+          blo[2] = (w1 & 0x000F000Fu) ^ 0x64086408u;
+          blo[3] = (w1s & 0x000F000Fu) ^ 0x64086408u;
+          bhi[0] = (w0 & 0x00F000F0u) ^ 0x64806480u;
+          bhi[1] = (w0s & 0x00F000F0u) ^ 0x64806480u;
+          bhi[2] = (w1 & 0x00F000F0u) ^ 0x64806480u;
+          bhi[3] = (w1s & 0x00F000F0u) ^ 0x64806480u;
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h]),
+                                                       __builtin_bit_cast(f16x8, blo), acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h + 1]),
+                                                       __builtin_bit_cast(f16x8, bhi), acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) total[v] = __builtin_fmaf(acc[v], s, total[v]);
+      }
+    }
+  };
+  auto next_or_flush = [&](int d, int tile) {
+    if (it_tile[(d + 1) % kW4pDepth] != tile) {
+      flush(tile);
+      total = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  // items of this wave: wave, wave + NWAVES, ... < nitems
+  const int nitems = ntiles * npairs;
+  int left = nitems > wave ? (nitems - wave + NWAVES - 1) / NWAVES : 0;
+  // steady state: every slot is consumed and refilled unconditionally, so the compiler's wait
+  // before each slot is exact (the 2 * (kW4pDepth - 1) younger loads stay in flight)
+  while (left >= 2 * kW4pDepth) {
+#pragma unroll
+    for (int d = 0; d < kW4pDepth; ++d) {
+      const int tile = it_tile[d], pair = it_pair[d];
+      process(d, tile, pair);
+      advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
+      issue(it_tile[d], it_pair[d], wq[d], true);
+      next_or_flush(d, tile);
+    }
+    left -= kW4pDepth;
+  }
+  // tail: fewer than 2 * kW4pDepth items are left; at most kW4pDepth - 1 refills
+#pragma unroll
+  for (int d = 0; d < kW4pDepth; ++d) {
+    const int tile = it_tile[d], pair = it_pair[d];
+    if (d < left) {
+      process(d, tile, pair);
+      advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
+      if (d + kW4pDepth < left) issue(it_tile[d], it_pair[d], wq[d], true);
+      next_or_flush(d, tile);
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < kW4pDepth - 1; ++d) {
+    const int tile = it_tile[d], pair = it_pair[d];
+    if (d + kW4pDepth < left) {
+      process(d, tile, pair);
+      advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
+      next_or_flush(d, tile);
+    }
+  }
+  __syncthreads();
+  if (tid < ntiles * M * 16) {
+    const int t = tid / (M * 16);
+    const int rem = tid - t * (M * 16);  // m * 16 + n
+    float sum = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < NWAVES; ++wv) sum += red[(t * NWAVES + wv) * M * 16 + rem];
+    const int m = rem >> 4;
+    const int row_l = t * 16 + (rem & 15);
+    if (row_l < rows_blk) {
+      out[(int64_t)m * N + row0 + row_l] = (f16)(sum + (float)bias_at_end(bias_raw));
+    }
+  }
+}
+
+inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block) {
+  const int G = K / group_size;
+  return (size_t)kW4pMaxTiles * nwaves * M * 16 * 4 + ((rows_per_block * G * 2 + 15) & ~15)
+         + (size_t)(K >> 7) * 64 + 64 + (size_t)M * K * 2;
 }
 
 // dynamic LDS bytes of gemv_w4s_f16

@@ -7,9 +7,12 @@
 // affine `* gamma + beta` is then carried out in T (two more roundings).
 // Observer (oneflow/user/kernels/min_max_observer_kernel.cu:117-131): scale = absmax / (2^(b-1)-1).
 //
-// One block per row.  The row is read from HBM once (128-bit loads) and kept in registers for
-// the three uses (sum, squared deviations, normalise); the block's absmax of the stored values
-// goes to workspace[row], and a second one-block launch folds the rows and divides.
+// Rows of up to 4096 elements: one WAVE per row.  The row is read from HBM once (128-bit loads,
+// 1 KB per wave instruction) and kept in registers for the three uses (sum, squared deviations,
+// normalise); the reductions are cross-lane only, so no barrier and no LDS is involved and the
+// waves of a CU drift apart, which overlaps one wave's loads with another's stores.  Longer rows
+// use one block per row.  The absmax of the stored values goes to the workspace (one float per
+// wave or per row) and a second one-wave launch folds them and divides.
 #include "ofq_device.h"
 
 namespace ofq {
@@ -114,6 +117,119 @@ ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
   if (threadIdx.x == 0) row_absmax[row] = amax;
 }
 
+// Raw 8-element packs (16 bytes of fp16/bf16, 32 bytes of fp32) and their widening to fp32.
+template<typename T>
+struct RawPack {
+  u32x4 q[sizeof(typename TT<T>::storage) * 8 / 16];
+};
+template<typename T>
+__device__ __forceinline__ RawPack<T> load_raw(const typename TT<T>::storage* p) {
+  RawPack<T> r;
+#pragma unroll
+  for (int i = 0; i < (int)(sizeof(r.q) / 16); ++i) r.q[i] = reinterpret_cast<const u32x4*>(p)[i];
+  return r;
+}
+template<typename T>
+__device__ __forceinline__ void widen(const RawPack<T>& r, float* f) {
+  typedef typename TT<T>::storage S;
+  const S* e = reinterpret_cast<const S*>(r.q);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f[i] = TT<T>::load(&e[i]);
+}
+
+// One wave per row; NP = packs of 8 elements each lane caches: cols <= 64 * 8 * NP and 8 | cols.
+// A wave walks rows gw, gw + nwaves, ... and leaves the absmax over all of them in wave_absmax[gw].
+// x, gamma and beta are all requested before anything is waited for and stay in registers in
+// storage format (half the registers of fp32 for the 16-bit types), so the row's critical path
+// holds one memory round trip, not two.
+template<typename T, int NP>
+__global__ void __launch_bounds__(kLnBlock)
+ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
+                      const typename TT<T>::storage* __restrict__ gamma,
+                      const typename TT<T>::storage* __restrict__ beta,
+                      typename TT<T>::storage* __restrict__ y, float* __restrict__ wave_absmax,
+                      int64_t rows, int64_t cols, float eps) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t gw = (int64_t)blockIdx.x * (kLnBlock / kWave) + (threadIdx.x >> 6);
+  const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / kWave);
+  const int npacks = (int)(cols / 8);
+  float amax = 0.0f;
+  RawPack<T> gr[NP], br[NP];
+  bool first = true;
+  for (int64_t row = gw; row < rows; row += nwaves) {
+    const typename TT<T>::storage* xr = x + row * cols;
+    typename TT<T>::storage* yr = y + row * cols;
+    RawPack<T> v[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + i * kWave;
+      if (p < npacks) v[i] = load_raw<T>(xr + (int64_t)p * 8);
+    }
+    if (first) {
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const int p = lane + i * kWave;
+        if (p < npacks) {
+          if (gamma) gr[i] = load_raw<T>(gamma + (int64_t)p * 8);
+          if (beta) br[i] = load_raw<T>(beta + (int64_t)p * 8);
+        }
+      }
+      first = false;
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + i * kWave;
+      if (p < npacks) {
+        float f[8];
+        widen<T>(v[i], f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += f[e];
+      }
+    }
+    sum = wave_reduce(sum, OpSum());
+    const float mean = sum / (float)cols;
+    float m2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + i * kWave;
+      if (p < npacks) {
+        float f[8];
+        widen<T>(v[i], f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = f[e] - mean;
+          m2 = __builtin_fmaf(d, d, m2);
+        }
+      }
+    }
+    m2 = wave_reduce(m2, OpSum());
+    const float var = fmaxf(m2 / (float)cols, 0.0f);
+    const float inv = 1.0f / __builtin_sqrtf(var + eps);
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + i * kWave;
+      if (p < npacks) {
+        float f[8], g[8], b[8], o[8];
+        widen<T>(v[i], f);
+        if (gamma) widen<T>(gr[i], g);
+        if (beta) widen<T>(br[i], b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float t = TT<T>::round((f[e] - mean) * inv);
+          if (gamma) t = TT<T>::round(t * g[e]);
+          if (beta) t = TT<T>::round(t + b[e]);
+          o[e] = t;
+          amax = fmaxf(amax, fabsf(t));
+        }
+        store8<T>(yr + (int64_t)p * 8, o);
+      }
+    }
+  }
+  amax = wave_reduce(amax, OpMax());
+  if (lane == 0 && gw < rows) wave_absmax[gw] = amax;
+}
+
 // any cols: three passes over the row through L2 (the row was just read, so only the first
 // pass touches HBM), scalar accesses.
 template<typename T>
@@ -151,13 +267,19 @@ ln_observer_rows_generic(const typename TT<T>::storage* __restrict__ x,
   if (threadIdx.x == 0) row_absmax[row] = amax;
 }
 
-__global__ void __launch_bounds__(kLnBlock)
-ln_observer_finalize(const float* __restrict__ row_absmax, int64_t rows, int bits,
+// one wave folds the n partial maxima
+__global__ void __launch_bounds__(kWave)
+ln_observer_finalize(const float* __restrict__ part, int64_t n, int bits,
                      float* __restrict__ scale, float* __restrict__ zero_point) {
-  __shared__ float smem[kLnBlock / kWave];
   float amax = 0.0f;
-  for (int64_t r = threadIdx.x; r < rows; r += kLnBlock) amax = fmaxf(amax, row_absmax[r]);
-  amax = block_reduce(amax, OpMax(), smem);
+  const int64_t n4 = (reinterpret_cast<uintptr_t>(part) & 15u) == 0 ? n / 4 : 0;
+  const f32x4* p4 = reinterpret_cast<const f32x4*>(part);
+  for (int64_t i = threadIdx.x; i < n4; i += kWave) {
+    const f32x4 q = p4[i];
+    amax = fmaxf(fmaxf(amax, fmaxf(q[0], q[1])), fmaxf(q[2], q[3]));
+  }
+  for (int64_t i = n4 * 4 + threadIdx.x; i < n; i += kWave) amax = fmaxf(amax, part[i]);
+  amax = wave_reduce(amax, OpMax());
   if (threadIdx.x == 0) {
     const float denominator = (float)(1 << (bits - 1)) - 1.0f;
     *scale = amax / denominator;
@@ -178,7 +300,28 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
                       && ofq_aligned16(gamma) && ofq_aligned16(beta)
                       && (cols * sizeof(S)) % 16 == 0;
   const int64_t npacks = cols / 8;
-  if (vec_ok && npacks <= kLnBlock) {
+  int64_t nparts = rows;
+  constexpr int kWavesPerBlock = kLnBlock / kWave;
+  // fp32 rows beyond 2048 elements would not fit a lane's registers at two waves per SIMD
+  const int64_t wave_packs = (sizeof(S) == 4 ? 4 : 8) * kWave;
+  if (vec_ok && npacks <= wave_packs) {
+    // every wave resident at once (8 per CU) when there are that many rows
+    const int64_t waves = rows < 256 * 8 ? rows : 256 * 8;
+    const int grid = (int)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+    nparts = (int64_t)grid * kWavesPerBlock < rows ? (int64_t)grid * kWavesPerBlock : rows;
+#define OFQ_LN_WAVE(NPV)                                                                  \
+  ln_observer_wave_rows<T, NPV><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, cols, eps)
+    if (npacks <= kWave) {
+      OFQ_LN_WAVE(1);
+    } else if (npacks <= 2 * kWave) {
+      OFQ_LN_WAVE(2);
+    } else if (npacks <= 4 * kWave) {
+      OFQ_LN_WAVE(4);
+    } else {
+      OFQ_LN_WAVE(8);
+    }
+#undef OFQ_LN_WAVE
+  } else if (vec_ok && npacks <= kLnBlock) {
     ln_observer_rows<T, 1><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
   } else if (vec_ok && npacks <= 2 * kLnBlock) {
     ln_observer_rows<T, 2><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
@@ -187,7 +330,7 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
   } else {
     ln_observer_rows_generic<T><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
   }
-  ln_observer_finalize<<<1, kLnBlock, 0, st>>>(ws, rows, bits, scale, zero_point);
+  ln_observer_finalize<<<1, kWave, 0, st>>>(ws, nparts, bits, scale, zero_point);
   return ofq_check_launch();
 }
 

@@ -114,9 +114,53 @@ bool w4s_supported(const LinearArgs& a) {
          && a.k <= (1 << 20) && a.n <= 0x7FFFFFFF - 16;
 }
 
+// Row-balanced kernel: grid = a whole number of blocks per CU (or one 16-row tile per block when
+// n is small), rows_per_block <= 64.
+template<int NW>
+int launch_w4p_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block, size_t lds,
+                    int cpg_shift) {
+  auto kern = gemv_w4p_f16<NW, 1>;
+  static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be allowed once
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
+                                  static_cast<const f16*>(a.scale),
+                                  static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
+                                  (int)a.m, (int)a.n, (int)a.k, (int)a.group_size, cpg_shift,
+                                  rows_per_block);
+  return ofq_check_launch();
+}
+
+// OFQ_ERR_UNSUPPORTED when the shape does not fit the row-balanced kernel
+int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift) {
+  constexpr int kCUs = 256;
+  const int64_t max_rows = 16 * kW4pMaxTiles;
+  // one block per CU when that keeps a block within 64 rows, else two, else as many 64-row
+  // blocks as it takes
+  int64_t grid = kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
+  const int rpb = (int)((a.n + grid - 1) / grid);
+  grid = (a.n + rpb - 1) / rpb;
+  const bool two_per_cu = grid > kCUs;
+  const int nw = two_per_cu ? 8 : 16;
+  if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
+  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb);
+  if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
+  return two_per_cu ? launch_w4p_inst<8>(st, a, (int)grid, rpb, lds, cpg_shift)
+                    : launch_w4p_inst<16>(st, a, (int)grid, rpb, lds, cpg_shift);
+}
+
 int launch_w4s(hipStream_t st, const LinearArgs& a) {
   const int64_t tiles = (a.n + 15) / 16;
   const int npairs = (int)((a.k / 128 + 1) / 2);
+  const int cpg_shift = ilog2_exact(a.group_size / 128);
   // waves per block: as many as still let every block be resident at once (<= 24 waves per CU on
   // 256 CUs), so the kernel runs as a single round of blocks; never more than there are pairs
   int nw = 16;
@@ -129,7 +173,12 @@ int launch_w4s(hipStream_t st, const LinearArgs& a) {
     staged = false;
     lds = gemv_w4s_lds_bytes(nw, false, (int)a.m, (int)a.k, (int)a.group_size);
   }
-  const int cpg_shift = ilog2_exact(a.group_size / 128);
+  // More than one 16-row tile per CU, or an x too large to stage per 16 rows: the row-balanced
+  // kernel (equal bytes per block, x staged once per block) is the faster one.
+  if (tiles > 256 || !staged) {
+    const int rc = launch_w4p(st, a, cpg_shift);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
 #define OFQ_W4S(NWV)                                                                   \
   if (nw == NWV)                                                                       \
     return staged ? launch_w4s_inst<NWV, true>(st, a, lds, cpg_shift)                  \

@@ -70,6 +70,30 @@ def test_decode_w4a16_llama_shapes(m, n, k, container):
     assert r < (5e-4 if container == np.int8 else 1e-4)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 5000, 256), (3, 4099, 384), (16, 6000, 128), (2, 40000, 256),
+                                   (5, 33000, 128), (8, 4112, 1024)])
+def test_decode_w4a16_row_balanced_shapes(m, n, k):
+    """n large enough that a block owns more than one 16-row tile, with row counts per block
+    that are not multiples of 16, partial last blocks and more blocks than fit the chip at once."""
+    rng = np.random.Generator(np.random.PCG64(n + m))
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), "f16")
+    codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    w = H.pack_int4(codes)
+    scale = H.as_T(rng.uniform(1e-3, 1e-2, size=(n, k // 128)).astype(np.float32), "f16")
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), "f16")
+    ref = O.fused_linear(x, w, scale, None, b, 4, True, 1, 128)
+    got = _run(x, w, scale, None, b, 4, True, 1, 128)
+    r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k}")
+    assert r < 5e-4
+    # exact integer case through the same path: scales 1, small integer x
+    xi = rng.integers(-2, 3, size=(m, k)).astype(np.float16)
+    ones = np.ones((n, k // 128), dtype=np.float16)
+    got = _run(xi, w, ones, None, None, 4, True, 1, 128)
+    exact = xi.astype(np.int64) @ codes.astype(np.int64).T
+    assert np.abs(exact).max() < 2048
+    assert np.array_equal(got.astype(np.int64), exact)
+
+
 def test_decode_m_invariance_and_integer_case():
     """Row i of an m=8 call agrees with the m=1 call on that row (the two batch sizes take
     different code paths: x staged in LDS or not, so agreement is to fp32-accumulation noise, at
