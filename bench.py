@@ -249,16 +249,24 @@ def secondary(L, _lib, torch, dev, args):
     sc = torch.empty((n, k // g), device=dev).uniform_(1e-3, 1e-2).to(torch.bfloat16)
     ze = torch.empty((n, k // g), device=dev).uniform_(120, 136).to(torch.bfloat16)
     o = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    ws_bytes = L.ofq_fused_linear_gq_workspace_bytes(_lib.U8, _lib.BF16, 8, 0, 1, g, m, n, k)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)  # the op's tmp_buffer
     us = timeit(lambda: chk(L.ofq_fused_linear_gq(cs(), x.data_ptr(), w.data_ptr(), sc.data_ptr(),
                                                   ze.data_ptr(), None, o.data_ptr(), _lib.U8,
-                                                  _lib.BF16, 8, 0, 1, g, m, n, k, None, 0), "prefill"))
+                                                  _lib.BF16, 8, 0, 1, g, m, n, k, ws.data_ptr(),
+                                                  ws_bytes), "prefill"))
+    us_fused = timeit(lambda: chk(L.ofq_fused_linear_gq(cs(), x.data_ptr(), w.data_ptr(),
+                                                        sc.data_ptr(), ze.data_ptr(), None,
+                                                        o.data_ptr(), _lib.U8, _lib.BF16, 8, 0, 1,
+                                                        g, m, n, k, None, 0), "prefill"))
     flops = 2.0 * m * n * k
     tf = flops / (us * 1e-6) / 1e12
     out["prefill_w8a16_bf16_m2048"] = {
-        "us": round(us, 2), "tflops": round(tf, 1),
+        "us": round(us, 2), "tflops": round(tf, 1), "workspace_bytes": ws_bytes,
+        "us_without_workspace": round(us_fused, 2),
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS["bf16"],
                      "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS["bf16"], 4)}}
-    del x, w, sc, ze, o
+    del x, w, sc, ze, o, ws
 
     # ---- config 2: groupwise_dequantize 11008x4096 uint8 asym g=128 -> fp16 ---------------------
     n, k, g = 11008, 4096, 128

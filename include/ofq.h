@@ -90,7 +90,11 @@ int ofq_groupwise_dequantize(void* stream, const void* in, const void* scale, co
  *   w_zero NULL iff symmetric, b[n] (t_dtype) or NULL, out[m,n] (t_dtype).
  * out = T( sum_k float(x * w~) + float(b) ), w~ = T(T(q)*scale) + zero as in groupwise_dequantize.
  * Any m is accepted (the reference kernel has no m limit either, :473,590).
- * workspace: ofq_fused_linear_gq_workspace_bytes() bytes, may be NULL when that is 0.
+ * workspace: optional.  ofq_fused_linear_gq_workspace_bytes() is non-zero only for large m on the
+ *   GEMM path (n*k*sizeof(T)): with it the weight is dequantised once into the workspace and a
+ *   copy-fed MFMA GEMM runs on the result (the functor's own m > 8 decomposition); with NULL or
+ *   a smaller buffer the weight tiles are dequantised inside the GEMM instead (same results up to
+ *   fp32 summation order, slower at large m).
  */
 size_t ofq_fused_linear_gq_workspace_bytes(int w_dtype, int t_dtype, int num_bits, int symmetric,
                                            int group_dim, int64_t group_size, int64_t m,

@@ -21,7 +21,38 @@
 #include "ofq_internal.h"
 
 namespace ofq {
+
+// The copy-fed GEMMs are bound by the L2 -> LDS traffic per MFMA, which falls with the tile area,
+// so a 256x352 tile (one per CU, 8 waves side by side along M) beats 256x128 whenever its tiles
+// fill whole rounds of the 256 CUs reasonably well; with a poor fill the idle tail costs more
+// than the traffic saves.
+bool wide_tiles_pay(int64_t m, int64_t n) {
+  const int64_t tiles = ((m + 255) / 256) * ((n + 351) / 352);
+  const int64_t rounds = (tiles + 255) / 256;
+  return tiles * 100 >= rounds * 256 * 80;
+}
+
 namespace {
+
+// x[m,k] * wt[n,k]^T with both operands in T (the dequantised weight of the two-pass path)
+template<typename T, class MF>
+int launch_plain(hipStream_t st, const LinearArgs& a, const void* wt) {
+  typedef typename TT<T>::storage S;
+  typedef EpBias<T> EP;
+  BCopyParams bp;
+  bp.b = static_cast<const uint8_t*>(wt);
+  bp.ldb = a.k * 2;
+  bp.N = (int)a.n;
+  typename EP::Params ep;
+  ep.bias = static_cast<const S*>(a.bias);
+  ep.out = static_cast<S*>(a.out);
+  if (wide_tiles_pay(a.m, a.n)) {
+    return launch_core2<MF, B2Copy<352, 512>, EP, 256, 352, 8, 1>(st, a.x, a.k * 2, bp, ep, a.m,
+                                                                  a.n, a.k / 64);
+  }
+  return launch_core2<MF, B2Copy<128, 512>, EP, 256, 128, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m, a.n,
+                                                                a.k / 64);
+}
 
 template<typename T, class MF, int BITS, bool SIGNED, int ZMODE>
 int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
@@ -73,19 +104,28 @@ bool gemm_wq_supported(const LinearArgs& a) {
   return true;
 }
 
-int launch_gemm_wq(hipStream_t st, const LinearArgs& a) {
-  if (a.t_dtype == OFQ_F16) return launch_wq_t<f16, MfmaF16>(st, a);
-  return launch_wq_t<bf16, MfmaBF16>(st, a);
+// Two passes pay once m is large: the in-tile path converts every weight tile once per 256 rows
+// of x (8 times at m = 2048) and that conversion, not the MFMAs, bounds it; converting the weight
+// once into the workspace and running the copy-fed GEMM on it is what the reference functor does
+// for m > 8 (oneflow/core/functional/impl/quantization.cpp:341-350).
+size_t gemm_wq_workspace_bytes(const LinearArgs& a) {
+  if (!gemm_wq_supported(a) || a.m < 1024) return 0;
+  return (size_t)a.n * (size_t)a.k * 2;
 }
 
-// The int8 GEMM is bound by the L2 -> LDS traffic per MFMA, which falls with the tile area, so a
-// 256x352 tile (one per CU, 8 waves side by side along M) beats 256x128 whenever its tiles fill
-// whole rounds of the 256 CUs reasonably well; with a poor fill the idle tail costs more than the
-// traffic saves.
-bool wide_tiles_pay(int64_t m, int64_t n) {
-  const int64_t tiles = ((m + 255) / 256) * ((n + 351) / 352);
-  const int64_t rounds = (tiles + 255) / 256;
-  return tiles * 100 >= rounds * 256 * 80;
+int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t workspace_bytes) {
+  const size_t need = gemm_wq_workspace_bytes(a);
+  if (need != 0 && workspace != nullptr && workspace_bytes >= need && ofq_aligned16(workspace)) {
+    const int rc = ofq_groupwise_dequantize(st, a.w, a.scale, a.zero, workspace,
+                                            a.w_signed ? OFQ_I8 : OFQ_U8, a.t_dtype, a.bits,
+                                            a.symmetric ? 1 : 0, a.n * (a.k / a.group_size),
+                                            a.group_size, 1);
+    if (rc != OFQ_OK) return rc;
+    if (a.t_dtype == OFQ_F16) return launch_plain<f16, MfmaF16>(st, a, workspace);
+    return launch_plain<bf16, MfmaBF16>(st, a, workspace);
+  }
+  if (a.t_dtype == OFQ_F16) return launch_wq_t<f16, MfmaF16>(st, a);
+  return launch_wq_t<bf16, MfmaBF16>(st, a);
 }
 
 }  // namespace ofq

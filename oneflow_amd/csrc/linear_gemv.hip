@@ -257,9 +257,23 @@ int launch_linear_generic(hipStream_t st, const LinearArgs& a) {
 
 using namespace ofq;
 
-extern "C" size_t ofq_fused_linear_gq_workspace_bytes(int, int, int, int, int, int64_t, int64_t,
-                                                      int64_t, int64_t) {
-  return 0;  // every path keeps its partial sums in registers / LDS
+extern "C" size_t ofq_fused_linear_gq_workspace_bytes(int w_dtype, int t_dtype, int num_bits,
+                                                      int symmetric, int group_dim,
+                                                      int64_t group_size, int64_t m, int64_t n,
+                                                      int64_t k) {
+  if ((num_bits != 4 && num_bits != 8) || group_size <= 0 || m <= 0 || n <= 0 || k <= 0) return 0;
+  LinearArgs a{};
+  a.t_dtype = t_dtype;
+  a.w_signed = w_dtype == OFQ_I8;
+  a.bits = num_bits;
+  a.symmetric = symmetric != 0;
+  a.group_dim = group_dim;
+  a.group_size = group_size;
+  a.m = m;
+  a.n = n;
+  a.k = k;
+  if (gemv_wq_supported(a)) return 0;
+  return gemm_wq_workspace_bytes(a);  // 0 for every path but the two-pass GEMM at large m
 }
 
 extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
@@ -267,8 +281,6 @@ extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
                                    void* out, int w_dtype, int t_dtype, int num_bits,
                                    int symmetric, int group_dim, int64_t group_size, int64_t m,
                                    int64_t n, int64_t k, void* workspace, size_t workspace_bytes) {
-  (void)workspace;
-  (void)workspace_bytes;
   // checks of FusedLinearWithGroupwiseQuantizedWeightKernel::Compute,
   // groupwise_quantization_kernels.cu:773-822
   OFQ_RETURN_IF(num_bits != 4 && num_bits != 8, OFQ_ERR_BAD_ATTR);
@@ -311,6 +323,6 @@ extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
   a.k = k;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (gemv_wq_supported(a)) return launch_gemv_wq(st, a);
-  if (gemm_wq_supported(a)) return launch_gemm_wq(st, a);
+  if (gemm_wq_supported(a)) return launch_gemm_wq(st, a, workspace, workspace_bytes);
   return launch_linear_generic(st, a);
 }

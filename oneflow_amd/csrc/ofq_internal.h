@@ -24,8 +24,12 @@ struct LinearArgs {
 
 // MFMA GEMM with in-tile dequantisation; groups along K.  Returns OFQ_ERR_UNSUPPORTED when the
 // shape does not meet the kernel's tiling constraints (caller falls back).
+// With a workspace of gemm_wq_workspace_bytes() (non-zero for large m only) the weight is
+// dequantised once into it and a copy-fed GEMM runs on the result; without one the in-tile path
+// is used.
 bool gemm_wq_supported(const LinearArgs& a);
-int launch_gemm_wq(hipStream_t st, const LinearArgs& a);
+size_t gemm_wq_workspace_bytes(const LinearArgs& a);
+int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t workspace_bytes);
 
 // Skinny-M (m <= 16) MFMA GEMV that streams the weights once.
 bool gemv_wq_supported(const LinearArgs& a);

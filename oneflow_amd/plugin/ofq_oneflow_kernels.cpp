@@ -155,10 +155,15 @@ class OfqFusedLinearKernel final : public user_op::OpKernel, public user_op::Cud
     if (b != nullptr) { CHECK_EQ(b->shape_view().At(0), n); }
     CHECK_EQ(out->shape_view().At(out->shape_view().NumAxes() - 1), n);
     CHECK_EQ(symmetric, w_zero == nullptr);
+    // tmp_buffer exists when the InferTmpSizeFn below asked for one (large m: the weight is
+    // dequantised once into it and a copy-fed GEMM runs on the result)
+    user_op::Tensor* tmp = ctx->Tensor4ArgNameAndIndex("tmp_buffer", 0);
     CheckOk(ofq_fused_linear_gq(RawStream(ctx), x->dptr(), w->dptr(), w_scale->dptr(),
                                 w_zero ? w_zero->dptr() : nullptr, b ? b->dptr() : nullptr,
                                 out->mut_dptr(), ToOfq(w->data_type()), ToOfq(data_type), num_bits,
-                                symmetric ? 1 : 0, (int)group_dim, group_size, m, n, k, nullptr, 0),
+                                symmetric ? 1 : 0, (int)group_dim, group_size, m, n, k,
+                                tmp ? tmp->mut_dptr() : nullptr,
+                                tmp ? (size_t)tmp->shape_view().elem_cnt() : 0),
             "fused_linear_with_groupwise_quantized_weight");
   }
   bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
@@ -169,6 +174,17 @@ class OfqFusedLinearKernel final : public user_op::OpKernel, public user_op::Cud
       .SetCreateFn<OfqFusedLinearKernel>()                                   \
       .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)       \
                        && (user_op::HobDataType("out", 0) == dtype))         \
+      .SetInferTmpSizeFn([](user_op::InferContext* ctx) -> size_t {          \
+        const ShapeView xs = ctx->InputShape("x", 0);                        \
+        const ShapeView ws = ctx->InputShape("w", 0);                        \
+        const int64_t k = xs.At(xs.NumAxes() - 1);                           \
+        return ofq_fused_linear_gq_workspace_bytes(                          \
+            ToOfq(ctx->InputDType("w", 0)), ToOfq(dtype),                    \
+            ctx->Attr<int32_t>("num_bits"), ctx->Attr<bool>("symmetric"),    \
+            (int)ctx->Attr<int64_t>("group_dim"),                            \
+            ctx->Attr<int64_t>("group_size"), xs.elem_cnt() / k, ws.At(0),   \
+            k);                                                              \
+      })                                                                     \
       .SetPriority(user_op::kKernelPriorityOptimized)
 REGISTER_OFQ_FUSED_LINEAR(DataType::kFloat16);
 REGISTER_OFQ_FUSED_LINEAR(DataType::kBFloat16);
@@ -317,6 +333,27 @@ extern "C" long long ofq_plugin_observer_tmp_bytes(int dtype, const long long* s
   user_op::InferContext ic;
   ic.shapes["in"] = std::vector<int64_t>(shape, shape + rank);
   ic.attrs["per_layer_quantization"].b = per_layer != 0;
+  return (long long)r->infer_tmp_size(&ic);
+}
+
+// tmp_buffer size the fused linear registration asks for (2-D x)
+extern "C" long long ofq_plugin_fused_linear_tmp_bytes(int t_dtype, int w_dtype, long long m,
+                                                       long long n, long long k, int num_bits,
+                                                       int symmetric, long long group_dim,
+                                                       long long group_size) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["out"] = (DataType)t_dtype;
+  const auto* r = Lookup("fused_linear_with_groupwise_quantized_weight", c);
+  if (r == nullptr || !r->infer_tmp_size) return -1;
+  user_op::InferContext ic;
+  ic.shapes["x"] = {m, k};
+  ic.shapes["w"] = {n, k * num_bits / 8};
+  ic.dtypes["w"] = (DataType)w_dtype;
+  ic.attrs["num_bits"].i = num_bits;
+  ic.attrs["symmetric"].b = symmetric != 0;
+  ic.attrs["group_dim"].i = group_dim;
+  ic.attrs["group_size"].i = group_size;
   return (long long)r->infer_tmp_size(&ic);
 }
 

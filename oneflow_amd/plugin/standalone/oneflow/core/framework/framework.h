@@ -135,6 +135,8 @@ class InferContext {
   T Attr(const std::string& name) const;
 };
 template<> inline bool InferContext::Attr<bool>(const std::string& n) const { return attrs.at(n).b; }
+template<> inline int32_t InferContext::Attr<int32_t>(const std::string& n) const { return (int32_t)attrs.at(n).i; }
+template<> inline int64_t InferContext::Attr<int64_t>(const std::string& n) const { return attrs.at(n).i; }
 
 class OpKernelState {};
 class OpKernelCache {};

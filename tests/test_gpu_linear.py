@@ -154,3 +154,39 @@ def test_prefill_ragged_m_and_n(m, num_bits, symmetric, qdt):
         ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
         got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
         H.assert_linear_parity(got, ref, t, f"m={m} {t}")
+
+
+def test_prefill_with_and_without_workspace():
+    """Large m: with the workspace the weight is dequantised once and a copy-fed GEMM runs on it,
+    without it the weight tiles are dequantised inside the GEMM.  Both must meet the contract, and
+    they differ from each other only by fp32 summation order."""
+    import torch
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    m, n, k, g = 1100, 1500, 512, 64
+    rng = np.random.Generator(np.random.PCG64(77))
+    for t, tcode in (("bf16", _lib.BF16), ("f16", _lib.F16)):
+        x = H.as_T(rng.standard_normal((m, k)).astype(np.float32) / 4, t)
+        w = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+        scale = H.as_T(rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float32), t)
+        zero = H.as_T(rng.uniform(-1.4, -1.1, size=(n, k // g)).astype(np.float32), t)
+        b = H.as_T(rng.standard_normal(n).astype(np.float32) / 10, t)
+        xt, wt, st, zt, bt = map(H.to_torch, (x, w, scale, zero, b))
+        need = L.ofq_fused_linear_gq_workspace_bytes(_lib.U8, tcode, 8, 0, 1, g, m, n, k)
+        assert need == n * k * 2
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        outs = []
+        for wptr, wbytes in ((ws.data_ptr(), need), (None, 0), (ws.data_ptr(), need - 16)):
+            out = torch.empty((m, n), dtype=xt.dtype, device="cuda")
+            rc = L.ofq_fused_linear_gq(torch.cuda.current_stream().cuda_stream, xt.data_ptr(),
+                                       wt.data_ptr(), st.data_ptr(), zt.data_ptr(), bt.data_ptr(),
+                                       out.data_ptr(), _lib.U8, tcode, 8, 0, 1, g, m, n, k, wptr, wbytes)
+            assert rc == 0
+            outs.append(H.to_numpy(out))
+        rows = np.array([0, 255, 256, 700, 1023, 1024, 1099])
+        ref = O.fused_linear(x[rows], w, scale, zero, b, 8, False, 1, g)
+        for got in outs:
+            H.assert_linear_parity(got[rows], ref, t, f"workspace paths {t}")
+        # a too-small workspace falls back to the in-tile path: identical to passing none
+        assert np.array_equal(outs[1], outs[2])
+        assert H.rel_l2(O.to_f32(outs[0]), O.to_f32(outs[1])) < 1e-3
