@@ -381,11 +381,15 @@ int launch_core(hipStream_t st, const void* A, int64_t lda, const typename BP::P
 //
 // LDS addressing.  A wave-level global_load_lds writes 64 x 16 bytes to consecutive LDS addresses,
 // i.e. 8 rows of 128 bytes.  Lane l fills slot (row = l/8, position p = l%8) and fetches the
-// global 16-byte piece c = p ^ (row & 7) of its row, so piece c of row r lives at position
-// c ^ (r & 7).  The fragment reads of 8 consecutive rows (same c) then touch 8 different
-// positions: conflict-free without padding.
+// global 16-byte piece c = p ^ key(row) of its row, key(r) = (r >> 1) & 7, so piece c of row r
+// lives at position c ^ key(r).  gfx950's LDS serves 256 bytes per clock: a ds_read_b128 retires
+// 16 lanes at a time and those must fall into 16 different 16-byte bank groups (address bits
+// 4..7 = position + 8 * (row & 1)).  The fragment reads of 16 consecutive rows (same c) see
+// every key twice, once per row parity: conflict-free without padding.  (Keying on row & 7
+// instead costs a two-way conflict on every fragment read: measured, half the LDS cycles.)
 // =================================================================================================
 constexpr int kStageRow = 128;
+__device__ __forceinline__ int swizzle_key(int row) { return (row >> 1) & 7; }
 
 __device__ __forceinline__ void async_copy16(const uint8_t* gsrc, uint8_t* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(
@@ -408,12 +412,12 @@ __device__ __forceinline__ void async_tile(const uint8_t* __restrict__ g, int64_
                                            int lane) {
   static_assert(ROWS % 8 == 0, "tile rows come in groups of 8");
   constexpr int kGroups = ROWS / 8;
-  const int sub = lane >> 3;                 // row within the 8-row group
-  const int piece = (lane & 7) ^ (sub & 7);  // global piece this lane fetches
+  const int sub = lane >> 3;  // row within the 8-row group
 #pragma unroll
   for (int j = 0; j < (kGroups + NWAVES - 1) / NWAVES; ++j) {
     const int grp = j * NWAVES + wave;  // 8-row group of the tile (wave-uniform)
     if (kGroups % NWAVES != 0 && grp >= kGroups) break;
+    const int piece = (lane & 7) ^ swizzle_key(grp * 8 + sub);  // global piece this lane fetches
     int row = row0 + grp * 8 + sub;
     row = row < row_limit ? row : row_limit - 1;
     async_copy16(g + (int64_t)row * ld + (int64_t)kt * kStageRow + piece * 16,
@@ -546,7 +550,7 @@ struct B2Dequant {
       const int row = q / kChunksPerRow;
       const int c = q % kChunksPerRow;
       uint8_t* rowp = lds + row * kStageRow;
-      const int sw = row & 7;
+      const int sw = swizzle_key(row);
       const float sc = TT<T>::load(&r.s[i]);
       float zc = 0.f;
       if (ZMODE == 2) zc = TT<T>::load(&r.z[i]);
@@ -644,9 +648,10 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
   __syncthreads();
 
   // fragment addressing: row = (wave tile row) + i*32 + lane%32, piece c = 2*ks + lane/32 stored
-  // at position c ^ (row & 7); row & 7 == lane & 7 because every tile origin is a multiple of 8
+  // at position c ^ key(row); key(row) depends on the lane only because every tile origin is a
+  // multiple of 16
   const int frag_row = lane & 31;
-  const int x7 = lane & 7;
+  const int x7 = swizzle_key(frag_row);
   const int half = lane >> 5;
   int frag_off[4];
 #pragma unroll
