@@ -381,6 +381,28 @@ def secondary(L, _lib, torch, dev, args):
         out[name] = {"us": round(us, 2), "gbps": round(gb, 1),
                      "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS,
                                   "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+    del wsrc, qo
+
+    # ---- weight quantise + pack: fp16 [11008,4096] -> symmetric int4, g=128 -------------------
+    n, k, g = 11008, 4096, 128
+    reps = 6  # 6 x 90 MB of distinct sources: beyond the caches
+    wsrc = [(torch.randn((n, k), device=dev) * 0.02).to(torch.float16) for _ in range(reps)]
+    qo = torch.empty((n, k // 2), dtype=torch.int8, device=dev)
+    so = torch.empty((n, k // g), dtype=torch.float16, device=dev)
+    it = [0]
+
+    def wq():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_groupwise_quantize(cs(), wsrc[i].data_ptr(), qo.data_ptr(), so.data_ptr(), None,
+                                     _lib.F16, _lib.I8, 4, 1, 1, g, n, k), "groupwise_quantize")
+    us = timeit(wq, iters=24)
+    nbytes = n * k * 2 + n * k // 2 + n * (k // g) * 2
+    gb = nbytes / (us * 1e-6) / 1e9
+    out["weight_quantize_f16_to_int4_11008x4096"] = {
+        "us": round(us, 2), "gbps": round(gb, 1),
+        "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
     return out
 
 

@@ -155,6 +155,23 @@ int ofq_fused_layer_norm_min_max_observer(void* stream, const void* x, const voi
                                           void* workspace, size_t workspace_bytes);
 
 /*
+ * groupwise_quantize: the producer of the weight format of the two ops above.
+ * The reference defines that format only through the helpers of its own test,
+ *   python/oneflow/test/modules/test_groupwise_quantization.py:26-35 (int4 packing) and :46-81
+ *   (`_quantize`),
+ * whose fp32 arithmetic this follows exactly: x[n,k] (t_dtype) -> q[n, k*num_bits/8] (q_dtype
+ * OFQ_U8 | OFQ_I8; asymmetric => OFQ_U8), scale and zero (t_dtype; zero NULL iff symmetric) of
+ * shape [n, k/group_size] (group_dim 1) or [n/group_size, k] (group_dim 0).
+ *   symmetric : scale = absmax/(2^(b-1)-1), q = rint(x/scale + offset), offset = 2^(b-1)-1 for
+ *               OFQ_U8 and 0 for OFQ_I8;  asymmetric: scale = (max-min)/(2^b-1),
+ *               q = rint((x-min)/scale), zero = min.
+ * Codes use the unrounded fp32 scale; a group with scale 0 gets the code of value 0.
+ */
+int ofq_groupwise_quantize(void* stream, const void* x, void* q, void* scale, void* zero,
+                           int t_dtype, int q_dtype, int num_bits, int symmetric, int group_dim,
+                           int64_t group_size, int64_t n, int64_t k);
+
+/*
  * matmul_quant
  * The op is named by the task but absent from the reference tree (only the env-var name
  * ONEFLOW_MLIR_GROUP_MATMUL_QUANT, python/oneflow/framework/infer_compiler/with_fx_graph.py:63);

@@ -275,6 +275,73 @@ static inline float group_zero(const void* zero, int64_t zi, float scale, int bi
   return t_round(-(float)((1 << (bits - 1)) - 1) * scale, t); /* -T(2^(b-1)-1) * scale, in T */
 }
 
+/* Weight quantiser + packer: the `_quantize` / `_pack_int8_to_int4` helpers of the reference's
+ * own test, python/oneflow/test/modules/test_groupwise_quantization.py:26-81, restated.  All
+ * arithmetic is fp32 (`x.float()`), `flow.round` rounds half to even, scale and zero are cast to
+ * T at the end; the codes are computed with the UNROUNDED fp32 scale.
+ *   symmetric : scale = absmax / (2^(b-1)-1);  q = rint(x / scale + offset),
+ *               offset = 2^(b-1)-1 for a uint8 container, 0 for int8
+ *   asymmetric: scale = (max - min) / (2^b - 1); q = rint((x - min) / scale); zero = min
+ * x is [n,k]; groups of `group_size` along axis `group_dim`; 4-bit codes are packed along k,
+ * element 2i in the high nibble.  A group whose scale is 0 (all elements equal / zero) would be
+ * 0/0 in the reference helper; here its codes are defined as `offset` (symmetric) or 0. */
+int ofq_ref_groupwise_quantize(const void* x, void* q, void* scale, void* zero, int t,
+                               int q_is_signed, int bits, int symmetric, int group_dim,
+                               int64_t group_size, int64_t n, int64_t k) {
+  if ((bits != 4 && bits != 8) || (group_dim != 0 && group_dim != 1) || group_size <= 0) return -1;
+  if (!symmetric && (q_is_signed || zero == NULL)) return -1;
+  if (bits == 4 && (k % 2) != 0) return -1;
+  const int64_t dim = group_dim == 0 ? n : k;
+  if (dim % group_size != 0) return -1;
+  const int64_t outer = group_dim == 0 ? 1 : n;
+  const int64_t groups = dim / group_size;
+  const int64_t inner = group_dim == 0 ? k : 1;
+  uint8_t* qb = (uint8_t*)q;
+  const float signed_max = (float)((1 << (bits - 1)) - 1);
+  const float unsigned_max = (float)((1 << bits) - 1);
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t g = 0; g < groups; ++g)
+      for (int64_t i = 0; i < inner; ++i) {
+        float mn = 0.0f, mx = 0.0f, amax = 0.0f;
+        for (int64_t j = 0; j < group_size; ++j) {
+          const float v = t_load(x, ((o * groups + g) * group_size + j) * inner + i, t);
+          if (j == 0 || v < mn) mn = v;
+          if (j == 0 || v > mx) mx = v;
+          if (fabsf(v) > amax) amax = fabsf(v);
+        }
+        const float sc = symmetric ? amax / signed_max : (mx - mn) / unsigned_max;
+        const float offset = symmetric ? (q_is_signed ? 0.0f : signed_max) : 0.0f;
+        t_store(scale, (o * groups + g) * inner + i, sc, t);
+        if (!symmetric) t_store(zero, (o * groups + g) * inner + i, mn, t);
+        for (int64_t j = 0; j < group_size; ++j) {
+          const int64_t idx = ((o * groups + g) * group_size + j) * inner + i;
+          const float v = t_load(x, idx, t);
+          float r;
+          if (sc == 0.0f) {
+            r = offset;
+          } else if (symmetric) {
+            const float d = v / sc;
+            r = nearbyintf(d + offset);
+          } else {
+            const float d = v - mn;
+            r = nearbyintf(d / sc);
+          }
+          const int code = (int)r;
+          if (bits == 8) {
+            qb[idx] = (uint8_t)code;
+          } else {
+            const uint8_t nib = (uint8_t)code & 0xF;
+            if ((idx & 1) == 0) {
+              qb[idx >> 1] = (uint8_t)((qb[idx >> 1] & 0x0F) | (nib << 4));
+            } else {
+              qb[idx >> 1] = (uint8_t)((qb[idx >> 1] & 0xF0) | nib);
+            }
+          }
+        }
+      }
+  return 0;
+}
+
 /* Dequantize3D / DequantizeInnerSize1: groupwise_quantization_kernels.cu:170-203, :275-299;
  * element arithmetic InplaceFma(Scalar) :97-103,123-130: elem * scale + zero, each op in T.
  * View: out[outer][group_size][inner]; scale/zero[outer][inner]; codes packed along the last

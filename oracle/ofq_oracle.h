@@ -40,6 +40,11 @@ int ofq_ref_groupwise_dequantize(const void* in, const void* scale, const void* 
                                  int in_is_signed, int t, int bits, int symmetric, int64_t outer,
                                  int64_t group_size, int64_t inner);
 
+/* weight quantiser + int4 packer of the reference's own test (x is [n,k]) */
+int ofq_ref_groupwise_quantize(const void* x, void* q, void* scale, void* zero, int t,
+                               int q_is_signed, int bits, int symmetric, int group_dim,
+                               int64_t group_size, int64_t n, int64_t k);
+
 int ofq_ref_fused_linear(const void* x, const void* w, const void* scale, const void* zero,
                          const void* bias, void* out, int w_is_signed, int t, int bits,
                          int symmetric, int group_dim, int64_t group_size, int64_t m, int64_t n,

@@ -142,6 +142,25 @@ def fake_quantization(x, scale, zero_point, quantization_formula="google", quant
                   quantization_scheme, zp_mode, 1)
 
 
+def groupwise_quantize(x, num_bits=8, symmetric=True, group_dim=1, group_size=-1, signed=True):
+    """x: 2-D fp32 / fp16 / bf16-bits array.  Returns (codes, scale, zero-or-None)."""
+    x = _c(x)
+    n, k = x.shape
+    dim = x.shape[group_dim]
+    if group_size < 0:
+        group_size = dim
+    q = np.zeros((n, k * num_bits // 8), dtype=np.int8 if signed else np.uint8)
+    sshape = (n // group_size, k) if group_dim == 0 else (n, k // group_size)
+    scale = np.empty(sshape, dtype=x.dtype)
+    zero = None if symmetric else np.empty(sshape, dtype=x.dtype)
+    rc = lib().ofq_ref_groupwise_quantize(
+        _p(x), _p(q), _p(scale), _p(zero), t_code(x), int(bool(signed)), int(num_bits),
+        int(bool(symmetric)), int(group_dim), _i64(group_size), _i64(n), _i64(k))
+    if rc != 0:
+        raise ValueError("oracle groupwise_quantize rejected the arguments")
+    return q, scale, zero
+
+
 def groupwise_dequantize(q, scale, zero=None, num_bits=8, symmetric=True, group_dim=-1,
                          group_size=-1):
     """q: int8/uint8 of any rank, codes packed along the last axis.  Returns an array with the

@@ -325,3 +325,67 @@ def test_matmul_quant_exact_integer_accumulation():
     expect = (acc.astype(np.float32) * (sa[0] * sb)[None, :] + bias.astype(np.float32)).astype(np.float16)
     with np.errstate(over="ignore"):
         assert np.array_equal(out.view(np.uint16), expect.view(np.uint16))
+
+
+# ---- weight quantiser + packer (the reference's test helper, restated) ---------------------------
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("symmetric,signed", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("group_dim,group_size", [(1, 64), (1, 8), (0, 16), (0, 4)])
+@pytest.mark.parametrize("t", ["f32", "f16"])
+def test_weight_quantizer_matches_the_numpy_restatement(bits, symmetric, signed, group_dim,
+                                                        group_size, t):
+    """The C oracle against an independent numpy restatement of the reference test's `_quantize`
+    (helpers.quantize_groupwise follows test_groupwise_quantization.py:46-81 with numpy fp32 ops
+    and np.rint): codes, scales and zeros must be identical bit for bit."""
+    rng = np.random.Generator(np.random.PCG64(bits * 100 + group_dim * 10 + group_size))
+    n, k = 32, 128
+    x = H.as_T(rng.standard_normal((n, k)).astype(np.float32), t)
+    qd = np.int8 if signed else np.uint8
+    w, scale, zero = H.quantize_groupwise(O.to_f32(x), bits, symmetric, group_dim, group_size, qd, t)
+    q2, s2, z2 = O.groupwise_quantize(x, bits, symmetric, group_dim, group_size, signed)
+    assert np.array_equal(w.view(np.uint8), q2.view(np.uint8))
+    assert np.array_equal(scale.view(np.uint8), s2.view(np.uint8))
+    if symmetric:
+        assert zero is None and z2 is None
+    else:
+        assert np.array_equal(O.to_f32(zero), O.to_f32(z2))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_weight_quantizer_closed_forms(bits):
+    """What the arithmetic fixes without any restatement: (1) integers times a power-of-two
+    scale come back as exactly those integers, in the nibble order of the reference packer;
+    (2) the extreme element of every group maps to +-(2^(b-1)-1) (symmetric) and min/max map to
+    0 / 2^b-1 (asymmetric); (3) dequantising the codes lands within half a step of the input;
+    (4) a uint8 container holds the int8 codes plus 2^(b-1)-1."""
+    smax = 2 ** (bits - 1) - 1
+    rng = np.random.Generator(np.random.PCG64(5 + bits))
+    n, k, g = 6, 64, 16
+    ints = rng.integers(-smax, smax + 1, size=(n, k))
+    ints[:, ::g] = smax  # the group maximum pins the scale to exactly 2^-3
+    x = (ints * 0.125).astype(np.float32)
+    q, s, _ = O.groupwise_quantize(x, bits, True, 1, g, True)
+    assert np.all(s == np.float32(0.125))
+    codes = H.unpack_int4(q) if bits == 4 else q
+    assert np.array_equal(codes.astype(np.int64), ints)
+    if bits == 4:  # element 2i is the high nibble of byte i
+        assert np.array_equal((q.view(np.uint8) >> 4).astype(np.int64), ints[:, 0::2] & 0xF)
+        assert np.array_equal((q.view(np.uint8) & 0xF).astype(np.int64), ints[:, 1::2] & 0xF)
+    qu, su, _ = O.groupwise_quantize(x, bits, True, 1, g, False)
+    cu = H.unpack_int4(qu) if bits == 4 else qu
+    assert np.array_equal(cu.astype(np.int64), ints + smax) and np.array_equal(su, s)
+    # random data: extremes and half-step bound
+    y = rng.standard_normal((n, k)).astype(np.float32)
+    q, s, _ = O.groupwise_quantize(y, bits, True, 1, g, True)
+    c = (H.unpack_int4(q) if bits == 4 else q).astype(np.float32).reshape(n, k // g, g)
+    yr = y.reshape(n, k // g, g)
+    assert np.all(np.abs(c).max(axis=2) == smax)
+    assert np.all(np.abs(c * s[:, :, None] - yr) <= 0.5 * s[:, :, None] * (1 + 1e-6))
+    q, s, z = O.groupwise_quantize(y, bits, False, 1, g, False)
+    c = (H.unpack_int4(q) if bits == 4 else q).astype(np.float32).reshape(n, k // g, g)
+    assert np.all(c.min(axis=2) == 0) and np.all(c.max(axis=2) == 2 ** bits - 1)
+    assert np.array_equal(z, yr.min(axis=2))
+    assert np.all(np.abs(c * s[:, :, None] + z[:, :, None] - yr) <= 0.5 * s[:, :, None] * (1 + 1e-5))
+    # a constant group has scale 0: codes are the code of value 0, not NaN-derived garbage
+    zq, zs, _ = O.groupwise_quantize(np.zeros((2, 16), np.float32), bits, True, 1, 16, False)
+    assert np.all(zs == 0) and np.all((H.unpack_int4(zq) if bits == 4 else zq) == smax)
