@@ -119,6 +119,26 @@ int ofq_min_max_observer(void* stream, const void* in, void* scale, void* zero_p
                          int scheme, int formula, void* workspace, size_t workspace_bytes);
 
 /*
+ * moving_average_min_max_observer (per-tensor only)
+ * Replaces GpuMovingAverageMinMaxObserverKernel<T>::Compute,
+ *   oneflow/user/kernels/moving_average_min_max_observer_kernel.cu:217-300
+ * with the arithmetic of the CPU kernel, moving_average_min_max_observer_kernel.cpp:22-107.
+ * in: elem_cnt values (OFQ_F32 | OFQ_F64); current_train_step: one int64 ON THE DEVICE (read by
+ * the kernel: no host synchronisation, unlike the reference's cudaMemcpy at .cu:249-251);
+ * moving_max / moving_min: one value each, updated in place while
+ * `training && *current_train_step <= stop_update_after_iters`; scale / zero_point: one value each.
+ * workspace: ofq_moving_average_min_max_observer_workspace_bytes().
+ */
+size_t ofq_moving_average_min_max_observer_workspace_bytes(int in_dtype, int64_t elem_cnt);
+int ofq_moving_average_min_max_observer(void* stream, const void* in,
+                                        const int64_t* current_train_step, void* moving_max,
+                                        void* moving_min, void* scale, void* zero_point,
+                                        int in_dtype, int64_t elem_cnt, int quantization_bit,
+                                        int scheme, int formula, float momentum,
+                                        int64_t stop_update_after_iters, int training,
+                                        void* workspace, size_t workspace_bytes);
+
+/*
  * quantization / fake_quantization
  * replace GpuQuantizationKernel<T>::Compute, oneflow/user/kernels/quantization_kernel.cu:107-144
  * (arithmetic :24-95) and GpuFakeQuantizationKernel<T>::Compute,

@@ -31,6 +31,9 @@ SIGNATURES = {
                                  _i64, _i64, _i64, _vp, _sz]),
     "ofq_min_max_observer_workspace_bytes": (_sz, [_i, _i64, _i64]),
     "ofq_min_max_observer": (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _i, _i, _vp, _sz]),
+    "ofq_moving_average_min_max_observer_workspace_bytes": (_sz, [_i, _i64]),
+    "ofq_moving_average_min_max_observer": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i,
+                                                 _i, _i, ctypes.c_float, _i64, _i, _vp, _sz]),
     "ofq_quantization": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _i64, _i, _i, _i, _i]),
     "ofq_fake_quantization": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _i, _i, _i]),
     "ofq_fused_layer_norm_min_max_observer_workspace_bytes": (_sz, [_i, _i64, _i64]),

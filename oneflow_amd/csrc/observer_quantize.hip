@@ -115,6 +115,81 @@ observer_finalize(const T* __restrict__ part, int64_t channels, int64_t splits, 
   }
 }
 
+// ---- moving_average_min_max_observer ------------------------------------------------------------
+// oneflow/user/kernels/moving_average_min_max_observer_kernel.cpp:22-107: while
+// current_train_step <= stop_update_after_iters (and training), moving_max / moving_min follow the
+// tensor's extremes (first value, then `moving * momentum + extreme * (1 - momentum)`, each
+// product and the sum rounded separately); scale / zero_point always come from the moving values.
+// The affine zero point rounds half away from zero (std::round, :78), unlike min_max_observer.
+// The step counter is read on the device, so the op can be captured in a graph (the reference's
+// CUDA kernel copies it to the host first, moving_average_min_max_observer_kernel.cu:249-251).
+template<typename T>
+__global__ void __launch_bounds__(kWave)
+moving_average_finalize(const T* __restrict__ part, int64_t splits,
+                        const int64_t* __restrict__ current_train_step,
+                        int64_t stop_update_after_iters, int training, float momentum, int bits,
+                        int scheme, int formula, T* __restrict__ moving_max,
+                        T* __restrict__ moving_min, T* __restrict__ scale,
+                        T* __restrict__ zero_point) {
+  const bool update = training != 0 && *current_train_step <= stop_update_after_iters;
+  T mmax = *moving_max, mmin = *moving_min;
+  if (update) {  // uniform
+    T vmax = part[0], vmin = part[1];
+    for (int64_t s = threadIdx.x; s < splits; s += kWave) {
+      vmax = OpMax()(vmax, part[2 * s]);
+      vmin = OpMin()(vmin, part[2 * s + 1]);
+    }
+    vmax = wave_reduce(vmax, OpMax());
+    vmin = wave_reduce(vmin, OpMin());
+    const T keep = (T)momentum;              // T * float: the float is widened to T
+    const T take = (T)(1 - momentum);        // (1 - momentum) is evaluated in float first
+    if (formula == OFQ_FORMULA_CAMBRICON || scheme == OFQ_SCHEME_SYMMETRIC) {
+      const T a = t_abs(vmax), b = t_abs(vmin);
+      const T amax = a < b ? b : a;
+      if (mmax == 0) {
+        mmax = amax;
+      } else {
+        const T p0 = mmax * keep, p1 = amax * take;
+        mmax = p0 + p1;
+      }
+      mmin = mmax;  // the symmetric schemes only use moving_max
+    } else {
+      if (mmax == 0) {
+        mmax = vmax;
+      } else {
+        const T p0 = mmax * keep, p1 = vmax * take;
+        mmax = p0 + p1;
+      }
+      if (mmin == 0) {
+        mmin = vmin;
+      } else {
+        const T p0 = mmin * keep, p1 = vmin * take;
+        mmin = p0 + p1;
+      }
+    }
+  }
+  if (threadIdx.x != 0) return;
+  if (update) {
+    *moving_max = mmax;
+    *moving_min = mmin;
+  }
+  if (formula == OFQ_FORMULA_CAMBRICON) {
+    const T lg = (T)log2((double)mmax);
+    *scale = floor(lg) - (T)(bits - 2);
+    *zero_point = 0;
+  } else if (scheme == OFQ_SCHEME_SYMMETRIC) {
+    const T denominator = (T)(1 << (bits - 1)) - 1;
+    *scale = mmax / denominator;
+    *zero_point = 0;
+  } else {
+    const T denominator = (T)(1 << bits) - 1;
+    const T sc = (mmax - mmin) / denominator;
+    const T r = mmin / sc;
+    *scale = sc;
+    *zero_point = -(r < 0 ? -floor(-r + (T)0.5) : floor(r + (T)0.5));  // -std::round(r)
+  }
+}
+
 // ---- quantization / fake quantization ---------------------------------------------------
 // IN: element type of `in`; C: type the arithmetic runs in (float for f16/bf16/f32 inputs,
 // double for f64); OUT: storage of the result (same as IN, or int8/uint8 codes).
@@ -353,6 +428,55 @@ extern "C" int ofq_min_max_observer(void* stream, const void* in, void* scale, v
         static_cast<const double*>(in), inner, splits, static_cast<double*>(workspace));
     observer_finalize<double><<<fin_grid, kObsBlock, 0, st>>>(
         static_cast<const double*>(workspace), channels, splits, quantization_bit, scheme, formula,
+        static_cast<double*>(scale), static_cast<double*>(zero_point));
+  }
+  return ofq_check_launch();
+}
+
+extern "C" size_t ofq_moving_average_min_max_observer_workspace_bytes(int in_dtype,
+                                                                      int64_t elem_cnt) {
+  return ofq_min_max_observer_workspace_bytes(in_dtype, elem_cnt, 1);
+}
+
+extern "C" int ofq_moving_average_min_max_observer(
+    void* stream, const void* in, const int64_t* current_train_step, void* moving_max,
+    void* moving_min, void* scale, void* zero_point, int in_dtype, int64_t elem_cnt,
+    int quantization_bit, int scheme, int formula, float momentum,
+    int64_t stop_update_after_iters, int training, void* workspace, size_t workspace_bytes) {
+  // attribute domain: oneflow/user/ops/moving_average_min_max_observer_op.cpp:72-86
+  OFQ_RETURN_IF(quantization_bit <= 1 || quantization_bit > 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(scheme != OFQ_SCHEME_SYMMETRIC && scheme != OFQ_SCHEME_AFFINE, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(formula != OFQ_FORMULA_GOOGLE && formula != OFQ_FORMULA_CAMBRICON,
+                OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(stop_update_after_iters <= 0, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(in_dtype != OFQ_F32 && in_dtype != OFQ_F64, OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(elem_cnt < 1, OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(in == nullptr || current_train_step == nullptr || moving_max == nullptr
+                    || moving_min == nullptr || scale == nullptr || zero_point == nullptr,
+                OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(!ofq_aligned16(in), OFQ_ERR_MISALIGNED);
+  const size_t need = ofq_moving_average_min_max_observer_workspace_bytes(in_dtype, elem_cnt);
+  OFQ_RETURN_IF(workspace == nullptr || workspace_bytes < need, OFQ_ERR_WORKSPACE);
+  const int64_t splits = obs_splits(elem_cnt);
+  OFQ_RETURN_IF(splits > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // The extremes are reduced whether or not this step updates the moving values: whether it does
+  // is known on the device only.
+  if (in_dtype == OFQ_F32) {
+    observer_partial<float><<<(int)splits, kObsBlock, 0, st>>>(
+        static_cast<const float*>(in), elem_cnt, splits, static_cast<float*>(workspace));
+    moving_average_finalize<float><<<1, kWave, 0, st>>>(
+        static_cast<const float*>(workspace), splits, current_train_step, stop_update_after_iters,
+        training, momentum, quantization_bit, scheme, formula, static_cast<float*>(moving_max),
+        static_cast<float*>(moving_min), static_cast<float*>(scale),
+        static_cast<float*>(zero_point));
+  } else {
+    observer_partial<double><<<(int)splits, kObsBlock, 0, st>>>(
+        static_cast<const double*>(in), elem_cnt, splits, static_cast<double*>(workspace));
+    moving_average_finalize<double><<<1, kWave, 0, st>>>(
+        static_cast<const double*>(workspace), splits, current_train_step,
+        stop_update_after_iters, training, momentum, quantization_bit, scheme, formula,
+        static_cast<double*>(moving_max), static_cast<double*>(moving_min),
         static_cast<double*>(scale), static_cast<double*>(zero_point));
   }
   return ofq_check_launch();

@@ -247,6 +247,43 @@ def min_max_observer(in_, quantization_formula="google", quantization_bit=8,
     return scale, zero_point
 
 
+def moving_average_min_max_observer(in_, current_train_step, moving_max, moving_min, training,
+                                    stop_update_after_iters, quantization_formula="google",
+                                    quantization_bit=8, quantization_scheme="symmetric",
+                                    momentum=0.95):
+    """MovingAverageMinMaxObserverFunctor (quantization.cpp:59-91, functional_api.yaml:1079-1084).
+    ``moving_max`` / ``moving_min`` (shape ``[1]``, dtype of ``in``) are updated in place while
+    training and ``current_train_step <= stop_update_after_iters``; ``current_train_step`` is a
+    device tensor of one int64 and is read on the device.  Returns ``(scale, zero_point)``."""
+    _check_quant_attrs(quantization_formula, quantization_bit, quantization_scheme)
+    _check(stop_update_after_iters > 0, "stop_update_after_iters should be greater than 0")
+    _check(in_.dtype in (torch.float32, torch.float64),
+           f"no moving_average_min_max_observer kernel for dtype {in_.dtype}")
+    # shape rules of moving_average_min_max_observer_op.cpp:29-32
+    for name, t in (("moving_max", moving_max), ("moving_min", moving_min),
+                    ("current_train_step", current_train_step)):
+        _check(t.dim() == 1 and t.shape[0] == 1, f"{name} should have shape [1]")
+    _check(moving_max.dtype == in_.dtype and moving_min.dtype == in_.dtype,
+           "moving_max and moving_min should have the dtype of in")
+    _check(current_train_step.dtype == torch.int64, "current_train_step should be int64")
+    _require_gpu(in_, current_train_step, moving_max, moving_min)
+    _check(moving_max.is_contiguous() and moving_min.is_contiguous(),
+           "moving_max and moving_min are updated in place and must be contiguous")
+    in_ = _contig(in_)
+    scale = torch.empty(1, dtype=in_.dtype, device=in_.device)
+    zero_point = torch.empty(1, dtype=in_.dtype, device=in_.device)
+    L = _lib.lib()
+    ws_bytes = L.ofq_moving_average_min_max_observer_workspace_bytes(_dt(in_), in_.numel())
+    ws = _workspace(ws_bytes, in_.device)
+    st = L.ofq_moving_average_min_max_observer(
+        _stream(in_), _ptr(in_), _ptr(current_train_step), _ptr(moving_max), _ptr(moving_min),
+        _ptr(scale), _ptr(zero_point), _dt(in_), in_.numel(), quantization_bit,
+        _lib.SCHEME[quantization_scheme], _lib.FORMULA[quantization_formula], float(momentum),
+        int(stop_update_after_iters), int(bool(training)), _ptr(ws), ws_bytes)
+    _lib.check("ofq_moving_average_min_max_observer", st)
+    return scale, zero_point
+
+
 def _quant_common(fn_name, in_, scale, zero_point, quantization_formula, quantization_bit,
                   quantization_scheme, out_dtype, zp_mode):
     _check_quant_attrs(quantization_formula, quantization_bit, quantization_scheme)

@@ -10,6 +10,7 @@
 //   groupwise_dequantize                          groupwise_quantization_kernels.cu:456-463
 //   fused_linear_with_groupwise_quantized_weight  groupwise_quantization_kernels.cu:844-851
 //   min_max_observer                              min_max_observer_kernel.cu:240-258
+//   moving_average_min_max_observer               moving_average_min_max_observer_kernel.cu:306-314
 //   quantization                                  quantization_kernel.cu:149-156
 //   fake_quantization                             fake_quantization_kernel.cu:150-157
 // bf16 variants are added; kernels carry kKernelPriorityOptimized so that they win over stock
@@ -228,6 +229,48 @@ class OfqMinMaxObserverKernel final : public user_op::OpKernel {
       .SetPriority(user_op::kKernelPriorityOptimized)
 REGISTER_OFQ_OBSERVER(DataType::kFloat);
 REGISTER_OFQ_OBSERVER(DataType::kDouble);
+
+// ---- moving_average_min_max_observer: in, current_train_step, moving_max, moving_min ->
+//      scale, zero_point (+ tmp_buffer); moving_* are updated in place ------------------------
+class OfqMovingAverageMinMaxObserverKernel final : public user_op::OpKernel {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx) const override {
+    const user_op::Tensor* in = ctx->Tensor4ArgNameAndIndex("in", 0);
+    const user_op::Tensor* step = ctx->Tensor4ArgNameAndIndex("current_train_step", 0);
+    user_op::Tensor* moving_max = ctx->Tensor4ArgNameAndIndex("moving_max", 0);
+    user_op::Tensor* moving_min = ctx->Tensor4ArgNameAndIndex("moving_min", 0);
+    user_op::Tensor* scale = ctx->Tensor4ArgNameAndIndex("scale", 0);
+    user_op::Tensor* zero_point = ctx->Tensor4ArgNameAndIndex("zero_point", 0);
+    user_op::Tensor* tmp = ctx->Tensor4ArgNameAndIndex("tmp_buffer", 0);
+    CheckOk(ofq_moving_average_min_max_observer(
+                RawStream(ctx), in->dptr(), static_cast<const int64_t*>(step->dptr()),
+                moving_max->mut_dptr(), moving_min->mut_dptr(), scale->mut_dptr(),
+                zero_point->mut_dptr(), ToOfq(in->data_type()), in->shape_view().elem_cnt(),
+                ctx->Attr<int32_t>("quantization_bit"),
+                Scheme(ctx->Attr<std::string>("quantization_scheme")),
+                Formula(ctx->Attr<std::string>("quantization_formula")),
+                ctx->Attr<float>("momentum"), ctx->Attr<int64_t>("stop_update_after_iters"),
+                ctx->Attr<bool>("training") ? 1 : 0, tmp->mut_dptr(),
+                (size_t)tmp->shape_view().elem_cnt()),
+            "moving_average_min_max_observer");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_MOVING_OBSERVER(dtype)                                                  \
+  REGISTER_USER_KERNEL("moving_average_min_max_observer")                                    \
+      .SetCreateFn<OfqMovingAverageMinMaxObserverKernel>()                                   \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)                       \
+                       && (user_op::HobDataType("in", 0) == dtype))                          \
+      .SetInferTmpSizeFn([](user_op::InferContext* ctx) -> size_t {                          \
+        return ofq_moving_average_min_max_observer_workspace_bytes(                          \
+            dtype == DataType::kDouble ? OFQ_F64 : OFQ_F32,                                  \
+            ctx->InputShape("in", 0).elem_cnt());                                            \
+      })                                                                                     \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_MOVING_OBSERVER(DataType::kFloat);
+REGISTER_OFQ_MOVING_OBSERVER(DataType::kDouble);
 
 // ---- quantization / fake_quantization: in, scale, zero_point -> out ---------------------------
 template<bool kFake>

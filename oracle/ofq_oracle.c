@@ -275,6 +275,66 @@ static inline float group_zero(const void* zero, int64_t zi, float scale, int bi
   return t_round(-(float)((1 << (bits - 1)) - 1) * scale, t); /* -T(2^(b-1)-1) * scale, in T */
 }
 
+/* moving_average_min_max_observer: GenQuantScalePerLayer{Symmetric,Affine,Cambricon},
+ * oneflow/user/kernels/moving_average_min_max_observer_kernel.cpp:22-107.  `T * float` widens
+ * the float; `(1 - momentum)` is a float expression; the affine zero point uses std::round
+ * (half away from zero, :78). */
+#define OFQ_DEFINE_MOVING_AVERAGE(T, SUFFIX, ROUND, FLOOR, LOG2, FABS)                            \
+  int ofq_ref_moving_average_min_max_observer_##SUFFIX(                                            \
+      const T* in, int64_t elem_cnt, int64_t current_train_step, int64_t stop_update_after_iters, \
+      int training, int bits, int scheme, int formula, float momentum, T* moving_max,             \
+      T* moving_min, T* scale, T* zero_point) {                                                   \
+    if (elem_cnt < 1) return -1;                                                                  \
+    if (current_train_step <= stop_update_after_iters && training) {                              \
+      T in_max = in[0], in_min = in[0];                                                           \
+      for (int64_t i = 1; i < elem_cnt; ++i) {                                                    \
+        if (in[i] > in_max) in_max = in[i];                                                       \
+        if (in[i] < in_min) in_min = in[i];                                                       \
+      }                                                                                           \
+      const int symmetric_like = formula == OFQ_REF_FORMULA_CAMBRICON                             \
+                                 || scheme == OFQ_REF_SCHEME_SYMMETRIC;                           \
+      if (symmetric_like) {                                                                       \
+        const T a = FABS(in_max), b = FABS(in_min);                                               \
+        in_max = a < b ? b : a;                                                                   \
+      }                                                                                           \
+      const T mm = *moving_max;                                                                   \
+      if (mm == 0) {                                                                              \
+        *moving_max = in_max;                                                                     \
+      } else {                                                                                    \
+        const T p0 = mm * momentum;                                                               \
+        const T p1 = in_max * (1 - momentum);                                                     \
+        *moving_max = p0 + p1;                                                                    \
+      }                                                                                           \
+      if (symmetric_like) {                                                                       \
+        *moving_min = *moving_max;                                                                \
+      } else {                                                                                    \
+        const T mn = *moving_min;                                                                 \
+        if (mn == 0) {                                                                            \
+          *moving_min = in_min;                                                                   \
+        } else {                                                                                  \
+          const T p0 = mn * momentum;                                                             \
+          const T p1 = in_min * (1 - momentum);                                                   \
+          *moving_min = p0 + p1;                                                                  \
+        }                                                                                         \
+      }                                                                                           \
+    }                                                                                             \
+    if (formula == OFQ_REF_FORMULA_CAMBRICON) {                                                   \
+      *scale = FLOOR(LOG2(*moving_max)) - (T)(bits - 2);                                          \
+      *zero_point = 0;                                                                            \
+    } else if (scheme == OFQ_REF_SCHEME_SYMMETRIC) {                                              \
+      const T denominator = (T)pow(2.0, bits - 1) - 1;                                            \
+      *scale = (*moving_max) / denominator;                                                       \
+      *zero_point = 0;                                                                            \
+    } else {                                                                                      \
+      const T denominator = (T)pow(2.0, bits) - 1;                                                \
+      *scale = ((*moving_max) - (*moving_min)) / denominator;                                     \
+      *zero_point = -ROUND((*moving_min) / (*scale));                                             \
+    }                                                                                             \
+    return 0;                                                                                     \
+  }
+OFQ_DEFINE_MOVING_AVERAGE(float, f32, roundf, floorf, log2f, fabsf)
+OFQ_DEFINE_MOVING_AVERAGE(double, f64, round, floor, log2, fabs)
+
 /* Weight quantiser + packer: the `_quantize` / `_pack_int8_to_int4` helpers of the reference's
  * own test, python/oneflow/test/modules/test_groupwise_quantization.py:26-81, restated.  All
  * arithmetic is fp32 (`x.float()`), `flow.round` rounds half to even, scale and zero are cast to

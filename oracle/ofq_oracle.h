@@ -40,6 +40,16 @@ int ofq_ref_groupwise_dequantize(const void* in, const void* scale, const void* 
                                  int in_is_signed, int t, int bits, int symmetric, int64_t outer,
                                  int64_t group_size, int64_t inner);
 
+/* moving_max / moving_min are updated in place */
+int ofq_ref_moving_average_min_max_observer_f32(
+    const float* in, int64_t elem_cnt, int64_t current_train_step,
+    int64_t stop_update_after_iters, int training, int bits, int scheme, int formula,
+    float momentum, float* moving_max, float* moving_min, float* scale, float* zero_point);
+int ofq_ref_moving_average_min_max_observer_f64(
+    const double* in, int64_t elem_cnt, int64_t current_train_step,
+    int64_t stop_update_after_iters, int training, int bits, int scheme, int formula,
+    float momentum, double* moving_max, double* moving_min, double* scale, double* zero_point);
+
 /* weight quantiser + int4 packer of the reference's own test (x is [n,k]) */
 int ofq_ref_groupwise_quantize(const void* x, void* q, void* scale, void* zero, int t,
                                int q_is_signed, int bits, int symmetric, int group_dim,

@@ -115,6 +115,27 @@ def min_max_observer(x, quantization_formula="google", quantization_bit=8,
     return scale, zp
 
 
+def moving_average_min_max_observer(x, current_train_step, moving_max, moving_min, training,
+                                    stop_update_after_iters, quantization_formula="google",
+                                    quantization_bit=8, quantization_scheme="symmetric",
+                                    momentum=0.95):
+    """moving_max / moving_min: arrays of one element, updated IN PLACE.  Returns (scale, zp)."""
+    x = _c(x)
+    assert x.dtype in (np.float32, np.float64)
+    assert moving_max.dtype == x.dtype and moving_min.dtype == x.dtype
+    scale = np.empty(1, dtype=x.dtype)
+    zp = np.empty(1, dtype=x.dtype)
+    fn = (lib().ofq_ref_moving_average_min_max_observer_f32 if x.dtype == np.float32
+          else lib().ofq_ref_moving_average_min_max_observer_f64)
+    rc = fn(_p(x), _i64(x.size), _i64(int(current_train_step)), _i64(int(stop_update_after_iters)),
+            int(bool(training)), int(quantization_bit), _SCHEME[quantization_scheme],
+            _FORMULA[quantization_formula], ctypes.c_float(momentum), _p(moving_max),
+            _p(moving_min), _p(scale), _p(zp))
+    if rc != 0:
+        raise ValueError("oracle moving_average_min_max_observer rejected the arguments")
+    return scale, zp
+
+
 def _quant(x, scale, zero_point, formula, bit, scheme, zp_mode, fake):
     x = _c(x)
     assert x.dtype in (np.float32, np.float64)

@@ -112,3 +112,55 @@ def test_cambricon_and_all_zero_channel():
     s, z = flow._C.min_max_observer(H.to_torch(xz), "google", 8, "symmetric", False)
     q = H.to_numpy(flow._C.quantization(H.to_torch(xz), s, z, "google", 8, "symmetric"))
     assert np.isnan(q[0]).all() and np.array_equal(q[1], np.full(8, 127.0, np.float32))
+
+
+@pytest.mark.parametrize("scheme", ["symmetric", "affine"])
+@pytest.mark.parametrize("formula", ["google", "cambricon"])
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_moving_average_observer_sequence(scheme, formula, dt):
+    """A training sequence that crosses stop_update_after_iters, then eval mode: moving values,
+    scale and zero point must equal the oracle's after every call (same values bit for bit: the
+    extremes are exact and the scalar arithmetic is the oracle's)."""
+    import torch
+    import oneflow_amd as flow
+    if formula == "cambricon" and scheme == "affine":
+        pytest.skip("cambricon ignores the scheme")
+    rng = np.random.Generator(np.random.PCG64(17))
+    obs = flow.nn.MovingAverageMinMaxObserver(stop_update_after_iters=3, quantization_formula=formula,
+                                              quantization_bit=8, quantization_scheme=scheme,
+                                              momentum=0.9).cuda()
+    rmax, rmin = np.zeros(1, dt), np.zeros(1, dt)
+    for step in range(6):
+        if step == 5:
+            obs.eval()
+        x = (rng.standard_normal((37, 1031)) * (1 + step)).astype(dt)
+        st = torch.tensor([step], dtype=torch.int64, device="cuda")
+        s, z = obs(H.to_torch(x), st)
+        rs, rz = O.moving_average_min_max_observer(x, step, rmax, rmin, step < 5, 3, formula, 8,
+                                                   scheme, 0.9)
+        assert np.array_equal(H.to_numpy(obs.moving_max), rmax), step
+        assert np.array_equal(H.to_numpy(obs.moving_min), rmin), step
+        assert np.array_equal(H.to_numpy(s), rs) and np.array_equal(H.to_numpy(z), rz), step
+    # the values froze after step 3
+    assert np.array_equal(rmax, H.to_numpy(obs.moving_max))
+    obs.reset_running_stats()
+    assert float(obs.moving_max[0]) == 0.0
+
+
+def test_moving_average_observer_large_and_checks():
+    import torch
+    import oneflow_amd as flow
+    x = H.rng_for(9, 0).standard_normal((4096, 4096)).astype(np.float32)
+    mmax = torch.zeros(1, device="cuda")
+    mmin = torch.zeros(1, device="cuda")
+    st = torch.zeros(1, dtype=torch.int64, device="cuda")
+    s, z = flow._C.moving_average_min_max_observer(H.to_torch(x), st, mmax, mmin, True, 1, "google",
+                                                   8, "affine", 0.95)
+    assert float(mmax[0]) == float(x.max()) and float(mmin[0]) == float(x.min())
+    assert np.float32(s.item()) == (x.max() - x.min()) / np.float32(255.0)
+    with pytest.raises(flow.CheckFailedError):
+        flow._C.moving_average_min_max_observer(H.to_torch(x), st, mmax, mmin, True, 0, "google", 8,
+                                                "affine", 0.95)
+    with pytest.raises(flow.CheckFailedError):
+        flow._C.moving_average_min_max_observer(H.to_torch(x), st.to(torch.int32), mmax, mmin, True, 1,
+                                                "google", 8, "affine", 0.95)

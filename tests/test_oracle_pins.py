@@ -389,3 +389,48 @@ def test_weight_quantizer_closed_forms(bits):
     # a constant group has scale 0: codes are the code of value 0, not NaN-derived garbage
     zq, zs, _ = O.groupwise_quantize(np.zeros((2, 16), np.float32), bits, True, 1, 16, False)
     assert np.all(zs == 0) and np.all((H.unpack_int4(zq) if bits == 4 else zq) == smax)
+
+
+# ---- moving_average_min_max_observer -------------------------------------------------------------
+def test_moving_average_observer_closed_forms():
+    """Step by step against numpy fp32 scalar arithmetic written out by hand (products and the sum
+    rounded separately), the freeze rule, the first-value rule, round-half-away for the affine
+    zero point (the per-tensor min_max_observer uses nearbyint instead) and cambricon powers of two."""
+    f = np.float32
+    mom = 0.9
+    mmax, mmin = np.zeros(1, f), np.zeros(1, f)
+    x0 = np.array([0.5, -2.0, 1.0], f)
+    s, z = O.moving_average_min_max_observer(x0, 0, mmax, mmin, True, 2, momentum=mom)
+    assert mmax[0] == f(2.0) and mmin[0] == f(2.0)          # first value: |min| wins, min := max
+    assert s[0] == f(2.0) / f(127.0) and z[0] == 0
+    x1 = np.array([4.0, -1.0], f)
+    s, z = O.moving_average_min_max_observer(x1, 1, mmax, mmin, True, 2, momentum=mom)
+    expect = f(f(2.0) * f(mom)) + f(f(4.0) * f(f(1) - f(mom)))
+    assert mmax[0] == f(expect) and mmin[0] == mmax[0] and s[0] == f(expect) / f(127.0)
+    frozen = mmax.copy()
+    for step, training in ((3, True), (1, False)):          # past the limit / not training: frozen
+        s2, _ = O.moving_average_min_max_observer(np.array([100.0], f), step, mmax, mmin, training,
+                                                  2, momentum=mom)
+        assert mmax[0] == frozen[0] and s2[0] == s[0]
+    # affine: both extremes move, zero point = -round(min/scale) with halves away from zero
+    mmax, mmin = np.zeros(1, f), np.zeros(1, f)
+    xa = np.array([-2.5, 0.0, 252.5], f)                     # scale = 255/255 = 1, min/scale = -2.5
+    s, z = O.moving_average_min_max_observer(xa, 0, mmax, mmin, True, 5, quantization_scheme="affine")
+    assert mmax[0] == f(252.5) and mmin[0] == f(-2.5) and s[0] == 1 and z[0] == 3   # nearbyint would give 2
+    xb = np.array([-4.5, 300.0], f)
+    s, z = O.moving_average_min_max_observer(xb, 1, mmax, mmin, True, 5, quantization_scheme="affine",
+                                             momentum=0.5)
+    assert mmax[0] == f(276.25) and mmin[0] == f(-3.5)
+    assert s[0] == f(279.75) / f(255.0)
+    assert z[0] == -np.round(np.float64(f(-3.5) / s[0]))
+    # cambricon: floor(log2(moving_max)) - (bits - 2)
+    mmax, mmin = np.zeros(1, f), np.zeros(1, f)
+    s, z = O.moving_average_min_max_observer(np.array([-8.0, 3.0], f), 0, mmax, mmin, True, 5,
+                                             quantization_formula="cambricon")
+    assert mmax[0] == 8 and s[0] == 3 - 6 and z[0] == 0
+    # double follows the same rules; momentum is a float attribute widened to double
+    dmax, dmin = np.zeros(1, np.float64), np.zeros(1, np.float64)
+    O.moving_average_min_max_observer(np.array([1.0, -3.0]), 0, dmax, dmin, True, 9, momentum=0.95)
+    O.moving_average_min_max_observer(np.array([5.0, 0.0]), 1, dmax, dmin, True, 9, momentum=0.95)
+    m32 = np.float64(np.float32(0.95))
+    assert dmax[0] == 3.0 * m32 + 5.0 * np.float64(np.float32(1) - np.float32(0.95))

@@ -30,11 +30,15 @@ def test_registrations(plugin):
         assert plugin.ofq_plugin_registration_info(i, name, 128, ctypes.byref(prio), ctypes.byref(tmp)) == 0
         seen.setdefault(name.value.decode(), []).append((prio.value, tmp.value))
     assert set(seen) == {"groupwise_dequantize", "fused_linear_with_groupwise_quantized_weight",
-                         "min_max_observer", "quantization", "fake_quantization"}
+                         "min_max_observer", "moving_average_min_max_observer", "quantization",
+                         "fake_quantization"}
     assert len(seen["groupwise_dequantize"]) == 3 and len(seen["min_max_observer"]) == 2
-    # every kernel outranks a stock registration (priority 0); only the observer needs tmp_buffer
+    assert len(seen["moving_average_min_max_observer"]) == 2
+    # every kernel outranks a stock registration (priority 0); the observers and the fused linear
+    # (dequantised weight at large m) declare a tmp_buffer
     assert all(p == 10 for v in seen.values() for p, _ in v)
-    assert all(t == 1 for _, t in seen["min_max_observer"])
+    assert all(t == 1 for _, t in seen["min_max_observer"] + seen["moving_average_min_max_observer"])
+    assert all(t == 1 for _, t in seen["fused_linear_with_groupwise_quantized_weight"])
     assert all(t == 0 for _, t in seen["quantization"] + seen["groupwise_dequantize"])
     has = plugin.ofq_plugin_has_kernel
     assert has(b"groupwise_dequantize", K_CUDA, b"scale", K_FLOAT16) == 1
