@@ -96,3 +96,34 @@ def test_weight_pipeline_llama_shape(bits, symmetric, signed):
     ref = O.fused_linear(x, q[cols], s[cols], None if z is None else z[cols], None, bits,
                          symmetric, 1, g)
     H.assert_linear_parity(H.to_numpy(out)[:, cols], ref, "f16", "pipeline")
+
+
+@pytest.mark.parametrize("num_bits,symmetric", [(4, True), (8, False)])
+@pytest.mark.parametrize("dtype_name", ["float16", "bfloat16"])
+def test_quantized_linear_module(num_bits, symmetric, dtype_name):
+    """QuantizedLinear.from_float against the float layer (within the quantisation error of the
+    weights), 3-D inputs, decode and prefill batch sizes, and a state_dict round trip."""
+    import torch
+    import oneflow_amd as flow
+    dtype = getattr(torch, dtype_name)
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(1024, 768, bias=True, device="cuda", dtype=dtype)
+    qt = torch.int8 if symmetric else torch.uint8
+    ql = flow.nn.QuantizedLinear.from_float(lin, num_bits=num_bits, symmetric=symmetric,
+                                            group_size=128, quant_type=qt)
+    wd = flow._C.groupwise_dequantize(ql.weight, ql.weight_scale, zero=ql.weight_zero,
+                                      num_bits=num_bits, symmetric=symmetric, group_dim=1,
+                                      group_size=128)
+    for shape in ((1, 1024), (2, 3, 1024), (150, 1024)):
+        x = torch.randn(shape, device="cuda", dtype=dtype)
+        y = ql(x)
+        assert y.shape == shape[:-1] + (768,) and y.dtype == dtype
+        ref = torch.nn.functional.linear(x.float(), wd.float(), lin.bias.float())
+        err = (y.float() - ref).norm() / ref.norm()
+        assert err < (3e-3 if dtype == torch.float16 else 1e-2), float(err)
+        full = torch.nn.functional.linear(x.float(), lin.weight.float(), lin.bias.float())
+        assert (y.float() - full).norm() / full.norm() < (0.2 if num_bits == 4 else 0.02)
+    clone = flow.nn.QuantizedLinear(1024, 768, True, num_bits, symmetric, 128, qt, dtype, "cuda")
+    clone.load_state_dict(ql.state_dict())
+    x = torch.randn((4, 1024), device="cuda", dtype=dtype)
+    assert torch.equal(clone(x), ql(x))
