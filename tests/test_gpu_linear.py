@@ -66,30 +66,37 @@ def test_decode_w4a16_llama_shapes(m, n, k, container):
     got = _run(x, w, scale, None, b, 4, True, 1, 128)
     r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k}")
     # int8 container: w~ = q*s is not rounded to fp16 inside the kernel (~3e-4 from the oracle);
-    # uint8 container: w~ formed exactly as the oracle does, only the sum order differs
+    # uint8 container: w~ = T(T(u*s) + T(-7s)) carries three roundings of magnitude ~7s around a
+    # small value, so it is formed exactly as the oracle does and only the sum order differs
     assert r < (5e-4 if container == np.int8 else 1e-4)
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 5000, 256), (3, 4099, 384), (16, 6000, 128), (2, 40000, 256),
                                    (5, 33000, 128), (8, 4112, 1024)])
-def test_decode_w4a16_row_balanced_shapes(m, n, k):
+@pytest.mark.parametrize("container", [np.int8, np.uint8])
+def test_decode_w4a16_row_balanced_shapes(m, n, k, container):
     """n large enough that a block owns more than one 16-row tile, with row counts per block
     that are not multiples of 16, partial last blocks and more blocks than fit the chip at once."""
     rng = np.random.Generator(np.random.PCG64(n + m))
     x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), "f16")
-    codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    if container == np.int8:
+        codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+        values = codes.astype(np.int64)
+    else:  # offset codes: value = code - 7, all 16 code points used
+        codes = rng.integers(0, 16, size=(n, k)).astype(np.uint8)
+        values = codes.astype(np.int64) - 7
     w = H.pack_int4(codes)
     scale = H.as_T(rng.uniform(1e-3, 1e-2, size=(n, k // 128)).astype(np.float32), "f16")
     b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), "f16")
     ref = O.fused_linear(x, w, scale, None, b, 4, True, 1, 128)
     got = _run(x, w, scale, None, b, 4, True, 1, 128)
     r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k}")
-    assert r < 5e-4
+    assert r < (5e-4 if container == np.int8 else 1e-4)
     # exact integer case through the same path: scales 1, small integer x
     xi = rng.integers(-2, 3, size=(m, k)).astype(np.float16)
     ones = np.ones((n, k // 128), dtype=np.float16)
     got = _run(xi, w, ones, None, None, 4, True, 1, 128)
-    exact = xi.astype(np.int64) @ codes.astype(np.int64).T
+    exact = xi.astype(np.int64) @ values.T
     assert np.abs(exact).max() < 2048
     assert np.array_equal(got.astype(np.int64), exact)
 
