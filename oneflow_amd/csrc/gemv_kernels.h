@@ -484,12 +484,21 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
 // ---------------------------------------------------------------------------------------------
 constexpr int kW4pMaxTiles = 4;
 
-template<int NWAVES, int kW4pDepth = 2>
+// EXACT = false: the unrounded arithmetic above (int8 container, symmetric).
+// EXACT = true : w~ = T(T(code) * s) + z formed with packed fp16 multiply and add exactly as the
+//   reference does, for either container and any zero mode.  It is needed wherever a zero term
+//   is involved: w~ is then a small difference of two values of magnitude ~7s, the reference's
+//   three roundings are relative to those, and leaving them out moves the result by ~1e-3
+//   relative to the dequantize->matmul composition (measured 6e-4 on uniform codes, more on
+//   bell-shaped ones).  x is staged in the k-order of unpack4_pairs, one MFMA per code word.
+template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
+         int ZMODE = kZeroNone>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
-             const f16* __restrict__ scale, const f16* __restrict__ bias,
-             f16* __restrict__ out, int M, int N, int K, int group_size, int cpg_shift,
-             int rows_per_block) {
+             const f16* __restrict__ scale, const f16* __restrict__ zero,
+             const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
+             int group_size, int cpg_shift, int rows_per_block) {
+  static_assert(EXACT || (SIGNED && ZMODE == kZeroNone), "the unrounded path has no zero term");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
   const int nchunks = K >> 7;
@@ -508,13 +517,16 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const bool has_x = r < M;
 
   // LDS: [red ntiles*NWAVES*M*16 f32][scales rows_per_block*G halves, padded to 16 B]
-  //      [corr nchunks*16 f32][64 zero bytes][x records M*nchunks*256 B]
+  //      [zeros, same size (asymmetric only)][corr nchunks*16 f32 (unrounded path only)]
+  //      [64 zero bytes][x records M*nchunks*256 B]
   float* red = reinterpret_cast<float*>(smem);
   const int red_floats = kW4pMaxTiles * NWAVES * M * 16;
+  const int tile_bytes = (rows_per_block * G * 2 + 15) & ~15;
   f16* sl = reinterpret_cast<f16*>(smem + (size_t)red_floats * 4);
+  f16* zl = reinterpret_cast<f16*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
   float* corr_l = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(sl)
-                                           + ((rows_per_block * G * 2 + 15) & ~15));
-  uint8_t* zrec = reinterpret_cast<uint8_t*>(corr_l) + nchunks * 64;
+                                           + (ZMODE == kZeroAsym ? 2 : 1) * tile_bytes);
+  uint8_t* zrec = reinterpret_cast<uint8_t*>(corr_l) + (EXACT ? 0 : nchunks * 64);
   uint8_t* xs = zrec + 64;
 
   // ---- requests that feed LDS go out first ----------------------------------------------------
@@ -534,10 +546,14 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const int tile_halves = rows_blk * G;
   const f16* stile = scale + (int64_t)row0 * G;
   const bool s_aligned = ((reinterpret_cast<uintptr_t>(stile)) & 15u) == 0;
-  u32x4 sreg;
+  const f16* ztile = ZMODE == kZeroAsym ? zero + (int64_t)row0 * G : stile;  // same alignment
+  u32x4 sreg, zreg;
   const int se = tid * 8;
   const bool s_vec = s_aligned && se + 8 <= tile_halves;
-  if (s_vec) sreg = *reinterpret_cast<const u32x4*>(stile + se);
+  if (s_vec) {
+    sreg = *reinterpret_cast<const u32x4*>(stile + se);
+    if (ZMODE == kZeroAsym) zreg = *reinterpret_cast<const u32x4*>(ztile + se);
+  }
   // bias of the output this thread folds at the end: tid = (tile * M + m) * 16 + n
   // (kept as raw bits: widening it here would wait for every load issued so far)
   uint16_t bias_raw = 0;
@@ -595,15 +611,31 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   for (int e = tid; e < red_floats / 4; e += NT) reinterpret_cast<f32x4*>(red)[e] = f32x4{0.f, 0.f, 0.f, 0.f};
   if (s_vec) {
     *reinterpret_cast<u32x4*>(sl + se) = sreg;
+    if (ZMODE == kZeroAsym) *reinterpret_cast<u32x4*>(zl + se) = zreg;
   } else if (se < tile_halves && s_aligned) {
-    for (int j = se; j < tile_halves && j < se + 8; ++j) sl[j] = stile[j];
+    for (int j = se; j < tile_halves && j < se + 8; ++j) {
+      sl[j] = stile[j];
+      if (ZMODE == kZeroAsym) zl[j] = ztile[j];
+    }
   }
-  for (int e = (s_aligned ? NT * 8 : 0) + tid; e < tile_halves; e += NT) sl[e] = stile[e];
+  for (int e = (s_aligned ? NT * 8 : 0) + tid; e < tile_halves; e += NT) {
+    sl[e] = stile[e];
+    if (ZMODE == kZeroAsym) zl[e] = ztile[e];
+  }
   if (tid < 16) reinterpret_cast<uint32_t*>(zrec)[tid] = 0u;
 #pragma unroll
   for (int i = 0; i < kGemvMaxUnits; ++i) {
     if (wave * 64 + i * NT >= nunits) break;
     const int u = tid + i * NT;
+    if (EXACT) {
+      // one record per code word: x in the pair order of unpack4_pairs
+      if (u < nunits) {
+        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32);
+        dst[0] = permute_x4(xu[i][0]);
+        dst[1] = permute_x4(xu[i][1]);
+      }
+      continue;
+    }
     if (u < nunits) {
       u32x4 lo, hi;
       permute_unit(xu[i][0], xu[i][1], lo, hi);
@@ -626,12 +658,14 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const uint8_t* xrec = has_x ? xs + ((size_t)r * nchunks) * 256 + kb * 64 : zrec;
   const int xrec_stride = has_x ? 256 : 0;
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
+  f32x4 total1 = {0.f, 0.f, 0.f, 0.f};  // second accumulator of the exact path
   auto flush = [&](int t) {
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int m = 4 * kb + v;
-      if (m < M) red[((t * NWAVES + wave) * M + m) * 16 + r] = total[v];
+      if (m < M) red[((t * NWAVES + wave) * M + m) * 16 + r] = total[v] + total1[v];
     }
+    total1 = f32x4{0.f, 0.f, 0.f, 0.f};
   };
 
   // one item = the chunk pair `pair` of tile `tile`, codes in slot d
@@ -645,7 +679,37 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
         u32x4 xa[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) xa[t] = xp[t];
-        const float s = (float)slr[cpg_shift >= 0 ? (c >> cpg_shift) : (c * 128 / group_size)];
+        const int grp = cpg_shift >= 0 ? (c >> cpg_shift) : (c * 128 / group_size);
+        if (EXACT) {
+          const f16 sh = slr[grp];
+          f16 zh = (f16)0.0f;
+          if (ZMODE == kZeroAsym) zh = zl[(tile * 16 + r) * G + grp];
+          if (ZMODE == kZeroSymU) zh = (f16)(-7.0f) * sh;
+          const f16x2 s2 = {sh, sh};
+          const f16x2 z2 = {zh, zh};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            f16x2 p[4];
+            unpack4_pairs<SIGNED>(wq[d][u][j], p);
+            u32x4 bop;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              f16x2 v = p[e] * s2;
+              if (ZMODE != kZeroNone) v = v + z2;
+              bop[e] = as_u32(v);
+            }
+            // two accumulators: consecutive MFMAs do not wait for each other
+            if (j & 1) {
+              total1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                  __builtin_bit_cast(f16x8, xa[j]), __builtin_bit_cast(f16x8, bop), total1, 0, 0, 0);
+            } else {
+              total = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                  __builtin_bit_cast(f16x8, xa[j]), __builtin_bit_cast(f16x8, bop), total, 0, 0, 0);
+            }
+          }
+          continue;
+        }
+        const float s = (float)slr[grp];
         f32x4 acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -728,10 +792,12 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   }
 }
 
-inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block) {
+inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,
+                                 bool exact, bool asym) {
   const int G = K / group_size;
-  return (size_t)kW4pMaxTiles * nwaves * M * 16 * 4 + ((rows_per_block * G * 2 + 15) & ~15)
-         + (size_t)(K >> 7) * 64 + 64 + (size_t)M * K * 2;
+  return (size_t)kW4pMaxTiles * nwaves * M * 16 * 4
+         + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15)
+         + (exact ? 0 : (size_t)(K >> 7) * 64) + 64 + (size_t)M * K * 2;
 }
 
 // dynamic LDS bytes of gemv_w4s_f16

@@ -116,10 +116,10 @@ bool w4s_supported(const LinearArgs& a) {
 
 // Row-balanced kernel: grid = a whole number of blocks per CU (or one 16-row tile per block when
 // n is small), rows_per_block <= 64.
-template<int NW>
+template<int NW, bool EXACT, bool SIGNED, int ZMODE>
 int launch_w4p_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block, size_t lds,
                     int cpg_shift) {
-  auto kern = gemv_w4p_f16<NW, 1>;
+  auto kern = gemv_w4p_f16<NW, 1, EXACT, SIGNED, ZMODE>;
   static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be allowed once
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -131,30 +131,53 @@ int launch_w4p_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_
   }
   kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
                                   static_cast<const f16*>(a.scale),
+                                  static_cast<const f16*>(a.zero),
                                   static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
                                   (int)a.m, (int)a.n, (int)a.k, (int)a.group_size, cpg_shift,
                                   rows_per_block);
   return ofq_check_launch();
 }
 
+// 4-bit codes, fp16, groups along K in multiples of 128: what the row-balanced kernel takes
+bool w4p_supported(const LinearArgs& a) {
+  return a.t_dtype == OFQ_F16 && a.bits == 4 && a.group_dim == 1 && a.m >= 1 && a.m <= 16
+         && a.k % 128 == 0 && a.group_size % 128 == 0 && a.k <= (1 << 20)
+         && a.n <= 0x7FFFFFFF - 16 && (a.symmetric || !a.w_signed);
+}
+
 // OFQ_ERR_UNSUPPORTED when the shape does not fit the row-balanced kernel
 int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift) {
   constexpr int kCUs = 256;
   const int64_t max_rows = 16 * kW4pMaxTiles;
-  // one block per CU when that keeps a block within 64 rows, else two, else as many 64-row
-  // blocks as it takes
+  // one block per CU when that keeps a block within 64 rows (a single 16-row tile per block
+  // when n is small), else two, else as many 64-row blocks as it takes
   int64_t grid = kCUs;
   if ((a.n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
   if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
-  const int rpb = (int)((a.n + grid - 1) / grid);
+  int rpb = (int)((a.n + grid - 1) / grid);
+  if (rpb < 16) rpb = 16;
   grid = (a.n + rpb - 1) / rpb;
   const bool two_per_cu = grid > kCUs;
   const int nw = two_per_cu ? 8 : 16;
   if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
-  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb);
+  const bool exact = !(a.symmetric && a.w_signed);
+  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                                        !a.symmetric);
   if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
-  return two_per_cu ? launch_w4p_inst<8>(st, a, (int)grid, rpb, lds, cpg_shift)
-                    : launch_w4p_inst<16>(st, a, (int)grid, rpb, lds, cpg_shift);
+#define OFQ_W4P(NWV)                                                                         \
+  if (nw == NWV) {                                                                           \
+    if (!exact)                                                                              \
+      return launch_w4p_inst<NWV, false, true, kZeroNone>(st, a, (int)grid, rpb, lds,        \
+                                                          cpg_shift);                        \
+    if (a.symmetric)                                                                         \
+      return launch_w4p_inst<NWV, true, false, kZeroSymU>(st, a, (int)grid, rpb, lds,        \
+                                                          cpg_shift);                        \
+    return launch_w4p_inst<NWV, true, false, kZeroAsym>(st, a, (int)grid, rpb, lds,          \
+                                                        cpg_shift);                          \
+  }
+  OFQ_W4P(16) OFQ_W4P(8)
+#undef OFQ_W4P
+  return OFQ_ERR_UNSUPPORTED;
 }
 
 int launch_w4s(hipStream_t st, const LinearArgs& a) {
@@ -228,6 +251,10 @@ bool gemv_wq_supported(const LinearArgs& a) {
 int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
   if (w4s_supported(a)) {
     const int rc = launch_w4s(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  } else if (w4p_supported(a)) {
+    // uint8 container / asymmetric: the row-balanced kernel with the reference's roundings
+    const int rc = launch_w4p(st, a, ilog2_exact(a.group_size / 128));
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
   }
   const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
