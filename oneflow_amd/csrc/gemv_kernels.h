@@ -215,15 +215,14 @@ __device__ __forceinline__ void permute_unit(const u32x4 a, const u32x4 b, u32x4
   for (int i = 0; i < 4; ++i) hi[i] = as_u32(as_h2(hi[i]) * sixteenth);
 }
 
-// 1032 * (sum of the low-nibble x) + 72 * (sum of the high-nibble x) of one permuted unit;
-// v_dot2_f32_f16 against (1, 1) adds two halves into an fp32 sum per instruction
+// 1032 * (sum of the low-nibble x) + 72 * (sum of the high-nibble x) of one permuted unit
 __device__ __forceinline__ float unit_corr(const u32x4 lo, const u32x4 hi) {
-  const f16x2 ones = {(f16)1.0f, (f16)1.0f};
   float sl = 0.f, sh = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    sl = __builtin_amdgcn_fdot2(as_h2(lo[i]), ones, sl, false);
-    sh = __builtin_amdgcn_fdot2(as_h2(hi[i]), ones, sh, false);
+    const f16x2 l = as_h2(lo[i]), h = as_h2(hi[i]);
+    sl += (float)l[0] + (float)l[1];
+    sh += (float)h[0] + (float)h[1];
   }
   return 1032.0f * sl + 1152.0f * sh;  // hi carries x/16: 72 * 16 = 1152
 }

@@ -129,12 +129,27 @@ __device__ __forceinline__ RawPack<T> load_raw(const typename TT<T>::storage* p)
   for (int i = 0; i < (int)(sizeof(r.q) / 16); ++i) r.q[i] = reinterpret_cast<const u32x4*>(p)[i];
   return r;
 }
+// (whole-vector bit casts: element access through the struct member, `r.q[0][w]`, came out of the
+// compiler as component 0 for every w)
 template<typename T>
 __device__ __forceinline__ void widen(const RawPack<T>& r, float* f) {
-  typedef typename TT<T>::storage S;
-  const S* e = reinterpret_cast<const S*>(r.q);
+  if constexpr (TT<T>::dtype == OFQ_F16) {
+    const f16x8 h = __builtin_bit_cast(f16x8, r.q[0]);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) f[i] = TT<T>::load(&e[i]);
+    for (int i = 0; i < 8; ++i) f[i] = (float)h[i];
+  } else if constexpr (TT<T>::dtype == OFQ_BF16) {
+    const u16x8 h = __builtin_bit_cast(u16x8, r.q[0]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = bf16_to_float(h[i]);
+  } else {
+    const f32x4 lo = __builtin_bit_cast(f32x4, r.q[0]);
+    const f32x4 hi = __builtin_bit_cast(f32x4, r.q[sizeof(r.q) / 16 - 1]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[i] = lo[i];
+      f[4 + i] = hi[i];
+    }
+  }
 }
 
 // One wave per row; NP = packs of 8 elements each lane caches: cols <= 64 * 8 * NP and 8 | cols.
@@ -181,6 +196,8 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
     for (int i = 0; i < NP; ++i) {
       const int p = lane + i * kWave;
       if (p < npacks) {
+        // (plain widen-and-add: a chain of v_dot2_f32_f16 on one accumulator came out of the
+        // compiler with the same source register in every link)
         float f[8];
         widen<T>(v[i], f);
 #pragma unroll
@@ -206,24 +223,43 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
     m2 = wave_reduce(m2, OpSum());
     const float var = fmaxf(m2 / (float)cols, 0.0f);
     const float inv = 1.0f / __builtin_sqrtf(var + eps);
+    f16x8 amax8 = {(f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f};
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
       const int p = lane + i * kWave;
       if (p < npacks) {
-        float f[8], g[8], b[8], o[8];
-        widen<T>(v[i], f);
-        if (gamma) widen<T>(gr[i], g);
-        if (beta) widen<T>(br[i], b);
+        if constexpr (TT<T>::dtype == OFQ_F16) {
+          // the affine in T is native packed fp16 arithmetic: one rounding per multiply and per
+          // add, which is what rounding the fp32 result of each step to fp16 gives as well
+          float f[8];
+          widen<T>(v[i], f);
+          f16x8 t;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float t = TT<T>::round((f[e] - mean) * inv);
-          if (gamma) t = TT<T>::round(t * g[e]);
-          if (beta) t = TT<T>::round(t + b[e]);
-          o[e] = t;
-          amax = fmaxf(amax, fabsf(t));
+          for (int e = 0; e < 8; ++e) t[e] = (f16)((f[e] - mean) * inv);
+          if (gamma) t = t * __builtin_bit_cast(f16x8, gr[i].q[0]);
+          if (beta) t = t + __builtin_bit_cast(f16x8, br[i].q[0]);
+          amax8 = __builtin_elementwise_max(amax8, __builtin_elementwise_abs(t));
+          *reinterpret_cast<u32x4*>(yr + (int64_t)p * 8) = __builtin_bit_cast(u32x4, t);
+        } else {
+          float f[8], g[8], b[8], o[8];
+          widen<T>(v[i], f);
+          if (gamma) widen<T>(gr[i], g);
+          if (beta) widen<T>(br[i], b);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float t = TT<T>::round((f[e] - mean) * inv);
+            if (gamma) t = TT<T>::round(t * g[e]);
+            if (beta) t = TT<T>::round(t + b[e]);
+            o[e] = t;
+            amax = fmaxf(amax, fabsf(t));
+          }
+          store8<T>(yr + (int64_t)p * 8, o);
         }
-        store8<T>(yr + (int64_t)p * 8, o);
       }
+    }
+    if constexpr (TT<T>::dtype == OFQ_F16) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) amax = fmaxf(amax, (float)amax8[e]);
     }
   }
   amax = wave_reduce(amax, OpMax());

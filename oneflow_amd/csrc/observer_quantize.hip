@@ -18,7 +18,7 @@ namespace ofq {
 namespace {
 
 constexpr int kObsBlock = 256;
-constexpr int64_t kObsSliceElems = 16384;  // elements one block reduces
+constexpr int64_t kObsSliceElems = 4096;  // elements one block reduces: 4 x 16 bytes per thread (fp32)
 
 __host__ __device__ inline int64_t obs_splits(int64_t inner) {
   int64_t s = (inner + kObsSliceElems - 1) / kObsSliceElems;
@@ -44,12 +44,24 @@ observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, T* __r
     const int64_t nvec = (end - begin) / V;
     typedef T vec_t __attribute__((ext_vector_type(V)));
     const vec_t* pv = reinterpret_cast<const vec_t*>(p + begin);
-    for (int64_t v = threadIdx.x; v < nvec; v += kObsBlock) {
-      const vec_t x = pv[v];
+    // all of a thread's loads are requested before the first is used (many blocks with a few
+    // 128-bit loads per thread stream better than few blocks with long loops)
+    constexpr int kMaxLoads = (int)(kObsSliceElems / V / kObsBlock);
+    vec_t x[kMaxLoads];
+    bool have[kMaxLoads];
+#pragma unroll
+    for (int i = 0; i < kMaxLoads; ++i) {
+      const int64_t v = threadIdx.x + (int64_t)i * kObsBlock;
+      have[i] = v < nvec;
+      if (have[i]) x[i] = __builtin_nontemporal_load(pv + v);
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxLoads; ++i) {
+      if (!have[i]) continue;
 #pragma unroll
       for (int e = 0; e < V; ++e) {
-        vmax = OpMax()(vmax, x[e]);
-        vmin = OpMin()(vmin, x[e]);
+        vmax = OpMax()(vmax, x[i][e]);
+        vmin = OpMin()(vmin, x[i][e]);
       }
     }
     i = begin + nvec * V;
@@ -267,7 +279,10 @@ __device__ __forceinline__ C effective_zp(C zp) {
   return zp;
 }
 
-// Each lane owns V consecutive elements (V*sizeof(IN) == 16 bytes when the panel allows it).
+// Each lane owns V consecutive elements: 16 bytes of input per load, two loads when the output
+// is one byte wide so that the store is 16 bytes too.  The channel of a pack costs a division
+// (V | panel, so the whole pack lies in one channel); it is skipped for a per-tensor scale and
+// done in 32 bits when the tensor allows it.
 template<typename IN, typename C, typename OUT, int MODE, bool FAKE, int V>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
@@ -275,19 +290,29 @@ quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
                 int64_t panel, int64_t scale_size, C upper, C lower, int cambricon) {
   const int64_t n_packs = elem_cnt / V;
   const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  const bool per_tensor = scale_size == 1;
+  const bool small = elem_cnt < 0x7FFFFFFF;
+  C s0 = scale[0];
+  if (cambricon) s0 = (C)exp2((double)(int)s0);  // scale = 2^int(shift)
+  const C zp0 = MODE == kModeSym ? (C)0 : effective_zp<C, MODE>(zero_point[0]);
   for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < n_packs; p += step) {
     const int64_t base = p * V;
-    int64_t ch = base / panel;  // V | panel, so the whole pack lies in one channel
-    if (ch > scale_size - 1) ch = scale_size - 1;
-    C s = scale[ch];
-    if (cambricon) s = (C)exp2((double)(int)s);  // scale = 2^int(shift)
-    const C zp = MODE == kModeSym ? (C)0 : effective_zp<C, MODE>(zero_point[ch]);
+    C s = s0, zp = zp0;
+    if (!per_tensor) {
+      int64_t ch = small ? (int64_t)((uint32_t)base / (uint32_t)panel) : base / panel;
+      if (ch > scale_size - 1) ch = scale_size - 1;
+      s = scale[ch];
+      if (cambricon) s = (C)exp2((double)(int)s);
+      zp = MODE == kModeSym ? (C)0 : effective_zp<C, MODE>(zero_point[ch]);
+    }
     IN xin[V];
-    if (V * sizeof(IN) == 16) {
-      *reinterpret_cast<u32x4*>(xin) = *reinterpret_cast<const u32x4*>(in + base);
-    } else if (V * sizeof(IN) == 32) {
-      reinterpret_cast<u32x4*>(xin)[0] = reinterpret_cast<const u32x4*>(in + base)[0];
-      reinterpret_cast<u32x4*>(xin)[1] = reinterpret_cast<const u32x4*>(in + base)[1];
+    constexpr int kInBytes = V * (int)sizeof(IN);
+    if (kInBytes % 16 == 0) {
+#pragma unroll
+      for (int i = 0; i < kInBytes / 16; ++i) {
+        reinterpret_cast<u32x4*>(xin)[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4*>(in + base) + i);
+      }
     } else {
 #pragma unroll
       for (int e = 0; e < V; ++e) xin[e] = in[base + e];
@@ -298,14 +323,16 @@ quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
       const C x = (C)Elem<IN>::ld(&xin[e]);
       Elem<OUT>::st(&r[e], quant_one<C, MODE, FAKE>(x, s, zp, upper, lower));
     }
-    if (V * sizeof(OUT) == 16) {
-      *reinterpret_cast<u32x4*>(out + base) = *reinterpret_cast<const u32x4*>(r);
-    } else if (V * sizeof(OUT) == 32) {
-      reinterpret_cast<u32x4*>(out + base)[0] = reinterpret_cast<const u32x4*>(r)[0];
-      reinterpret_cast<u32x4*>(out + base)[1] = reinterpret_cast<const u32x4*>(r)[1];
-    } else if (V * sizeof(OUT) == 8) {
+    constexpr int kOutBytes = V * (int)sizeof(OUT);
+    if (kOutBytes % 16 == 0) {
+#pragma unroll
+      for (int i = 0; i < kOutBytes / 16; ++i) {
+        __builtin_nontemporal_store(reinterpret_cast<const u32x4*>(r)[i],
+                                    reinterpret_cast<u32x4*>(out + base) + i);
+      }
+    } else if (kOutBytes == 8) {
       *reinterpret_cast<u32x2*>(out + base) = *reinterpret_cast<const u32x2*>(r);
-    } else if (V * sizeof(OUT) == 4) {
+    } else if (kOutBytes == 4) {
       *reinterpret_cast<uint32_t*>(out + base) = *reinterpret_cast<const uint32_t*>(r);
     } else {
 #pragma unroll
@@ -326,7 +353,9 @@ template<typename IN, typename C, typename OUT, int MODE, bool FAKE>
 int launch_quant(hipStream_t st, const void* in, const void* scale, const void* zp, void* out,
                  int64_t elem_cnt, int64_t panel, int64_t scale_size, C upper, C lower,
                  int cambricon) {
-  constexpr int V = 16 / sizeof(IN);  // 4 floats, 2 doubles, 8 halves
+  // 16 bytes of input per lane (4 floats, 2 doubles, 8 halves); 32 when the output is bytes and
+  // the input halves, so that loads and the store are all 128-bit
+  constexpr int V = (sizeof(OUT) == 1 && sizeof(IN) == 2) ? 16 : 16 / (int)sizeof(IN);
   const IN* i = static_cast<const IN*>(in);
   OUT* o = static_cast<OUT*>(out);
   const C* s = static_cast<const C*>(scale);
