@@ -341,8 +341,9 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
   // fp32 rows beyond 2048 elements would not fit a lane's registers at two waves per SIMD
   const int64_t wave_packs = (sizeof(S) == 4 ? 4 : 8) * kWave;
   if (vec_ok && npacks <= wave_packs) {
-    // every wave resident at once (8 per CU) when there are that many rows
-    const int64_t waves = rows < 256 * 8 ? rows : 256 * 8;
+    // four waves per CU: 32 KB of rows in flight per CU streams best; with more rows than
+    // waves a wave walks several rows and the waves of a CU drift apart
+    const int64_t waves = rows < 256 * 4 ? rows : 256 * 4;
     const int grid = (int)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
     nparts = (int64_t)grid * kWavesPerBlock < rows ? (int64_t)grid * kWavesPerBlock : rows;
 #define OFQ_LN_WAVE(NPV)                                                                  \
