@@ -1,21 +1,15 @@
 // MFMA GEMMs for gfx950:
-//   (1) fused_linear_with_groupwise_quantized_weight for m > 16 ("prefill"): the weight tile is
-//       dequantised on its way into LDS and feeds fp16/bf16 MFMA, so the fp16/bf16 copy of the
-//       weight that the reference materialises for m > 8
-//       (oneflow/core/functional/impl/quantization.cpp:341-350) never touches HBM;
+//   (1) fused_linear_with_groupwise_quantized_weight for m > 16: either the weight tile is
+//       dequantised on its way into LDS and feeds fp16/bf16 MFMA (the fp16/bf16 copy of the
+//       weight that the reference materialises for m > 8,
+//       oneflow/core/functional/impl/quantization.cpp:341-350, then never touches HBM), or, at
+//       large m with a workspace, the weight is dequantised once and a copy-fed GEMM runs on it;
 //   (2) matmul_quant: int8 x int8 -> int32 MFMA with a per-row/per-tensor scale epilogue.
 //
-// Both are instances of one byte-oriented core.  A tile row is always 128 bytes of K
-// (64 fp16/bf16 or 128 int8 elements), a k-step of the 32x32 MFMA consumes 32 of those bytes per
-// row (16 bytes per lane), so the same LDS layout and fragment addressing serve every type.
-//
-//   block tile BM x BN, WM x WN waves, each wave owns (BM/WM) x (BN/WN) as 32x32 MFMA tiles;
-//   LDS rows are padded from 128 to 144 bytes: the 16-byte fragment reads of 8 consecutive rows
-//   then fall in 8 distinct 16-byte bank groups;
-//   global -> register loads of tile kt+1 are issued before the MFMAs of tile kt, and LDS is
-//   double buffered, so one barrier per k-tile suffices;
-//   block ids are remapped so that the m-tiles sharing one weight tile run on the same XCD and
-//   hit its L2.
+// All are instances of one byte-oriented core (gemm_kernels.h).  A tile row is always 128 bytes
+// of K (64 fp16/bf16 or 128 int8 elements), a k-step of the 32x32 MFMA consumes 32 of those bytes
+// per row (16 bytes per lane), so the same LDS layout and fragment addressing serve every type.
+// This file only picks tile shapes and fills parameter blocks.
 #include "gemm_kernels.h"
 #include "ofq_device.h"
 #include "ofq_internal.h"
@@ -58,7 +52,7 @@ template<typename T, class MF, int BITS, bool SIGNED, int ZMODE>
 int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
   typedef typename TT<T>::storage S;
   typedef EpBias<T> EP;
-  typename BDequant<T, BITS, SIGNED, ZMODE, 128>::Params bp;
+  WqParams<T> bp;
   bp.w = static_cast<const uint8_t*>(a.w);
   bp.scale = static_cast<const S*>(a.scale);
   bp.zero = static_cast<const S*>(a.zero);
@@ -72,6 +66,13 @@ int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
   // 256x128 tiles on 8 waves when there are enough rows of x to fill them, else 128x128 on 4
   if (a.m > 128) {
     return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 512>, EP, 256, 128, 4, 2>(
+        st, a.x, a.k * 2, bp, ep, a.m, a.n, a.k / 64);
+  }
+  // few rows of x: 128-wide weight tiles would leave most CUs without a block (86 tiles for
+  // n = 11008), so the weight tile shrinks until the grid covers the chip
+  const int64_t n_tiles128 = (a.n + 127) / 128;
+  if (n_tiles128 < 192) {
+    return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 32, 256>, EP, 128, 32, 4, 1>(
         st, a.x, a.k * 2, bp, ep, a.m, a.n, a.k / 64);
   }
   return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 256>, EP, 128, 128, 2, 2>(
@@ -148,7 +149,7 @@ extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, cons
                 OFQ_ERR_NULL_POINTER);
   OFQ_RETURN_IF(!ofq_aligned16(a) || !ofq_aligned16(b) || !ofq_aligned16(out), OFQ_ERR_MISALIGNED);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  BCopy<128>::Params bp;
+  BCopyParams bp;
   bp.b = static_cast<const uint8_t*>(b);
   bp.ldb = k;
   bp.N = (int)n;
