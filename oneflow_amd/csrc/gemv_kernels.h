@@ -339,7 +339,9 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
         u32x4 lo, hi;
         permute_unit(xu[i][0], xu[i][1], lo, hi);
         // unit u = (m, chunk, j): j -> kb = j/2, t = 2*(j%2) + {0: lo, 1: hi}; 32 bytes per unit
-        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32);
+        // rows of x are skewed by 16 bytes each: the lanes of different m that read the same
+        // chunk then hit different LDS bank groups (their records are a multiple of 256 B apart)
+        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32 + ((u >> 3) / nchunks) * 16);
         dst[0] = lo;
         dst[1] = hi;
       }
@@ -357,7 +359,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   }
   __syncthreads();
 
-  const uint8_t* xrec = has_x ? xs + ((size_t)r * nchunks) * 256 + kb * 64 : zrec;
+  const uint8_t* xrec = has_x ? xs + (size_t)r * (nchunks * 256 + 16) + kb * 64 : zrec;
   const int xrec_stride = has_x ? 256 : 0;
   const f16* xrow = x + (int64_t)(has_x ? r : 0) * K + kb * 32;
   const f16* slr = sl + r * G;
@@ -629,7 +631,9 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
     if (EXACT) {
       // one record per code word: x in the pair order of unpack4_pairs
       if (u < nunits) {
-        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32);
+        // rows of x are skewed by 16 bytes each: the lanes of different m that read the same
+        // chunk then hit different LDS bank groups (their records are a multiple of 256 B apart)
+        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32 + ((u >> 3) / nchunks) * 16);
         dst[0] = permute_x4(xu[i][0]);
         dst[1] = permute_x4(xu[i][1]);
       }
@@ -638,7 +642,7 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
     if (u < nunits) {
       u32x4 lo, hi;
       permute_unit(xu[i][0], xu[i][1], lo, hi);
-      u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32);
+      u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32 + ((u >> 3) / nchunks) * 16);
       dst[0] = lo;
       dst[1] = hi;
     }
@@ -654,7 +658,7 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   }
   __syncthreads();
 
-  const uint8_t* xrec = has_x ? xs + ((size_t)r * nchunks) * 256 + kb * 64 : zrec;
+  const uint8_t* xrec = has_x ? xs + (size_t)r * (nchunks * 256 + 16) + kb * 64 : zrec;
   const int xrec_stride = has_x ? 256 : 0;
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
   f32x4 total1 = {0.f, 0.f, 0.f, 0.f};  // second accumulator of the exact path
@@ -796,14 +800,14 @@ inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int r
   const int G = K / group_size;
   return (size_t)kW4pMaxTiles * nwaves * M * 16 * 4
          + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15)
-         + (exact ? 0 : (size_t)(K >> 7) * 64) + 64 + (size_t)M * K * 2;
+         + (exact ? 0 : (size_t)(K >> 7) * 64) + 64 + (size_t)M * (K * 2 + 16);
 }
 
 // dynamic LDS bytes of gemv_w4s_f16
 inline size_t gemv_w4s_lds_bytes(int nwaves, bool staged, int M, int K, int group_size) {
   const int G = K / group_size;
   return (size_t)nwaves * 64 * 16 + ((16 * G * 2 + 15) & ~15) + 64
-         + (staged ? (size_t)(K >> 7) * 64 + (size_t)M * K * 2 : 0);
+         + (staged ? (size_t)(K >> 7) * 64 + (size_t)M * (K * 2 + 16) : 0);
 }
 
 }  // namespace
