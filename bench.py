@@ -94,23 +94,23 @@ def main():
                 w = torch.randint(-128, 128, (n, k // 2), dtype=torch.int8, device=dev)
                 scale = torch.empty((n, k // 128), dtype=torch.float16, device=dev).uniform_(1e-3, 1e-2)
                 bias = (torch.randn(n, device=dev) * 0.01).to(torch.float16)
-                out = torch.empty((M, n), dtype=torch.float16, device=dev)
+                out = torch.empty((max(M, 8), n), dtype=torch.float16, device=dev)
                 mats.append((name, n, k, w, scale, bias, out))
         layers.append(mats)
-    x_by_k = {k: torch.randn((M, k), device=dev).to(torch.float16) for k in (4096, 11008)}
+    x_by_k = {k: torch.randn((max(M, 8), k), device=dev).to(torch.float16) for k in (4096, 11008)}
 
-    def launch(mat):
+    def launch(mat, m=M):
         name, n, k, w, scale, bias, out = mat
         st = L.ofq_fused_linear_gq(torch.cuda.current_stream().cuda_stream, x_by_k[k].data_ptr(),
                                    w.data_ptr(), scale.data_ptr(), None, bias.data_ptr(),
-                                   out.data_ptr(), _lib.I8, _lib.F16, 4, 1, 1, 128, M, n, k, None, 0)
+                                   out.data_ptr(), _lib.I8, _lib.F16, 4, 1, 1, 128, m, n, k, None, 0)
         if st != 0:
             raise RuntimeError(f"ofq_fused_linear_gq status {st}")
 
-    def step_all():
+    def step_all(m=M):
         for mats in layers:
             for mat in mats:
-                launch(mat)
+                launch(mat, m)
 
     def step_dominant():
         for mats in layers:
@@ -191,9 +191,22 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(M)
     if not args.no_secondary:
+        # the same decode step at the other batch sizes of the decode configuration
+        other = {}
+        for m in (4, 8):
+            if m == M:
+                continue
+            run_m = make_runner(lambda: step_all(m))
+            _, wall_m = time_region(run_m, 10, 2)
+            b_m = sum(gemv_bytes(m, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER) * args.layers
+            gbps = b_m / (wall_m / 10 * 1e-3) / 1e9
+            other[f"decode_w4a16_m{m}"] = {
+                "ms_per_step": round(wall_m / 10, 4), "gbps": round(gbps, 1),
+                "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+                             "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
         del layers
         torch.cuda.empty_cache()
-        result["secondary"] = secondary(L, _lib, torch, dev, args)
+        result["secondary"] = {**other, **secondary(L, _lib, torch, dev, args)}
     print(json.dumps(result))
 
 

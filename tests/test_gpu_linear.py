@@ -101,6 +101,22 @@ def test_decode_w4a16_row_balanced_shapes(m, n, k, container):
     assert np.array_equal(got.astype(np.int64), exact)
 
 
+@pytest.mark.parametrize("m,n,k", [(16, 80, 8192), (8, 48, 11008), (13, 4096, 4096)])
+@pytest.mark.parametrize("symmetric,qdt", VARIANTS)
+def test_decode_w4a16_large_x(m, n, k, symmetric, qdt):
+    """m * k too large for x to be staged in LDS: the kernels that read x from L2 per chunk, for
+    all three code variants."""
+    rng = np.random.Generator(np.random.PCG64(m * 131 + n))
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), "f16")
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    w, scale, zero = H.quantize_groupwise(wf, 4, symmetric, 1, 128, qdt, "f16")
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), "f16")
+    ref = O.fused_linear(x, w, scale, zero, b, 4, symmetric, 1, 128)
+    got = _run(x, w, scale, zero, b, 4, symmetric, 1, 128)
+    r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k}")
+    assert r < (5e-4 if (symmetric and qdt == np.int8) else 1e-4)
+
+
 def test_decode_m_invariance_and_integer_case():
     """Row i of an m=8 call agrees with the m=1 call on that row (the two batch sizes take
     different code paths: x staged in LDS or not, so agreement is to fp32-accumulation noise, at
