@@ -396,6 +396,38 @@ def secondary(L, _lib, torch, dev, args):
                                   "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
     del wsrc, qo
 
+    # ---- decode through the natural-order kernel: bf16 W4 asymmetric g=128 and fp16 W8 g=64, --
+    # m = 1 and 16, gate/up shape; 8 weight sets cycled so that no launch finds its codes in cache
+    n, k = 11008, 4096
+    for tag, tcode, tdt, bits, g in (("bf16_w4_asym_g128", _lib.BF16, torch.bfloat16, 4, 128),
+                                     ("f16_w8_asym_g64", _lib.F16, torch.float16, 8, 64)):
+        reps = 8
+        ws = [torch.randint(0, 256, (n, k * bits // 8), dtype=torch.uint8, device=dev) for _ in range(reps)]
+        sc = torch.empty((n, k // g), device=dev).uniform_(1e-3, 1e-2).to(tdt)
+        ze = torch.empty((n, k // g), device=dev).uniform_(0.01, 0.05).to(tdt)
+        for m in (1, 16):
+            xx = torch.randn((m, k), device=dev).to(tdt)
+            oo = torch.empty((m, n), dtype=tdt, device=dev)
+
+            def dec():
+                for i in range(reps):
+                    chk(L.ofq_fused_linear_gq(cs(), xx.data_ptr(), ws[i].data_ptr(), sc.data_ptr(),
+                                              ze.data_ptr(), None, oo.data_ptr(), _lib.U8, tcode, bits,
+                                              0, 1, g, m, n, k, None, 0), "decode " + tag)
+            dec()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                dec()
+            us = timeit(gr.replay, iters=10) / reps
+            nbytes = n * k * bits // 8 + 2 * n * (k // g) * 2 + m * k * 2 + m * n * 2
+            gb = nbytes / (us * 1e-6) / 1e9
+            out[f"decode_{tag}_11008x4096_m{m}"] = {
+                "us": round(us, 2), "gbps": round(gb, 1),
+                "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS,
+                             "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+        del ws
+
     # ---- weight quantise + pack: fp16 [11008,4096] -> symmetric int4, g=128 -------------------
     n, k, g = 11008, 4096, 128
     reps = 6  # 6 x 90 MB of distinct sources: beyond the caches

@@ -3,6 +3,7 @@
 // experiments can instantiate tile configurations directly.
 #pragma once
 
+#include "dequant_regs.h"
 #include "ofq_device.h"
 
 namespace ofq {
@@ -205,71 +206,6 @@ struct B2Copy {
   }
   static __device__ __forceinline__ void store_part(const Params&, const Regs&, uint8_t*, int, int) {}
 };
-
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-
-// 16 values of T (two 128-bit pieces) from 16 byte codes, w~ = T(T(q)*s) + z.
-// bf16: v_cvt_f32_ubyteN, v_mul_f32, v_cvt_pk_bf16_f32, re-widen, v_add_f32, v_cvt_pk_bf16_f32
-// (5 vector instructions per element); fp16: the 0x6400 trick with packed fp16 math (2 per element).
-template<typename T, bool SIGNED, int ZMODE>
-__device__ __forceinline__ void dequant16_b8(const u32x4 codes, float s, float z, u32x4& o0,
-                                             u32x4& o1) {
-  uint32_t r[8];
-  if constexpr (TT<T>::dtype == OFQ_BF16 && !SIGNED) {
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const uint32_t x = codes[w];
-      const f32x2 p01 = {(float)(x & 0xFFu) * s, (float)((x >> 8) & 0xFFu) * s};
-      const f32x2 p23 = {(float)((x >> 16) & 0xFFu) * s, (float)(x >> 24) * s};
-      uint32_t r01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(p01, bf16x2_t));
-      uint32_t r23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(p23, bf16x2_t));
-      if (ZMODE != 0) {
-        const f32x2 a01 = {__builtin_bit_cast(float, r01 << 16) + z,
-                           __builtin_bit_cast(float, r01 & 0xFFFF0000u) + z};
-        const f32x2 a23 = {__builtin_bit_cast(float, r23 << 16) + z,
-                           __builtin_bit_cast(float, r23 & 0xFFFF0000u) + z};
-        r01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(a01, bf16x2_t));
-        r23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(a23, bf16x2_t));
-      }
-      r[2 * w] = r01;
-      r[2 * w + 1] = r23;
-    }
-  } else if constexpr (TT<T>::dtype == OFQ_F16) {
-    const f16 sh = (f16)s, zh = (f16)z;  // s and z were widened from fp16: exact
-    const f16x2 s2 = {sh, sh}, z2 = {zh, zh};
-    const f16 off = SIGNED ? (f16)(-1152.0f) : (f16)(-1024.0f);
-    const f16x2 off2 = {off, off};
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      uint32_t word = codes[w];
-      if (SIGNED) word ^= 0x80808080u;
-      f16x2 a = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(word, 0x64646464u, 0x00050004u)) + off2;
-      f16x2 b = __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(word, 0x64646464u, 0x00070006u)) + off2;
-      a = a * s2;
-      b = b * s2;
-      if (ZMODE != 0) {
-        a = a + z2;
-        b = b + z2;
-      }
-      r[2 * w] = __builtin_bit_cast(uint32_t, a);
-      r[2 * w + 1] = __builtin_bit_cast(uint32_t, b);
-    }
-  } else {
-    typename TT<T>::storage vals[16];
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const uint32_t b = (codes[e >> 2] >> ((e & 3) * 8)) & 0xFFu;
-      const int code = SIGNED ? (int)(int8_t)b : (int)b;
-      float v = TT<T>::round((float)code * s);
-      if (ZMODE != 0) v = v + z;
-      TT<T>::store(&vals[e], v);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = reinterpret_cast<const uint32_t*>(vals)[i];
-  }
-  o0 = u32x4{r[0], r[1], r[2], r[3]};
-  o1 = u32x4{r[4], r[5], r[6], r[7]};
-}
 
 // Groupwise-quantised weights: codes are loaded as stored
 // ([N, K*bits/8] bytes) two k-tiles ahead, and turned into T when written to the swizzled LDS tile.

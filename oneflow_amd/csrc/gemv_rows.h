@@ -1,0 +1,294 @@
+// Decode kernel of fused_linear_with_groupwise_quantized_weight for every 16-bit element type
+// and both code widths, with x kept in its natural order.
+//
+// Same row split as gemv_w4p_f16 (a whole number of blocks per CU, each owning consecutive
+// weight rows that it walks as 16-row tiles; the m <= 16 rows of x ride as the first operand of
+// a 16x16x32 MFMA, so the weights stream from HBM once whatever m is), but the codes are
+// expanded to T in natural element order by dequant8_b4 / dequant16_b8:
+//   w~ = T(T(q) * s) + z  with the reference's roundings
+//   (oneflow/user/kernels/groupwise_quantization_kernels.cu:73-117, :582-642),
+// so bf16 (whose products have to be rounded in fp32 arithmetic: there is no packed bf16 math)
+// and 8-bit codes get the same treatment as the fp16 4-bit case.  Groups may be as short as one
+// lane's 16 bytes of codes (32 4-bit or 16 8-bit elements).
+#pragma once
+
+#include "dequant_regs.h"
+#include "ofq_device.h"
+
+namespace ofq {
+namespace {
+
+constexpr int kRowsMaxTiles = 4;   // 16-row tiles per block
+constexpr int kRowsMaxUnits = 8;   // 16-byte pieces of x a thread may stage
+
+template<typename T>
+struct MfmaK32;
+template<>
+struct MfmaK32<f16> {
+  static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template<>
+struct MfmaK32<bf16> {
+  static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+// raw bits of a T -> float at the point of use (keeps the load's wait where the value is needed)
+template<typename T>
+__device__ __forceinline__ float raw16_at_end(uint16_t raw) {
+  uint32_t v = raw;
+  asm volatile("" : "+v"(v));
+  if constexpr (TT<T>::dtype == OFQ_BF16) {
+    return __builtin_bit_cast(float, v << 16);
+  } else {
+    return (float)__builtin_bit_cast(f16, (uint16_t)v);
+  }
+}
+
+// STAGED: x is copied to LDS once per block (m * k small enough); otherwise every wave reads the
+// x of its chunk pairs straight from global memory (x stays in L2: it is re-read by every block).
+// Either way a wave takes chunk pairs p = wave, wave + NWAVES, ... and walks all tiles of the
+// block for each, so x is fetched once per pair and the per-tile sums stay in registers.
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, bool STAGED>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_rows(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
+          const uint16_t* __restrict__ scale, const uint16_t* __restrict__ zero,
+          const uint16_t* __restrict__ bias, uint16_t* __restrict__ out, int M, int N, int K,
+          int group_size, int gs_shift, int rows_per_block) {
+  typedef typename TT<T>::storage S;
+  static_assert(sizeof(S) == 2, "16-bit element types");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NT = NWAVES * 64;
+  constexpr int CK = BITS == 4 ? 128 : 64;  // elements per chunk: 64 bytes of codes per row
+  constexpr int LK = CK / 4;                // elements per lane and chunk
+  constexpr int XV = LK / 8;                // 16-byte pieces of x per lane and chunk
+  const int nchunks = K / CK;
+  const int npairs = (nchunks + 1) >> 1;
+  const int row_bytes = nchunks * 64;
+  const int G = K / group_size;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15;
+  const int kb = lane >> 4;
+  const int row0 = blockIdx.x * rows_per_block;
+  int rows_blk = N - row0;
+  if (rows_blk > rows_per_block) rows_blk = rows_per_block;
+  if (rows_blk <= 0) return;
+  const int ntiles = (rows_blk + 15) >> 4;
+  const bool has_x = r < M;
+
+  // LDS: [red kRowsMaxTiles*NWAVES*M*16 f32][scales rows_per_block*G, padded to 16 B]
+  //      [zeros, same size (asymmetric only)][64 zero bytes][x: M rows of K*2+16 bytes (STAGED)]
+  float* red = reinterpret_cast<float*>(smem);
+  const int red_floats = kRowsMaxTiles * NWAVES * M * 16;
+  const int tile_bytes = (rows_per_block * G * 2 + 15) & ~15;
+  uint16_t* sl = reinterpret_cast<uint16_t*>(smem + (size_t)red_floats * 4);
+  uint16_t* zl = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
+  uint8_t* zrec = reinterpret_cast<uint8_t*>(sl) + (ZMODE == kZeroAsym ? 2 : 1) * tile_bytes;
+  uint8_t* xs = zrec + 64;
+  const int x_pitch = K * 2 + 16;  // rows skewed by 16 bytes: lanes of different m reading the
+                                   // same k hit different LDS bank groups
+
+  // ---- requests that feed LDS go out first ----------------------------------------------------
+  const int upr = K >> 3;  // 16-byte pieces per row of x
+  const int nunits = M * upr;
+  u32x4 xu[kRowsMaxUnits];
+  if (STAGED) {
+#pragma unroll
+    for (int i = 0; i < kRowsMaxUnits; ++i) {
+      if (wave * 64 + i * NT >= nunits) break;
+      const int u = tid + i * NT;
+      if (u < nunits) xu[i] = *reinterpret_cast<const u32x4*>(x + (int64_t)u * 8);
+    }
+  }
+  const int tile_halves = rows_blk * G;
+  const uint16_t* stile = scale + (int64_t)row0 * G;
+  const bool s_aligned = ((reinterpret_cast<uintptr_t>(stile)) & 15u) == 0;
+  const uint16_t* ztile = ZMODE == kZeroAsym ? zero + (int64_t)row0 * G : stile;
+  u32x4 sreg, zreg;
+  const int se = tid * 8;
+  const bool s_vec = s_aligned && se + 8 <= tile_halves;
+  if (s_vec) {
+    sreg = *reinterpret_cast<const u32x4*>(stile + se);
+    if (ZMODE == kZeroAsym) zreg = *reinterpret_cast<const u32x4*>(ztile + se);
+  }
+  // bias of the first output this thread folds at the end: tid = (tile * M + m) * 16 + n
+  uint16_t bias_raw = 0;
+  {
+    const int t = tid / (M * 16);
+    const int row_l = t * 16 + (tid & 15);
+    if (bias != nullptr && t < ntiles && row_l < rows_blk) bias_raw = bias[row0 + row_l];
+  }
+
+  // ---- codes of (tile, pair): one 16-byte load per lane and chunk ------------------------------
+  const uint8_t* wbase = w + (int64_t)row0 * row_bytes + kb * 16;
+  // Straight-line on purpose: a load under a branch makes the compiler wait for everything in
+  // flight at the first LDS fill.  A slot without an item reads one and the same 16 bytes in
+  // every lane; lanes past the block's rows re-read its first row (never stored).
+  auto issue = [&](int tile, int pair, u32x4 (&dst)[2], bool live) {
+    const int row_l = tile * 16 + r;
+    const bool ok = row_l < rows_blk;
+    const uint8_t* p = wbase + (int64_t)(ok ? row_l : 0) * row_bytes;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = 2 * pair + u;
+      const uint8_t* q = p + (c < nchunks ? c : 0) * 64;
+      dst[u] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4*>(live ? q : w + (int64_t)row0 * row_bytes));
+    }
+  };
+  int pair = wave;
+  u32x4 wq[2];
+  {
+    const bool live = pair < npairs;
+    issue(0, live ? pair : 0, wq, live);
+  }
+
+  // ---- fill LDS -------------------------------------------------------------------------------
+  if (s_vec) {
+    *reinterpret_cast<u32x4*>(sl + se) = sreg;
+    if (ZMODE == kZeroAsym) *reinterpret_cast<u32x4*>(zl + se) = zreg;
+  } else if (se < tile_halves && s_aligned) {
+    for (int j = se; j < tile_halves && j < se + 8; ++j) {
+      sl[j] = stile[j];
+      if (ZMODE == kZeroAsym) zl[j] = ztile[j];
+    }
+  }
+  for (int e = (s_aligned ? NT * 8 : 0) + tid; e < tile_halves; e += NT) {
+    sl[e] = stile[e];
+    if (ZMODE == kZeroAsym) zl[e] = ztile[e];
+  }
+  if (STAGED) {
+    if (tid < 16) reinterpret_cast<uint32_t*>(zrec)[tid] = 0u;
+    // piece u of x lies in row u / upr; rows advance by (NT / upr, NT % upr) per step
+    const int qstep = NT / upr, rstep = NT - qstep * upr;
+    int xrow = tid / upr, xrem = tid - xrow * upr;
+#pragma unroll
+    for (int i = 0; i < kRowsMaxUnits; ++i) {
+      if (wave * 64 + i * NT >= nunits) break;
+      if (tid + i * NT < nunits) {
+        *reinterpret_cast<u32x4*>(xs + (size_t)xrow * x_pitch + xrem * 16) = xu[i];
+      }
+      xrow += qstep;
+      xrem += rstep;
+      if (xrem >= upr) {
+        xrem -= upr;
+        ++xrow;
+      }
+    }
+  }
+  __syncthreads();
+
+  // this lane's 2 * LK bytes of x per chunk: row r, k-slot kb.  Lanes r >= M feed rows of the
+  // product that are never stored: a zero record (STAGED) or row 0 again (same addresses as the
+  // lanes of r = 0, no extra traffic).
+  const uint8_t* xlane;
+  int xstride = CK * 2;
+  if (STAGED) {
+    xlane = has_x ? xs + (size_t)r * x_pitch + kb * (LK * 2) : zrec;
+    if (!has_x) xstride = 0;
+  } else {
+    xlane = reinterpret_cast<const uint8_t*>(x) + ((size_t)(has_x ? r : 0) * K + kb * LK) * 2;
+  }
+  f32x4 acc[kRowsMaxTiles][2];
+#pragma unroll
+  for (int t = 0; t < kRowsMaxTiles; ++t) {
+    acc[t][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc[t][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  while (pair < npairs) {
+    u32x4 xa[2][XV];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = 2 * pair + u;
+      const u32x4* xp = reinterpret_cast<const u32x4*>(xlane + (size_t)(c < nchunks ? c : 0) * xstride);
+#pragma unroll
+      for (int j = 0; j < XV; ++j) xa[u][j] = xp[j];
+    }
+#pragma unroll
+    for (int t = 0; t < kRowsMaxTiles; ++t) {
+      if (t < ntiles) {
+        const int srow = (t * 16 + r) * G;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int c = 2 * pair + u;
+          if (c < nchunks) {
+            const int k0 = c * CK + kb * LK;
+            const int grp = gs_shift >= 0 ? (k0 >> gs_shift) : (k0 / group_size);
+            const float s = TT<T>::load(reinterpret_cast<const S*>(sl) + srow + grp);
+            float z = 0.f;
+            if (ZMODE == kZeroAsym) z = TT<T>::load(reinterpret_cast<const S*>(zl) + srow + grp);
+            if (ZMODE == kZeroSymU) z = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * s);
+            if constexpr (BITS == 4) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const u32x4 b = dequant8_b4<T, SIGNED, ZMODE>(wq[u][j], s, z);
+                // two accumulators: consecutive MFMAs do not wait for each other
+                acc[t][j & 1] = MfmaK32<T>::mma(xa[u][j], b, acc[t][j & 1]);
+              }
+            } else {
+              u32x4 b0, b1;
+              dequant16_b8<T, SIGNED, ZMODE>(wq[u], s, z, b0, b1);
+              acc[t][0] = MfmaK32<T>::mma(xa[u][0], b0, acc[t][0]);
+              acc[t][1] = MfmaK32<T>::mma(xa[u][1], b1, acc[t][1]);
+            }
+          }
+        }
+        // codes of the next item: the next tile of this pair, else tile 0 of the wave's next pair
+        const bool last_t = t + 1 >= ntiles;
+        const int np = last_t ? pair + NWAVES : pair;
+        const bool live = np < npairs;
+        issue(last_t ? 0 : t + 1, live ? np : 0, wq, live);
+      }
+    }
+    pair += NWAVES;
+  }
+  // every wave writes its sums of every tile (zeros when it had no pair)
+#pragma unroll
+  for (int t = 0; t < kRowsMaxTiles; ++t) {
+    if (t < ntiles) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = 4 * kb + v;
+        if (m < M) red[((t * NWAVES + wave) * M + m) * 16 + r] = acc[t][0][v] + acc[t][1][v];
+      }
+    }
+  }
+  __syncthreads();
+  const int nout = ntiles * M * 16;
+  for (int o = tid; o < nout; o += NT) {
+    const int t = o / (M * 16);
+    const int rem = o - t * (M * 16);  // m * 16 + n
+    float sum = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < NWAVES; ++wv) sum += red[(t * NWAVES + wv) * M * 16 + rem];
+    const int m = rem >> 4;
+    const int row_l = t * 16 + (rem & 15);
+    if (row_l < rows_blk) {
+      float bv;
+      if (o == tid) {
+        bv = raw16_at_end<T>(bias_raw);
+      } else {
+        bv = bias != nullptr ? TT<T>::load(reinterpret_cast<const S*>(bias) + row0 + row_l) : 0.f;
+      }
+      TT<T>::store(reinterpret_cast<S*>(out) + (int64_t)m * N + row0 + row_l, sum + bv);
+    }
+  }
+}
+
+inline size_t gemv_rows_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,
+                                  bool asym, bool staged) {
+  const int G = K / group_size;
+  return (size_t)kRowsMaxTiles * nwaves * M * 16 * 4
+         + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15) + 64
+         + (staged ? (size_t)M * (K * 2 + 16) : 0);
+}
+
+}  // namespace
+}  // namespace ofq

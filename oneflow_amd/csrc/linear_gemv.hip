@@ -27,6 +27,7 @@
 //   - partial sums of the waves are combined through LDS, bias is added in fp32, one rounding
 //     to T.
 #include "gemv_kernels.h"
+#include "gemv_rows.h"
 #include "ofq_device.h"
 #include "ofq_internal.h"
 
@@ -160,6 +161,8 @@ int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift) {
   const bool two_per_cu = grid > kCUs;
   const int nw = two_per_cu ? 8 : 16;
   if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
+  // one thread folds one output of the block
+  if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) return OFQ_ERR_UNSUPPORTED;
   const bool exact = !(a.symmetric && a.w_signed);
   const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
                                         !a.symmetric);
@@ -178,6 +181,87 @@ int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift) {
   OFQ_W4P(16) OFQ_W4P(8)
 #undef OFQ_W4P
   return OFQ_ERR_UNSUPPORTED;
+}
+
+// ---- natural-order row-balanced kernel (gemv_rows): fp16 / bf16, 4- and 8-bit ----------------
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
+int launch_rows_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block,
+                     size_t lds, int gs_shift) {
+  auto kern = gemv_rows<T, BITS, SIGNED, ZMODE, NW, STAGED>;
+  static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be allowed once
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, NW * 64, lds, st>>>(
+      static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.w),
+      static_cast<const uint16_t*>(a.scale), static_cast<const uint16_t*>(a.zero),
+      static_cast<const uint16_t*>(a.bias), static_cast<uint16_t*>(a.out), (int)a.m, (int)a.n,
+      (int)a.k, (int)a.group_size, gs_shift, rows_per_block);
+  return ofq_check_launch();
+}
+
+bool rows_supported(const LinearArgs& a) {
+  if (a.t_dtype != OFQ_F16 && a.t_dtype != OFQ_BF16) return false;
+  if (a.bits != 4 && a.bits != 8) return false;
+  const int ck = a.bits == 4 ? 128 : 64;
+  return a.group_dim == 1 && a.m >= 1 && a.m <= 16 && a.k % ck == 0
+         && a.group_size % (ck / 4) == 0 && a.k <= (1 << 20) && a.n <= 0x7FFFFFFF - 16
+         && (a.symmetric || !a.w_signed);
+}
+
+template<typename T, int NW>
+int launch_rows_t(hipStream_t st, const LinearArgs& a, int grid, int rpb, size_t lds,
+                  bool staged) {
+  const int gs_shift = ilog2_exact(a.group_size);
+  const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
+#define OFQ_R(B, SG, ZM)                                              \
+  if (a.bits == B && a.w_signed == SG && zmode == ZM)                 \
+    return staged ? launch_rows_inst<T, B, SG, ZM, NW, true>(st, a, grid, rpb, lds, gs_shift) \
+                  : launch_rows_inst<T, B, SG, ZM, NW, false>(st, a, grid, rpb, lds, gs_shift);
+  OFQ_R(4, true, kZeroNone)
+  OFQ_R(4, false, kZeroSymU)
+  OFQ_R(4, false, kZeroAsym)
+  OFQ_R(8, true, kZeroNone)
+  OFQ_R(8, false, kZeroSymU)
+  OFQ_R(8, false, kZeroAsym)
+#undef OFQ_R
+  return OFQ_ERR_UNSUPPORTED;
+}
+
+// OFQ_ERR_UNSUPPORTED when x does not fit the block's registers and LDS
+int launch_rows(hipStream_t st, const LinearArgs& a) {
+  constexpr int kCUs = 256;
+  const int64_t max_rows = 16 * kRowsMaxTiles;
+  int64_t grid = kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
+  int rpb = (int)((a.n + grid - 1) / grid);
+  if (rpb < 16) rpb = 16;
+  grid = (a.n + rpb - 1) / rpb;
+  const bool two_per_cu = grid > kCUs;
+  const int nw = two_per_cu ? 8 : 16;
+  const size_t cap = (two_per_cu ? 80u : 160u) * 1024u;
+  // x goes to LDS when it fits there and in the staging registers; else it is read from L2
+  bool staged = a.m * a.k / 8 <= (int64_t)kRowsMaxUnits * nw * 64;
+  size_t lds = gemv_rows_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb,
+                                   !a.symmetric, staged);
+  if (staged && lds > cap) {
+    staged = false;
+    lds = gemv_rows_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, !a.symmetric,
+                              false);
+  }
+  if (lds > cap) return OFQ_ERR_UNSUPPORTED;
+  if (a.t_dtype == OFQ_BF16) {
+    return nw == 16 ? launch_rows_t<bf16, 16>(st, a, (int)grid, rpb, lds, staged)
+                    : launch_rows_t<bf16, 8>(st, a, (int)grid, rpb, lds, staged);
+  }
+  return nw == 16 ? launch_rows_t<f16, 16>(st, a, (int)grid, rpb, lds, staged)
+                  : launch_rows_t<f16, 8>(st, a, (int)grid, rpb, lds, staged);
 }
 
 int launch_w4s(hipStream_t st, const LinearArgs& a) {
@@ -199,8 +283,14 @@ int launch_w4s(hipStream_t st, const LinearArgs& a) {
   // More than one 16-row tile per CU, or an x too large to stage per 16 rows: the row-balanced
   // kernel (equal bytes per block, x staged once per block) is the faster one.
   if (tiles > 256 || !staged) {
-    const int rc = launch_w4p(st, a, cpg_shift);
+    int rc = launch_w4p(st, a, cpg_shift);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+    // x too large for either staged kernel: the natural-order kernel reads x from L2 once per
+    // block, the one below once per 16 rows
+    if (!staged) {
+      rc = launch_rows(st, a);
+      if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+    }
   }
 #define OFQ_W4S(NWV)                                                                   \
   if (nw == NWV)                                                                       \
@@ -240,6 +330,7 @@ int launch_gemv_variant(hipStream_t st, const LinearArgs& a) {
 }  // namespace
 
 bool gemv_wq_supported(const LinearArgs& a) {
+  if (rows_supported(a)) return true;
   if (a.t_dtype != OFQ_F16 || a.group_dim != 1 || a.m > 16 || a.m < 1) return false;
   const int ch = a.bits == 4 ? 128 : 64;
   const int lk = ch / 4;
@@ -256,6 +347,15 @@ int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
     // uint8 container / asymmetric: the row-balanced kernel with the reference's roundings
     const int rc = launch_w4p(st, a, ilog2_exact(a.group_size / 128));
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
+  if (rows_supported(a)) {
+    const int rc = launch_rows(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
+  if (a.t_dtype != OFQ_F16) return OFQ_ERR_UNSUPPORTED;  // the kernels below are fp16 only
+  {
+    const int ch = a.bits == 4 ? 128 : 64;
+    if (a.k % ch != 0 || a.group_size % (ch / 4) != 0) return OFQ_ERR_UNSUPPORTED;
   }
   const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
 #define OFQ_V(B, SG, ZM) \
@@ -349,7 +449,10 @@ extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
   a.n = n;
   a.k = k;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (gemv_wq_supported(a)) return launch_gemv_wq(st, a);
+  if (gemv_wq_supported(a)) {
+    const int rc = launch_gemv_wq(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;  // e.g. bf16 with an x too large to stage
+  }
   if (gemm_wq_supported(a)) return launch_gemm_wq(st, a, workspace, workspace_bytes);
   return launch_linear_generic(st, a);
 }

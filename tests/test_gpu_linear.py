@@ -117,6 +117,38 @@ def test_decode_w4a16_large_x(m, n, k, symmetric, qdt):
     assert r < (5e-4 if (symmetric and qdt == np.int8) else 1e-4)
 
 
+@pytest.mark.parametrize("m,n,k,group_size", [
+    (1, 4096, 4096, 128), (4, 11008, 4096, 64), (16, 5000, 512, 32), (3, 4099, 384, 64),
+    (2, 40000, 256, 128), (16, 16400, 1024, 128), (5, 4096, 11008, 128), (7, 100, 128, 16)])
+@pytest.mark.parametrize("num_bits", [4, 8])
+@pytest.mark.parametrize("t", ["bf16", "f16"])
+def test_decode_natural_order_kernel(m, n, k, group_size, num_bits, t):
+    """Decode (m <= 16) for bf16 and for 8-bit codes, fp16 with groups shorter than 128, all three
+    code variants: row counts per block that are not multiples of 16, partial last blocks, two
+    blocks per CU, more outputs per block than threads, groups as short as one lane's load."""
+    if num_bits == 4 and group_size % 32 != 0:
+        group_size = 32
+    rng = np.random.Generator(np.random.PCG64(m * 977 + n + num_bits))
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), t)
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), t)
+    for symmetric, qdt in VARIANTS:
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, group_size, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, group_size)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, group_size)
+        r, e = H.assert_linear_parity(got, ref, t, f"{t} b{num_bits} m={m} n={n} k={k} {symmetric} {qdt}")
+        # w~ is formed with the oracle's roundings, only the order of the sum differs: the
+        # outputs agree to a rounding of T on a few elements
+        # (fp16, int8 container, 4 bits, groups of 128 take the kernel that leaves w~ = q*s
+        # unrounded: ~3e-4)
+        shortcut = t == "f16" and num_bits == 4 and qdt == np.int8 and group_size % 128 == 0
+        assert r < (3e-3 if t == "bf16" else 5e-4 if shortcut else 1e-4), (r, symmetric, qdt)
+        # and no element is off by more than one rounding of T (2e-4 absolute where cancellation
+        # leaves an output far smaller than its terms)
+        gf, rf = O.to_f32(got).astype(np.float64), O.to_f32(ref).astype(np.float64)
+        assert (np.abs(gf - rf) <= np.maximum(H.ulp_of(rf, t), 2e-4) * (1 + 1e-9)).all() or shortcut
+
+
 def test_decode_m_invariance_and_integer_case():
     """Row i of an m=8 call agrees with the m=1 call on that row (the two batch sizes take
     different code paths: x staged in LDS or not, so agreement is to fp32-accumulation noise, at
