@@ -2,8 +2,10 @@
 //   (1) fused_linear_with_groupwise_quantized_weight for m > 16: either the weight tile is
 //       dequantised on its way into LDS and feeds fp16/bf16 MFMA (the fp16/bf16 copy of the
 //       weight that the reference materialises for m > 8,
-//       oneflow/core/functional/impl/quantization.cpp:341-350, then never touches HBM), or, at
-//       large m with a workspace, the weight is dequantised once and a copy-fed GEMM runs on it;
+//       oneflow/core/functional/impl/quantization.cpp:341-350, then never touches HBM), cut
+//       along K into separate blocks when a workspace for partial sums is given and the tiles
+//       alone would not fill the chip; or, at large m with a workspace, the weight is
+//       dequantised once and a copy-fed GEMM runs on it;
 //   (2) matmul_quant: int8 x int8 -> int32 MFMA with a per-row/per-tensor scale epilogue.
 //
 // All are instances of one byte-oriented core (gemm_kernels.h).  A tile row is always 128 bytes
@@ -48,8 +50,64 @@ int launch_plain(hipStream_t st, const LinearArgs& a, const void* wt) {
                                                                 a.k / 64);
 }
 
+// Few blocks (m small against the tile height, or few weight tiles): K is cut into `splits`
+// slices that run as separate blocks, each writing fp32 partial sums of the whole output tile to
+// its slice of the workspace; splitk_finalize adds the slices in order (so the result does not
+// depend on scheduling), adds the bias and rounds to T once.
+template<typename T, int VEC>
+__global__ void __launch_bounds__(256)
+splitk_finalize(const float* __restrict__ part, const typename TT<T>::storage* __restrict__ bias,
+                typename TT<T>::storage* __restrict__ out, int64_t MN, int N, int splits) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (i >= MN) return;
+  float acc[VEC];
+  if constexpr (VEC == 4) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(part + i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = v[e];
+    for (int sidx = 1; sidx < splits; ++sidx) {
+      const f32x4 u = *reinterpret_cast<const f32x4*>(part + (int64_t)sidx * MN + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] += u[e];
+    }
+  } else {
+    acc[0] = part[i];
+    for (int sidx = 1; sidx < splits; ++sidx) acc[0] += part[(int64_t)sidx * MN + i];
+  }
+  const int n = (int)(i % N);  // VEC divides N: the VEC elements share a row
+  typename TT<T>::storage o[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    float v = acc[e];
+    if (bias != nullptr) v += TT<T>::load(bias + n + e);
+    TT<T>::store(&o[e], v);
+  }
+  if constexpr (VEC == 4) {
+    *reinterpret_cast<u32x2*>(out + i) = *reinterpret_cast<const u32x2*>(o);
+  } else {
+    out[i] = o[0];
+  }
+}
+
+// Slices of K for the in-tile path: as many as still fit the blocks into one resident round
+// (256x128 tiles: one 8-wave block per CU; 128x128: two 4-wave blocks), each at least 4 k-tiles.
+int wq_splits(const LinearArgs& a) {
+  if (a.m >= 1024) return 1;  // two-pass territory
+  const int64_t bm = a.m > 128 ? 256 : 128;
+  const int64_t slots = a.m > 128 ? 256 : 512;
+  const int64_t blocks = ((a.m + bm - 1) / bm) * ((a.n + 127) / 128);
+  int64_t s = slots / blocks;
+  const int64_t kt = a.k / 64;
+  if (s > 8) s = 8;
+  if (s > kt / 4) s = kt / 4;
+  if (s < 1) s = 1;
+  // no empty last slice
+  while (s > 1 && ((kt + s - 1) / s) * (s - 1) >= kt) --s;
+  return (int)s;
+}
+
 template<typename T, class MF, int BITS, bool SIGNED, int ZMODE>
-int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
+int launch_wq_variant(hipStream_t st, const LinearArgs& a, float* partials, int splits) {
   typedef typename TT<T>::storage S;
   typedef EpBias<T> EP;
   WqParams<T> bp;
@@ -63,6 +121,28 @@ int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
   typename EP::Params ep;
   ep.bias = static_cast<const S*>(a.bias);
   ep.out = static_cast<S*>(a.out);
+  if (partials != nullptr && splits > 1) {
+    EpPartial::Params pp;
+    pp.out = partials;
+    int rc;
+    if (a.m > 128) {
+      rc = launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 512>, EpPartial, 256, 128, 4,
+                        2>(st, a.x, a.k * 2, bp, pp, a.m, a.n, a.k / 64, splits);
+    } else {
+      rc = launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 256>, EpPartial, 128, 128, 2,
+                        2>(st, a.x, a.k * 2, bp, pp, a.m, a.n, a.k / 64, splits);
+    }
+    if (rc != OFQ_OK) return rc;
+    const int64_t mn = a.m * a.n;
+    if (a.n % 4 == 0) {
+      splitk_finalize<T, 4><<<(unsigned)((mn / 4 + 255) / 256), 256, 0, st>>>(
+          partials, ep.bias, ep.out, mn, (int)a.n, splits);
+    } else {
+      splitk_finalize<T, 1><<<(unsigned)((mn + 255) / 256), 256, 0, st>>>(
+          partials, ep.bias, ep.out, mn, (int)a.n, splits);
+    }
+    return ofq_check_launch();
+  }
   // 256x128 tiles on 8 waves when there are enough rows of x to fill them, else 128x128 on 4
   if (a.m > 128) {
     return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 512>, EP, 256, 128, 4, 2>(
@@ -80,11 +160,11 @@ int launch_wq_variant(hipStream_t st, const LinearArgs& a) {
 }
 
 template<typename T, class MF>
-int launch_wq_t(hipStream_t st, const LinearArgs& a) {
+int launch_wq_t(hipStream_t st, const LinearArgs& a, float* partials, int splits) {
   const int zmode = !a.symmetric ? 2 : (a.w_signed ? 0 : 1);
 #define OFQ_V(B, SG, ZM)                                       \
   if (a.bits == B && a.w_signed == SG && zmode == ZM)          \
-    return launch_wq_variant<T, MF, B, SG, ZM>(st, a);
+    return launch_wq_variant<T, MF, B, SG, ZM>(st, a, partials, splits);
   OFQ_V(4, true, 0)
   OFQ_V(4, false, 1)
   OFQ_V(4, false, 2)
@@ -110,13 +190,23 @@ bool gemm_wq_supported(const LinearArgs& a) {
 // once into the workspace and running the copy-fed GEMM on it is what the reference functor does
 // for m > 8 (oneflow/core/functional/impl/quantization.cpp:341-350).
 size_t gemm_wq_workspace_bytes(const LinearArgs& a) {
-  if (!gemm_wq_supported(a) || a.m < 1024) return 0;
-  return (size_t)a.n * (size_t)a.k * 2;
+  if (!gemm_wq_supported(a)) return 0;
+  if (a.m >= 1024) return (size_t)a.n * (size_t)a.k * 2;
+  const int splits = wq_splits(a);
+  return splits > 1 ? (size_t)splits * (size_t)a.m * (size_t)a.n * 4 : 0;  // fp32 partial sums
 }
 
 int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t workspace_bytes) {
   const size_t need = gemm_wq_workspace_bytes(a);
-  if (need != 0 && workspace != nullptr && workspace_bytes >= need && ofq_aligned16(workspace)) {
+  const bool have_ws =
+      need != 0 && workspace != nullptr && workspace_bytes >= need && ofq_aligned16(workspace);
+  if (have_ws && a.m < 1024) {
+    float* partials = static_cast<float*>(workspace);
+    const int splits = wq_splits(a);
+    if (a.t_dtype == OFQ_F16) return launch_wq_t<f16, MfmaF16>(st, a, partials, splits);
+    return launch_wq_t<bf16, MfmaBF16>(st, a, partials, splits);
+  }
+  if (have_ws) {
     const int rc = ofq_groupwise_dequantize(st, a.w, a.scale, a.zero, workspace,
                                             a.w_signed ? OFQ_I8 : OFQ_U8, a.t_dtype, a.bits,
                                             a.symmetric ? 1 : 0, a.n * (a.k / a.group_size),
@@ -125,8 +215,8 @@ int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t 
     if (a.t_dtype == OFQ_F16) return launch_plain<f16, MfmaF16>(st, a, workspace);
     return launch_plain<bf16, MfmaBF16>(st, a, workspace);
   }
-  if (a.t_dtype == OFQ_F16) return launch_wq_t<f16, MfmaF16>(st, a);
-  return launch_wq_t<bf16, MfmaBF16>(st, a);
+  if (a.t_dtype == OFQ_F16) return launch_wq_t<f16, MfmaF16>(st, a, nullptr, 1);
+  return launch_wq_t<bf16, MfmaBF16>(st, a, nullptr, 1);
 }
 
 }  // namespace ofq

@@ -91,6 +91,22 @@ struct EpBias {
     return o;
   }
   typedef T elem_t;
+  static constexpr bool kSplit = false;
+};
+// Split-K: the block's fp32 partial sums go to slice blockIdx.y of a [splits, M, N] workspace;
+// a second kernel adds the slices in order and applies the real epilogue.
+struct EpPartial {
+  struct Params {
+    float* out;
+  };
+  static __device__ __forceinline__ void convert4(const Params&, const float* acc, int,
+                                                  float* out4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out4[e] = acc[e];
+  }
+  static __device__ __forceinline__ float convert1(const Params&, float acc, int) { return acc; }
+  typedef float elem_t;
+  static constexpr bool kSplit = true;
 };
 template<typename T>
 struct EpScale {
@@ -136,6 +152,7 @@ struct EpScale {
     return o;
   }
   typedef T elem_t;
+  static constexpr bool kSplit = false;
 };
 
 // =================================================================================================
@@ -246,7 +263,6 @@ struct B2Dequant {
   // dequantise and store a quarter of the thread's chunks (all of them when there are fewer)
   static __device__ __forceinline__ void store_part(const Params&, const Regs& r, uint8_t* lds,
                                                     int tid, int part) {
-    typedef typename TT<T>::storage S;
 #pragma unroll
     for (int i = 0; i < kChunks; ++i) {
       if ((kChunks >= 4 ? (i & 3) : (i * (4 / kChunks))) != part) continue;
@@ -266,20 +282,10 @@ struct B2Dequant {
         *reinterpret_cast<u32x4*>(rowp + (((2 * c) ^ sw) << 4)) = o0;
         *reinterpret_cast<u32x4*>(rowp + (((2 * c + 1) ^ sw) << 4)) = o1;
       } else {
-        S vals[32];
-#pragma unroll
-        for (int e = 0; e < 32; ++e) {
-          const uint32_t b = (r.v[i][e >> 3] >> (((e >> 1) & 3) * 8)) & 0xFFu;
-          const int nib = (e & 1) ? (b & 0xF) : (b >> 4);
-          const int code = SIGNED ? ((nib ^ 8) - 8) : nib;
-          float v = TT<T>::round((float)code * sc);
-          if (ZMODE != 0) v = v + zc;
-          TT<T>::store(&vals[e], v);
-        }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           *reinterpret_cast<u32x4*>(rowp + (((4 * c + j) ^ sw) << 4)) =
-              reinterpret_cast<const u32x4*>(vals)[j];
+              dequant8_b4<T, SIGNED, ZMODE>(r.v[i][j], sc, zc);
       }
     }
   }
@@ -291,13 +297,20 @@ struct B2Dequant {
 template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2, int DBG = 0>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
-           typename EP::Params ep, int M, int N, int KT, int m_tiles, int n_tiles) {
+           typename EP::Params ep, int M, int N, int KT_total, int kt_split, int m_tiles,
+           int n_tiles) {
   constexpr int NWAVES = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int kABytes = BM * kStageRow;
   constexpr int kStage = (BM + BN) * kStageRow;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  // split-K: blockIdx.y owns k-tiles [kt_base, kt_base + KT); tile t below is the block's t-th
+  const int kt_base = EP::kSplit ? (int)blockIdx.y * kt_split : 0;
+  const int KT = EP::kSplit ? (KT_total - kt_base < kt_split ? KT_total - kt_base : kt_split)
+                            : KT_total;
+  if (EP::kSplit) ep.out += (int64_t)blockIdx.y * M * N;
 
   const int nblocks = m_tiles * n_tiles;
   int logical;
@@ -333,17 +346,17 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
   constexpr int kCopyOps = BM / (8 * NWAVES) + (BP::kDirect ? BN / (8 * NWAVES) : 0);
   auto stage_of = [&](int t) { return lds + (t % NSTAGE) * kStage; };
   auto issue_copies = [&](int t, typename BP::Regs& regs) {
-    async_tile<BM, NWAVES>(A, lda, m0, M, t, stage_of(t), wave, lane);
-    if (BP::kDirect) BP::load(bp, n0, t, wave, lane, tid, regs, stage_of(t) + kABytes);
+    async_tile<BM, NWAVES>(A, lda, m0, M, kt_base + t, stage_of(t), wave, lane);
+    if (BP::kDirect) BP::load(bp, n0, kt_base + t, wave, lane, tid, regs, stage_of(t) + kABytes);
   };
 
   // ---- prologue: tile 0 complete in its stage, copies of tiles 1..D-1 and the codes of tile 1
   //      in flight --------------------------------------------------------------------------------
   if (!BP::kDirect) {
-    BP::load(bp, n0, 0, wave, lane, tid, breg0, nullptr);
+    BP::load(bp, n0, kt_base, wave, lane, tid, breg0, nullptr);
 #pragma unroll
     for (int part = 0; part < 4; ++part) BP::store_part(bp, breg0, lds + kABytes, tid, part);
-    if (KT > 1) BP::load(bp, n0, 1, wave, lane, tid, breg1, nullptr);
+    if (KT > 1) BP::load(bp, n0, kt_base + 1, wave, lane, tid, breg1, nullptr);
   }
   issue_copies(0, breg0);
   wait_vmem_all();
@@ -371,7 +384,7 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
   auto iteration = [&](int kt, typename BP::Regs& st_regs, typename BP::Regs& ld_regs) {
     const bool more_copies = DBG != 2 && kt + D < KT;
     if (DBG != 2 && !BP::kDirect && kt + 2 < KT)
-      BP::load(bp, n0, kt + 2, wave, lane, tid, ld_regs, nullptr);
+      BP::load(bp, n0, kt_base + kt + 2, wave, lane, tid, ld_regs, nullptr);
     if (more_copies) issue_copies(kt + D, ld_regs);
     uint8_t* cur = stage_of(kt);
     uint8_t* nxt = stage_of(kt + 1);
@@ -510,7 +523,8 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
 
 template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2, int DBG = 0>
 int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::Params& bp,
-                 const typename EP::Params& ep, int64_t M, int64_t N, int64_t KT) {
+                 const typename EP::Params& ep, int64_t M, int64_t N, int64_t KT,
+                 int splits = 1) {
   const int m_tiles = (int)((M + BM - 1) / BM);
   const int n_tiles = (int)((N + BN - 1) / BN);
   // the stages; the epilogue stages its output panels in the same memory
@@ -527,8 +541,12 @@ int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::
       attr_set = true;
     }
   }
-  kern<<<m_tiles * n_tiles, WM * WN * 64, lds_bytes, st>>>(
-      static_cast<const uint8_t*>(A), lda, bp, ep, (int)M, (int)N, (int)KT, m_tiles, n_tiles);
+  if (splits < 1 || (splits > 1 && !EP::kSplit)) return OFQ_ERR_UNSUPPORTED;
+  const int kt_split = (int)((KT + splits - 1) / splits);
+  if ((int64_t)kt_split * (splits - 1) >= KT) return OFQ_ERR_UNSUPPORTED;  // an empty slice
+  kern<<<dim3(m_tiles * n_tiles, splits), WM * WN * 64, lds_bytes, st>>>(
+      static_cast<const uint8_t*>(A), lda, bp, ep, (int)M, (int)N, (int)KT, kt_split, m_tiles,
+      n_tiles);
   return ofq_check_launch();
 }
 

@@ -245,3 +245,45 @@ def test_prefill_with_and_without_workspace():
         # a too-small workspace falls back to the in-tile path: identical to passing none
         assert np.array_equal(outs[1], outs[2])
         assert H.rel_l2(O.to_f32(outs[0]), O.to_f32(outs[1])) < 1e-3
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 300, 1024), (100, 203, 1536), (130, 520, 2048),
+                                   (128, 1000, 4096), (300, 384, 1024)])
+@pytest.mark.parametrize("num_bits", [4, 8])
+def test_midsize_m_split_k(m, n, k, num_bits):
+    """16 < m < 1024 with few output tiles: given the workspace the op cuts K into slices that run
+    as separate blocks and folds their fp32 partial sums; without it one block walks all of K.
+    Both meet the contract and agree with each other up to summation order.  n not a multiple of
+    4 takes the scalar fold."""
+    import torch
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    g = 64
+    rng = np.random.Generator(np.random.PCG64(m * 7 + n + num_bits))
+    for t, tcode in (("bf16", _lib.BF16), ("f16", _lib.F16)):
+        x = H.as_T(rng.standard_normal((m, k)).astype(np.float32) / 4, t)
+        wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+        b = H.as_T(rng.standard_normal(n).astype(np.float32) / 10, t)
+        for symmetric, qdt in VARIANTS:
+            w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, g, qdt, t)
+            wcode = _lib.I8 if qdt == np.int8 else _lib.U8
+            need = L.ofq_fused_linear_gq_workspace_bytes(wcode, tcode, num_bits, int(symmetric), 1,
+                                                         g, m, n, k)
+            assert need > 0 and need % (m * n * 4) == 0 and need // (m * n * 4) >= 2, need
+            ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+            xt, wt, st, bt = map(H.to_torch, (x, w, scale, b))
+            zt = H.to_torch(zero)
+            outs = []
+            for wptr, wbytes in ((ws.data_ptr(), need), (None, 0)):
+                out = torch.empty((m, n), dtype=xt.dtype, device="cuda")
+                rc = L.ofq_fused_linear_gq(torch.cuda.current_stream().cuda_stream, xt.data_ptr(),
+                                           wt.data_ptr(), st.data_ptr(),
+                                           zt.data_ptr() if zt is not None else None, bt.data_ptr(),
+                                           out.data_ptr(), wcode, tcode, num_bits, int(symmetric), 1,
+                                           g, m, n, k, wptr, wbytes)
+                assert rc == 0
+                outs.append(H.to_numpy(out))
+            ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+            for got in outs:
+                H.assert_linear_parity(got, ref, t, f"m={m} n={n} k={k} {t} {symmetric} {qdt}")
+            assert H.rel_l2(O.to_f32(outs[0]), O.to_f32(outs[1])) < 1e-3
