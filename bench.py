@@ -332,6 +332,20 @@ def secondary(L, _lib, torch, dev, args):
         "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gb / HBM_PEAK_GBPS, 4)}}
 
+    def sln():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_fused_skip_layer_norm_min_max_observer(
+            cs(), xs[i].data_ptr(), None, xs[(i + 1) % reps].data_ptr(), 1.0, gamma.data_ptr(),
+            beta.data_ptr(), ys[i].data_ptr(), s.data_ptr(), z.data_ptr(), _lib.F16, m, k, 1e-5, 8,
+            ws.data_ptr(), m * 4), "skip_ln_observer")
+    us = timeit(sln, iters=40)
+    gb = (3 * m * k * 2) / (us * 1e-6) / 1e9
+    out["skip_layer_norm_observer_f16_2048x4096"] = {
+        "us": round(us, 2), "gbps": round(gb, 1),
+        "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+
     def qz():
         i = it[0] % reps
         it[0] += 1

@@ -175,6 +175,20 @@ int ofq_fused_layer_norm_min_max_observer(void* stream, const void* x, const voi
                                           void* workspace, size_t workspace_bytes);
 
 /*
+ * fused_skip_layer_norm_min_max_observer: the op above on the input of skip_layer_norm,
+ *   oneflow/user/kernels/skip_layer_norm_kernel.cu:36-67 (functional signature
+ *   oneflow/core/functional/functional_api.yaml:1545-1546): the row that is normalised is
+ *   (x + bias[c]) + skip * T(alpha), every operation in t_dtype; bias ([cols]) and skip
+ *   ([rows, cols]) may each be NULL and then enter as zero.  Workspace as above.
+ */
+int ofq_fused_skip_layer_norm_min_max_observer(void* stream, const void* x, const void* bias,
+                                               const void* skip, double alpha, const void* gamma,
+                                               const void* beta, void* y, float* scale,
+                                               float* zero_point, int t_dtype, int64_t rows,
+                                               int64_t cols, double epsilon, int quantization_bit,
+                                               void* workspace, size_t workspace_bytes);
+
+/*
  * groupwise_quantize: the producer of the weight format of the two ops above.
  * The reference defines that format only through the helpers of its own test,
  *   python/oneflow/test/modules/test_groupwise_quantization.py:26-35 (int4 packing) and :46-81

@@ -6,6 +6,9 @@
 // var = max(M2/n, 0), inv = rsqrt(var + eps); the normalised value is rounded to T first and the
 // affine `* gamma + beta` is then carried out in T (two more roundings).
 // Observer (oneflow/user/kernels/min_max_observer_kernel.cu:117-131): scale = absmax / (2^(b-1)-1).
+// With SKIP the normalised input is that of skip_layer_norm
+// (oneflow/user/kernels/skip_layer_norm_kernel.cu:36-67): (x + bias[c]) + skip * T(alpha), every
+// operation rounded to T, an absent bias or skip entering as zero.
 //
 // Rows of up to 4096 elements: one WAVE per row.  The row is read from HBM once (128-bit loads,
 // 1 KB per wave instruction) and kept in registers for the three uses (sum, squared deviations,
@@ -53,14 +56,27 @@ __device__ __forceinline__ void store8(typename TT<T>::storage* p, const float* 
   }
 }
 
+// the residual inputs of skip_layer_norm; alpha already rounded to T
+template<typename T>
+struct SkipArgs {
+  const typename TT<T>::storage* bias;  // [cols] or null
+  const typename TT<T>::storage* skip;  // [rows, cols] or null
+  float alpha;
+};
+
+template<typename T>
+__device__ __forceinline__ float skip_sum(float x, float b, float s, float alpha) {
+  return TT<T>::round(TT<T>::round(x + b) + TT<T>::round(s * alpha));
+}
+
 // NP = packs of 8 elements each lane caches; cols <= kLnBlock * 8 * NP and 8 | cols.
-template<typename T, int NP>
+template<typename T, int NP, bool SKIP>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
                  const typename TT<T>::storage* __restrict__ gamma,
                  const typename TT<T>::storage* __restrict__ beta,
                  typename TT<T>::storage* __restrict__ y, float* __restrict__ row_absmax,
-                 int64_t cols, float eps) {
+                 int64_t cols, float eps, SkipArgs<T> sk) {
   __shared__ float smem[kLnBlock / kWave];
   const int64_t row = blockIdx.x;
   const typename TT<T>::storage* xr = x + row * cols;
@@ -73,6 +89,14 @@ ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
     const int p = threadIdx.x + i * kLnBlock;
     if (p < npacks) {
       load8<T>(xr + (int64_t)p * 8, v[i]);
+      if (SKIP) {
+        float bb[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float ss[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (sk.bias) load8<T>(sk.bias + (int64_t)p * 8, bb);
+        if (sk.skip) load8<T>(sk.skip + row * cols + (int64_t)p * 8, ss);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = skip_sum<T>(v[i][e], bb[e], ss[e], sk.alpha);
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) sum += v[i][e];
     }
@@ -152,18 +176,38 @@ __device__ __forceinline__ void widen(const RawPack<T>& r, float* f) {
   }
 }
 
+template<typename T>
+__device__ __forceinline__ RawPack<T> narrow(const float* f) {
+  RawPack<T> r;
+  if constexpr (TT<T>::dtype == OFQ_F16) {
+    f16x8 h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = (f16)f[i];
+    r.q[0] = __builtin_bit_cast(u32x4, h);
+  } else if constexpr (TT<T>::dtype == OFQ_BF16) {
+    u16x8 h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = float_to_bf16(f[i]);
+    r.q[0] = __builtin_bit_cast(u32x4, h);
+  } else {
+    r.q[0] = __builtin_bit_cast(u32x4, f32x4{f[0], f[1], f[2], f[3]});
+    r.q[sizeof(r.q) / 16 - 1] = __builtin_bit_cast(u32x4, f32x4{f[4], f[5], f[6], f[7]});
+  }
+  return r;
+}
+
 // One wave per row; NP = packs of 8 elements each lane caches: cols <= 64 * 8 * NP and 8 | cols.
 // A wave walks rows gw, gw + nwaves, ... and leaves the absmax over all of them in wave_absmax[gw].
 // x, gamma and beta are all requested before anything is waited for and stay in registers in
 // storage format (half the registers of fp32 for the 16-bit types), so the row's critical path
 // holds one memory round trip, not two.
-template<typename T, int NP>
+template<typename T, int NP, bool SKIP>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
                       const typename TT<T>::storage* __restrict__ gamma,
                       const typename TT<T>::storage* __restrict__ beta,
                       typename TT<T>::storage* __restrict__ y, float* __restrict__ wave_absmax,
-                      int64_t rows, int64_t cols, float eps) {
+                      int64_t rows, int64_t cols, float eps, SkipArgs<T> sk) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t gw = (int64_t)blockIdx.x * (kLnBlock / kWave) + (threadIdx.x >> 6);
   const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / kWave);
@@ -179,6 +223,33 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
     for (int i = 0; i < NP; ++i) {
       const int p = lane + i * kWave;
       if (p < npacks) v[i] = load_raw<T>(xr + (int64_t)p * 8);
+    }
+    if (SKIP) {
+      // the residual sum, rounded to T, takes the place of x in the registers
+      RawPack<T> sr[NP], bb[NP];
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const int p = lane + i * kWave;
+        if (p < npacks) {
+          if (sk.skip) sr[i] = load_raw<T>(sk.skip + row * cols + (int64_t)p * 8);
+          if (sk.bias) bb[i] = load_raw<T>(sk.bias + (int64_t)p * 8);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const int p = lane + i * kWave;
+        if (p < npacks) {
+          float fx[8], fb[8], fs[8], o[8];
+          widen<T>(v[i], fx);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) fb[e] = fs[e] = 0.f;
+          if (sk.bias) widen<T>(bb[i], fb);
+          if (sk.skip) widen<T>(sr[i], fs);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] = skip_sum<T>(fx[e], fb[e], fs[e], sk.alpha);
+          v[i] = narrow<T>(o);
+        }
+      }
     }
     if (first) {
 #pragma unroll
@@ -268,24 +339,31 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
 
 // any cols: three passes over the row through L2 (the row was just read, so only the first
 // pass touches HBM), scalar accesses.
-template<typename T>
+template<typename T, bool SKIP>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_rows_generic(const typename TT<T>::storage* __restrict__ x,
                          const typename TT<T>::storage* __restrict__ gamma,
                          const typename TT<T>::storage* __restrict__ beta,
                          typename TT<T>::storage* __restrict__ y, float* __restrict__ row_absmax,
-                         int64_t cols, float eps) {
+                         int64_t cols, float eps, SkipArgs<T> sk) {
   __shared__ float smem[kLnBlock / kWave];
   const int64_t row = blockIdx.x;
   const typename TT<T>::storage* xr = x + row * cols;
   typename TT<T>::storage* yr = y + row * cols;
+  auto input = [&](int64_t c) {
+    const float xv = TT<T>::load(xr + c);
+    if (!SKIP) return xv;
+    const float bv = sk.bias ? TT<T>::load(sk.bias + c) : 0.f;
+    const float sv = sk.skip ? TT<T>::load(sk.skip + row * cols + c) : 0.f;
+    return skip_sum<T>(xv, bv, sv, sk.alpha);
+  };
   float sum = 0.0f;
-  for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) sum += TT<T>::load(xr + c);
+  for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) sum += input(c);
   sum = block_reduce(sum, OpSum(), smem);
   const float mean = sum / (float)cols;
   float m2 = 0.0f;
   for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
-    const float d = TT<T>::load(xr + c) - mean;
+    const float d = input(c) - mean;
     m2 = __builtin_fmaf(d, d, m2);
   }
   m2 = block_reduce(m2, OpSum(), smem);
@@ -293,7 +371,7 @@ ln_observer_rows_generic(const typename TT<T>::storage* __restrict__ x,
   const float inv = 1.0f / __builtin_sqrtf(var + eps);
   float amax = 0.0f;
   for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
-    float t = TT<T>::round((TT<T>::load(xr + c) - mean) * inv);
+    float t = TT<T>::round((input(c) - mean) * inv);
     if (gamma) t = TT<T>::round(t * TT<T>::load(gamma + c));
     if (beta) t = TT<T>::round(t + TT<T>::load(beta + c));
     TT<T>::store(yr + c, t);
@@ -323,18 +401,39 @@ ln_observer_finalize(const float* __restrict__ part, int64_t n, int bits,
   }
 }
 
+// host-side rounding of a float to T (round to nearest even)
 template<typename T>
+float round_to_T_host(float v) {
+  if (TT<T>::dtype == OFQ_F16) return (float)(_Float16)v;
+  if (TT<T>::dtype == OFQ_BF16) {
+    uint32_t u;
+    __builtin_memcpy(&u, &v, 4);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return v;  // NaN stays NaN
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    u &= 0xFFFF0000u;
+    __builtin_memcpy(&v, &u, 4);
+    return v;
+  }
+  return v;
+}
+
+template<typename T, bool SKIP>
 int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, void* y,
            float* scale, float* zero_point, int64_t rows, int64_t cols, float eps, int bits,
-           float* ws) {
+           float* ws, const void* bias, const void* skip, double alpha) {
   typedef typename TT<T>::storage S;
   const S* xs = static_cast<const S*>(x);
   const S* gs = static_cast<const S*>(gamma);
   const S* bs = static_cast<const S*>(beta);
   S* ys = static_cast<S*>(y);
+  SkipArgs<T> sk;
+  sk.bias = static_cast<const S*>(bias);
+  sk.skip = static_cast<const S*>(skip);
+  // T(alpha): the reference casts its float alpha to T (skip_layer_norm_kernel.cu:36,62)
+  sk.alpha = round_to_T_host<T>((float)alpha);
   const bool vec_ok = cols % 8 == 0 && ofq_aligned16(x) && ofq_aligned16(y)
-                      && ofq_aligned16(gamma) && ofq_aligned16(beta)
-                      && (cols * sizeof(S)) % 16 == 0;
+                      && ofq_aligned16(gamma) && ofq_aligned16(beta) && ofq_aligned16(bias)
+                      && ofq_aligned16(skip) && (cols * sizeof(S)) % 16 == 0;
   const int64_t npacks = cols / 8;
   int64_t nparts = rows;
   constexpr int kWavesPerBlock = kLnBlock / kWave;
@@ -346,8 +445,9 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
     const int64_t waves = rows < 256 * 4 ? rows : 256 * 4;
     const int grid = (int)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
     nparts = (int64_t)grid * kWavesPerBlock < rows ? (int64_t)grid * kWavesPerBlock : rows;
-#define OFQ_LN_WAVE(NPV)                                                                  \
-  ln_observer_wave_rows<T, NPV><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, cols, eps)
+#define OFQ_LN_WAVE(NPV)                                                                       \
+  ln_observer_wave_rows<T, NPV, SKIP><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, cols, \
+                                                                 eps, sk)
     if (npacks <= kWave) {
       OFQ_LN_WAVE(1);
     } else if (npacks <= 2 * kWave) {
@@ -359,16 +459,45 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
     }
 #undef OFQ_LN_WAVE
   } else if (vec_ok && npacks <= kLnBlock) {
-    ln_observer_rows<T, 1><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+    ln_observer_rows<T, 1, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else if (vec_ok && npacks <= 2 * kLnBlock) {
-    ln_observer_rows<T, 2><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+    ln_observer_rows<T, 2, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else if (vec_ok && npacks <= 4 * kLnBlock) {
-    ln_observer_rows<T, 4><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+    ln_observer_rows<T, 4, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else {
-    ln_observer_rows_generic<T><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps);
+    ln_observer_rows_generic<T, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols,
+                                                                      eps, sk);
   }
   ln_observer_finalize<<<1, kWave, 0, st>>>(ws, nparts, bits, scale, zero_point);
   return ofq_check_launch();
+}
+
+int run(void* stream, const void* x, const void* bias, const void* skip, double alpha,
+        bool with_skip, const void* gamma, const void* beta, void* y, float* scale,
+        float* zero_point, int t_dtype, int64_t rows, int64_t cols, double epsilon,
+        int quantization_bit, void* workspace, size_t workspace_bytes) {
+  OFQ_RETURN_IF(quantization_bit <= 1 || quantization_bit > 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(t_dtype != OFQ_F16 && t_dtype != OFQ_BF16 && t_dtype != OFQ_F32,
+                OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(rows < 1 || cols < 1 || rows > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(x == nullptr || y == nullptr || scale == nullptr || zero_point == nullptr,
+                OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(workspace == nullptr || workspace_bytes < (size_t)rows * sizeof(float),
+                OFQ_ERR_WORKSPACE);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  const float eps = (float)epsilon;
+#define OFQ_LN_RUN(T)                                                                          \
+  return with_skip ? launch<T, true>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps, \
+                                     quantization_bit, ws, bias, skip, alpha)                  \
+                   : launch<T, false>(st, x, gamma, beta, y, scale, zero_point, rows, cols,    \
+                                      eps, quantization_bit, ws, nullptr, nullptr, 0.0)
+  switch (t_dtype) {
+    case OFQ_F16: OFQ_LN_RUN(f16);
+    case OFQ_BF16: OFQ_LN_RUN(bf16);
+    default: OFQ_LN_RUN(float);
+  }
+#undef OFQ_LN_RUN
 }
 
 }  // namespace
@@ -385,26 +514,15 @@ extern "C" int ofq_fused_layer_norm_min_max_observer(void* stream, const void* x
                                                      int64_t rows, int64_t cols, double epsilon,
                                                      int quantization_bit, void* workspace,
                                                      size_t workspace_bytes) {
-  OFQ_RETURN_IF(quantization_bit <= 1 || quantization_bit > 8, OFQ_ERR_BAD_ATTR);
-  OFQ_RETURN_IF(t_dtype != OFQ_F16 && t_dtype != OFQ_BF16 && t_dtype != OFQ_F32,
-                OFQ_ERR_BAD_DTYPE);
-  OFQ_RETURN_IF(rows < 1 || cols < 1 || rows > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
-  OFQ_RETURN_IF(x == nullptr || y == nullptr || scale == nullptr || zero_point == nullptr,
-                OFQ_ERR_NULL_POINTER);
-  OFQ_RETURN_IF(workspace == nullptr || workspace_bytes < (size_t)rows * sizeof(float),
-                OFQ_ERR_WORKSPACE);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  float* ws = static_cast<float*>(workspace);
-  const float eps = (float)epsilon;
-  switch (t_dtype) {
-    case OFQ_F16:
-      return ofq::launch<ofq::f16>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps,
-                                   quantization_bit, ws);
-    case OFQ_BF16:
-      return ofq::launch<ofq::bf16>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps,
-                                    quantization_bit, ws);
-    default:
-      return ofq::launch<float>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps,
-                                quantization_bit, ws);
-  }
+  return ofq::run(stream, x, nullptr, nullptr, 0.0, false, gamma, beta, y, scale, zero_point,
+                  t_dtype, rows, cols, epsilon, quantization_bit, workspace, workspace_bytes);
+}
+
+extern "C" int ofq_fused_skip_layer_norm_min_max_observer(
+    void* stream, const void* x, const void* bias, const void* skip, double alpha,
+    const void* gamma, const void* beta, void* y, float* scale, float* zero_point, int t_dtype,
+    int64_t rows, int64_t cols, double epsilon, int quantization_bit, void* workspace,
+    size_t workspace_bytes) {
+  return ofq::run(stream, x, bias, skip, alpha, true, gamma, beta, y, scale, zero_point, t_dtype,
+                  rows, cols, epsilon, quantization_bit, workspace, workspace_bytes);
 }

@@ -363,6 +363,41 @@ def fused_layer_norm_min_max_observer(x, gamma=None, beta=None, epsilon=1e-5, qu
     return y, scale, zero_point
 
 
+def fused_skip_layer_norm_min_max_observer(x, gamma=None, beta=None, bias=None, skip=None,
+                                           epsilon=1e-5, alpha=1e1, quantization_bit=8):
+    """``skip_layer_norm`` (same arguments and defaults as the reference functional,
+    functional_api.yaml:1545-1546: the row normalised is ``(x + bias) + skip * alpha`` in the
+    dtype of x) + per-tensor symmetric observer of the result.  Returns
+    ``(y, scale, zero_point)``."""
+    _check(1 < quantization_bit <= 8, "quantization_bit should be in range (1, 8].")
+    _check(x.dtype in (torch.float16, torch.bfloat16, torch.float32),
+           f"no fused_skip_layer_norm_min_max_observer kernel for dtype {x.dtype}")
+    _check(x.dim() >= 2, "number of axes of x should be greater than or equal to 2")
+    cols = x.shape[-1]
+    for name, p in (("gamma", gamma), ("beta", beta), ("bias", bias)):
+        if p is not None:
+            _check(p.dtype == x.dtype and p.dim() == 1 and p.numel() == cols,
+                   f"{name} should be 1-D with the dtype of x and x.shape[-1] elements")
+    if skip is not None:
+        _check(skip.dtype == x.dtype and tuple(skip.shape) == tuple(x.shape),
+               "skip should have the shape and dtype of x")
+    _require_gpu(x, gamma, beta, bias, skip)
+    x, gamma, beta, bias, skip = map(_contig, (x, gamma, beta, bias, skip))
+    rows = x.numel() // cols
+    y = torch.empty_like(x)
+    scale = torch.empty(1, dtype=torch.float32, device=x.device)
+    zero_point = torch.empty(1, dtype=torch.float32, device=x.device)
+    L = _lib.lib()
+    ws_bytes = L.ofq_fused_layer_norm_min_max_observer_workspace_bytes(_dt(x), rows, cols)
+    ws = _workspace(ws_bytes, x.device)
+    st = L.ofq_fused_skip_layer_norm_min_max_observer(
+        _stream(x), _ptr(x), _ptr(bias), _ptr(skip), float(alpha), _ptr(gamma), _ptr(beta),
+        _ptr(y), _ptr(scale), _ptr(zero_point), _dt(x), rows, cols, float(epsilon),
+        quantization_bit, _ptr(ws), ws_bytes)
+    _lib.check("ofq_fused_skip_layer_norm_min_max_observer", st)
+    return y, scale, zero_point
+
+
 def matmul_quant(a, b, a_scale, b_scale, bias=None, out_dtype=torch.float16):
     """int8 ``a[m,k]`` x int8 ``b[n,k]`` -> ``out_dtype[m,n]``; exact int32 accumulation, then
     ``acc * (a_scale * b_scale[n]) + bias[n]``."""

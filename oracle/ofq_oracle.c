@@ -493,17 +493,34 @@ int ofq_ref_fused_linear(const void* x, const void* w, const void* scale, const 
  * Observer: per-tensor symmetric, scale = absmax(y) / (2^(b-1)-1) as one fp32 divide
  *   (min_max_observer_kernel.cpp:22-34 applied to the T-rounded y), zero_point = 0.
  * ---------------------------------------------------------------------------------------- */
-int ofq_ref_layer_norm_min_max_observer(const void* x, const void* gamma, const void* beta,
-                                        void* y, float* scale, float* zero_point, int64_t rows,
-                                        int64_t cols, double eps, int t, int bits) {
+/* The input of the normalisation with the optional residual of skip_layer_norm
+ * (user/kernels/skip_layer_norm_kernel.cu:36-67): (x + bias[c]) + skip * T(alpha), every
+ * operation in T; an absent bias or skip enters as zero, exactly as there. */
+static float skip_input(const void* x, const void* bias, const void* skip, float alpha_t,
+                        int64_t r, int64_t c, int64_t cols, int t, int with_skip) {
+  const float xv = t_load(x, r * cols + c, t);
+  if (!with_skip) return xv;
+  const float bv = bias ? t_load(bias, c, t) : 0.0f;
+  const float sv = skip ? t_load(skip, r * cols + c, t) : 0.0f;
+  const float a = t_round(xv + bv, t);
+  const float b = t_round(sv * alpha_t, t);
+  return t_round(a + b, t);
+}
+
+static int layer_norm_observer_impl(const void* x, const void* bias, const void* skip,
+                                    double alpha, int with_skip, const void* gamma,
+                                    const void* beta, void* y, float* scale, float* zero_point,
+                                    int64_t rows, int64_t cols, double eps, int t, int bits) {
   float absmax = 0.0f;
+  const float alpha_t = t_round((float)alpha, t);
   for (int64_t r = 0; r < rows; ++r) {
     double sum = 0.0;
-    for (int64_t c = 0; c < cols; ++c) sum += (double)t_load(x, r * cols + c, t);
+    for (int64_t c = 0; c < cols; ++c)
+      sum += (double)skip_input(x, bias, skip, alpha_t, r, c, cols, t, with_skip);
     const double mean = sum / (double)cols;
     double m2 = 0.0;
     for (int64_t c = 0; c < cols; ++c) {
-      const double d = (double)t_load(x, r * cols + c, t) - mean;
+      const double d = (double)skip_input(x, bias, skip, alpha_t, r, c, cols, t, with_skip) - mean;
       m2 += d * d;
     }
     double var = m2 / (double)cols;
@@ -511,7 +528,8 @@ int ofq_ref_layer_norm_min_max_observer(const void* x, const void* gamma, const 
     const float mean_f = (float)mean;
     const float inv_f = (float)(1.0 / sqrt(var + eps));
     for (int64_t c = 0; c < cols; ++c) {
-      const float xn = t_round((t_load(x, r * cols + c, t) - mean_f) * inv_f, t);
+      const float xin = skip_input(x, bias, skip, alpha_t, r, c, cols, t, with_skip);
+      const float xn = t_round((xin - mean_f) * inv_f, t);
       float v = xn;
       if (gamma) v = t_round(v * t_load(gamma, c, t), t);
       if (beta) v = t_round(v + t_load(beta, c, t), t);
@@ -524,6 +542,23 @@ int ofq_ref_layer_norm_min_max_observer(const void* x, const void* gamma, const 
   *scale = absmax / denominator;
   *zero_point = 0.0f;
   return 0;
+}
+
+int ofq_ref_layer_norm_min_max_observer(const void* x, const void* gamma, const void* beta,
+                                        void* y, float* scale, float* zero_point, int64_t rows,
+                                        int64_t cols, double eps, int t, int bits) {
+  return layer_norm_observer_impl(x, NULL, NULL, 0.0, 0, gamma, beta, y, scale, zero_point, rows,
+                                  cols, eps, t, bits);
+}
+
+/* fused_skip_layer_norm_min_max_observer: the same with the input of skip_layer_norm. */
+int ofq_ref_skip_layer_norm_min_max_observer(const void* x, const void* bias, const void* skip,
+                                             double alpha, const void* gamma, const void* beta,
+                                             void* y, float* scale, float* zero_point,
+                                             int64_t rows, int64_t cols, double eps, int t,
+                                             int bits) {
+  return layer_norm_observer_impl(x, bias, skip, alpha, 1, gamma, beta, y, scale, zero_point,
+                                  rows, cols, eps, t, bits);
 }
 
 /* quantization with a low-precision input and int8 codes (the dynamic activation path): the

@@ -63,6 +63,11 @@ int ofq_ref_fused_linear(const void* x, const void* w, const void* scale, const 
 int ofq_ref_layer_norm_min_max_observer(const void* x, const void* gamma, const void* beta,
                                         void* y, float* scale, float* zero_point, int64_t rows,
                                         int64_t cols, double eps, int t, int bits);
+int ofq_ref_skip_layer_norm_min_max_observer(const void* x, const void* bias, const void* skip,
+                                             double alpha, const void* gamma, const void* beta,
+                                             void* y, float* scale, float* zero_point,
+                                             int64_t rows, int64_t cols, double eps, int t,
+                                             int bits);
 
 int ofq_ref_quantize_to_int8(const void* in, const float* scale, int8_t* out, int64_t elem_cnt,
                              int64_t scale_size, int64_t shape0, int t, int bits);

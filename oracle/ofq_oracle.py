@@ -248,6 +248,26 @@ def layer_norm_min_max_observer(x, gamma, beta, eps=1e-5, quantization_bit=8):
     return y, scale, zp
 
 
+def skip_layer_norm_min_max_observer(x, gamma, beta, bias=None, skip=None, eps=1e-5, alpha=1e1,
+                                     quantization_bit=8):
+    """skip_layer_norm (skip_layer_norm_kernel.cu:36-67) followed by the per-tensor observer."""
+    x = _c(x)
+    gamma = _c(gamma)
+    beta = _c(beta)
+    bias = _c(bias)
+    skip = _c(skip)
+    cols = x.shape[-1]
+    rows = x.size // cols
+    y = np.empty_like(x)
+    scale = np.empty(1, dtype=np.float32)
+    zp = np.empty(1, dtype=np.float32)
+    rc = lib().ofq_ref_skip_layer_norm_min_max_observer(
+        _p(x), _p(bias), _p(skip), ctypes.c_double(alpha), _p(gamma), _p(beta), _p(y), _p(scale),
+        _p(zp), _i64(rows), _i64(cols), ctypes.c_double(eps), t_code(x), int(quantization_bit))
+    assert rc == 0
+    return y, scale, zp
+
+
 def quantize_to_int8(x, scale, quantization_bit=8):
     x = _c(x)
     scale = _c(scale, np.float32)

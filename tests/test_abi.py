@@ -87,7 +87,7 @@ def test_observer_and_quantization_argument_errors(lib):
     obs = lib.ofq_min_max_observer
     need = lib.ofq_min_max_observer_workspace_bytes(F32, 4096 * 4096, 4096)
     assert need == 4096 * 2 * 4
-    assert lib.ofq_min_max_observer_workspace_bytes(F64, 1 << 20, 1) == (1 << 20) // 16384 * 2 * 8
+    assert lib.ofq_min_max_observer_workspace_bytes(F64, 1 << 20, 1) == (1 << 20) // 4096 * 2 * 8
     assert obs(None, P, P, P, F32, 1024, 4, 9, 0, 0, P, 1 << 20) == BAD_ATTR
     assert obs(None, P, P, P, F32, 1024, 4, 1, 0, 0, P, 1 << 20) == BAD_ATTR
     assert obs(None, P, P, P, F32, 1024, 4, 8, 2, 0, P, 1 << 20) == BAD_ATTR
@@ -116,6 +116,11 @@ def test_layer_norm_and_matmul_quant_argument_errors(lib):
     assert ln(None, P, P, P, P, P, P, F16, 0, 64, 1e-5, 8, P, 64) == BAD_SHAPE
     assert ln(None, None, P, P, P, P, P, F16, 8, 64, 1e-5, 8, P, 64) == NULLP
     assert ln(None, P, P, P, P, P, P, F16, 8, 64, 1e-5, 8, P, 16) == WORKSPACE
+    sl = lib.ofq_fused_skip_layer_norm_min_max_observer
+    assert sl(None, P, P, P, 1.0, P, P, P, P, P, F16, 8, 64, 1e-5, 9, P, 64) == BAD_ATTR
+    assert sl(None, P, None, None, 1.0, P, P, P, P, P, U8, 8, 64, 1e-5, 8, P, 64) == BAD_DTYPE
+    assert sl(None, P, P, P, 1.0, P, P, None, P, P, F16, 8, 64, 1e-5, 8, P, 64) == NULLP
+    assert sl(None, P, P, P, 1.0, P, P, P, P, P, F16, 8, 64, 1e-5, 8, None, 0) == WORKSPACE
     mq = lib.ofq_matmul_quant
     assert mq(None, P, P, P, P, None, P, I8, 16, 16, 128) == BAD_DTYPE
     assert mq(None, P, P, P, P, None, P, F16, 16, 16, 0) == BAD_SHAPE

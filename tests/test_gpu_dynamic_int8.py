@@ -47,6 +47,46 @@ def test_layer_norm_observer(t, rows, cols):
     assert abs(float(H.to_numpy(s)[0]) - float(s_ref[0])) <= 2e-3 * float(s_ref[0])
 
 
+@pytest.mark.parametrize("t,rows,cols", [("f16", 2048, 4096), ("bf16", 300, 4096), ("f32", 33, 1000),
+                                         ("f16", 7, 8200), ("bf16", 5, 24), ("f32", 40, 2048),
+                                         ("bf16", 9, 16384)])
+@pytest.mark.parametrize("use_bias,use_skip", [(True, True), (False, True), (True, False)])
+def test_skip_layer_norm_observer(t, rows, cols, use_bias, use_skip):
+    """The residual input of skip_layer_norm in front of the same LayerNorm + observer: every
+    kernel variant (one wave per row, one block per row, scalar any-length rows)."""
+    import oneflow_amd as flow
+    x, gamma, beta = _cfg5_inputs(rows, cols, t)
+    bias = H.as_T((0.5 * H.rng_for(6, 0).standard_normal(cols)).astype(np.float32), t) if use_bias else None
+    skip = H.as_T(H.rng_for(6, 1).standard_normal((rows, cols)).astype(np.float32), t) if use_skip else None
+    alpha = 0.37
+    y_ref, s_ref, z_ref = O.skip_layer_norm_min_max_observer(x, gamma, beta, bias, skip, 1e-5, alpha, 8)
+    y, s, z = flow._C.fused_skip_layer_norm_min_max_observer(
+        H.to_torch(x), H.to_torch(gamma), H.to_torch(beta), H.to_torch(bias), H.to_torch(skip),
+        1e-5, alpha, 8)
+    y_np = H.to_numpy(y)
+    yf, yr = O.to_f32(y_np).astype(np.float64), O.to_f32(y_ref).astype(np.float64)
+    if t == "f32":
+        assert np.allclose(yf, yr, rtol=4e-6, atol=4e-6)
+    else:
+        mag = np.abs(yr) + np.abs(O.to_f32(beta).astype(np.float64))[None, :]
+        assert (np.abs(yf - yr) <= 2.0001 * H.ulp_of(mag, t)).all()
+        assert (yf != yr).mean() < 0.02
+    expect = np.float32(np.abs(O.to_f32(y_np)).max()) / np.float32(127.0)
+    assert H.to_numpy(s)[0] == expect and H.to_numpy(z)[0] == 0.0
+    assert abs(float(H.to_numpy(s)[0]) - float(s_ref[0])) <= 2e-3 * float(s_ref[0])
+
+
+def test_skip_layer_norm_without_residual_is_the_plain_op():
+    """bias = skip = None adds zeros: the same bits as fused_layer_norm_min_max_observer."""
+    import oneflow_amd as flow
+    x, gamma, beta = _cfg5_inputs(64, 4096, "f16")
+    a = flow._C.fused_layer_norm_min_max_observer(H.to_torch(x), H.to_torch(gamma), H.to_torch(beta), 1e-5, 8)
+    b = flow._C.fused_skip_layer_norm_min_max_observer(H.to_torch(x), H.to_torch(gamma), H.to_torch(beta),
+                                                       None, None, 1e-5, 1e1, 8)
+    for u, v in zip(a, b):
+        assert np.array_equal(H.to_numpy(u), H.to_numpy(v))
+
+
 def test_layer_norm_closed_form():
     """Rows of +-c have mean 0 and variance c^2: y = +-c/sqrt(c^2+eps) * gamma + beta."""
     import oneflow_amd as flow

@@ -308,6 +308,42 @@ def test_layer_norm_observer_closed_forms():
     assert np.array_equal(q, np.clip(np.rint(y.astype(np.float32) / s[0]), -128, 127).astype(np.int8))
 
 
+def test_skip_layer_norm_observer_against_the_reference_composition():
+    """The reference's own test defines skip_layer_norm as add(x, bias), add(., skip * alpha),
+    layer_norm (test_skip_layer_norm.py:37-64); the kernel does the three operations in T
+    (skip_layer_norm_kernel.cu:62-63).  The pinned LayerNorm oracle applied to that sum, formed
+    here with numpy in T, must give the same bits; a dropped alpha, a swapped bias/skip or an
+    unrounded intermediate would not."""
+    rng = np.random.default_rng(11)
+    rows, cols = 5, 96
+    for dt in (np.float16, np.float32):
+        x = rng.standard_normal((rows, cols)).astype(dt)
+        bias = rng.standard_normal(cols).astype(dt)
+        skip = rng.standard_normal((rows, cols)).astype(dt)
+        g = (1 + 0.1 * rng.standard_normal(cols)).astype(dt)
+        b = (0.1 * rng.standard_normal(cols)).astype(dt)
+        for alpha in (1e1, 0.3, 1e-5):
+            for use_bias, use_skip in ((True, True), (False, True), (True, False), (False, False)):
+                pre = x + (bias if use_bias else dt(0))
+                pre = (pre + ((skip if use_skip else np.zeros_like(skip)) * dt(alpha)).astype(dt)).astype(dt)
+                want = O.layer_norm_min_max_observer(pre, g, b, 1e-6, 8)
+                got = O.skip_layer_norm_min_max_observer(x, g, b, bias if use_bias else None,
+                                                         skip if use_skip else None, 1e-6, alpha, 8)
+                for a_, b_ in zip(got, want):
+                    assert np.array_equal(a_, b_)
+    # bf16: the same with the oracle's own bf16 rounding for the three operations
+    bits = O.f32_to_bf16_bits
+    xb = bits(rng.standard_normal((3, 64)).astype(np.float32))
+    sb = bits(rng.standard_normal((3, 64)).astype(np.float32))
+    bb = bits(rng.standard_normal(64).astype(np.float32))
+    r = lambda a: O.to_f32(bits(np.asarray(a, dtype=np.float32)))
+    pre = r(r(O.to_f32(xb) + O.to_f32(bb)) + r(O.to_f32(sb) * r(np.float32(0.3))))
+    want = O.layer_norm_min_max_observer(bits(pre), None, None, 1e-5, 8)
+    got = O.skip_layer_norm_min_max_observer(xb, None, None, bb, sb, 1e-5, 0.3, 8)
+    for a_, b_ in zip(got, want):
+        assert np.array_equal(a_, b_)
+
+
 def test_matmul_quant_exact_integer_accumulation():
     rng = np.random.default_rng(4)
     m, n, k = 7, 19, 4096

@@ -52,15 +52,17 @@ def test_registrations(plugin):
     plugin.ofq_plugin_observer_tmp_bytes.restype = ctypes.c_longlong
     shape = (ctypes.c_longlong * 2)(4096, 4096)
     assert plugin.ofq_plugin_observer_tmp_bytes(K_FLOAT, shape, 2, 0) == 4096 * 2 * 4
-    assert plugin.ofq_plugin_observer_tmp_bytes(K_FLOAT, shape, 2, 1) == 1024 * 2 * 4
-    # fused linear: a tmp_buffer for the dequantised weight at large m only
+    assert plugin.ofq_plugin_observer_tmp_bytes(K_FLOAT, shape, 2, 1) == (4096 * 4096 // 4096) * 2 * 4  # one (min, max) pair per 4096-element slice
+    # fused linear: a tmp_buffer for the dequantised weight at large m, for fp32 partial sums of
+    # K slices at mid-size m with few output tiles, none for decode
     ll = ctypes.c_longlong
     plugin.ofq_plugin_fused_linear_tmp_bytes.restype = ll
     plugin.ofq_plugin_fused_linear_tmp_bytes.argtypes = [ctypes.c_int] * 2 + [ll] * 3 + [ctypes.c_int] * 2 + [ll] * 2
     tmp = plugin.ofq_plugin_fused_linear_tmp_bytes
     assert tmp(K_BFLOAT16, K_UINT8, 2048, 11008, 4096, 8, 0, 1, 64) == 11008 * 4096 * 2
     assert tmp(K_FLOAT16, K_INT8, 1, 4096, 4096, 4, 1, 1, 128) == 0
-    assert tmp(K_FLOAT16, K_INT8, 128, 4096, 4096, 4, 1, 1, 128) == 0
+    assert tmp(K_FLOAT16, K_INT8, 128, 4096, 4096, 4, 1, 1, 128) == 8 * 128 * 4096 * 4
+    assert tmp(K_FLOAT16, K_INT8, 16, 4096, 4096, 4, 1, 1, 128) == 0
     assert tmp(K_FLOAT, K_UINT8, 2048, 4096, 4096, 8, 0, 1, 64) == 0
 
 
