@@ -204,6 +204,40 @@ def main():
                 "ms_per_step": round(wall_m / 10, 4), "gbps": round(gbps, 1),
                 "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                              "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
+        # the same step with the block's neighbouring ops fused: q/k/v as one grouped launch,
+        # o, gate|up as one launch plus the SiLU gating, down: 5 GEMV launches per layer, not 7
+        glu_y = torch.empty((max(M, 8), 11008), dtype=torch.float16, device=dev)
+        vp = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+        i64 = lambda v: (ctypes.c_int64 * len(v))(*v)
+
+        def step_fused(m=M):
+            stream = torch.cuda.current_stream().cuda_stream
+            for mats in layers:
+                qkv, o, gate, up, down = mats[0:3], mats[3], mats[4], mats[5], mats[6]
+                x4 = x_by_k[4096]
+                st = L.ofq_grouped_linear_gq(
+                    stream, 3, vp([x4] * 3), vp([q[3] for q in qkv]), vp([q[4] for q in qkv]), None,
+                    vp([q[5] for q in qkv]), vp([q[6] for q in qkv]), i64([m] * 3), i64([4096] * 3),
+                    i64([4096] * 3), _lib.I8, _lib.F16, 4, 1, 1, 128)
+                if st != 0:
+                    raise RuntimeError(f"ofq_grouped_linear_gq status {st}")
+                launch(o, m)
+                st = L.ofq_fused_glu_gq(stream, x4.data_ptr(), up[3].data_ptr(), up[4].data_ptr(), None,
+                                        up[5].data_ptr(), gate[3].data_ptr(), gate[4].data_ptr(), None,
+                                        gate[5].data_ptr(), glu_y.data_ptr(), up[6].data_ptr(),
+                                        gate[6].data_ptr(), 5, _lib.I8, _lib.F16, 4, 1, 1, 128, m,
+                                        11008, 4096)
+                if st != 0:
+                    raise RuntimeError(f"ofq_fused_glu_gq status {st}")
+                launch(down, m)
+        run_f = make_runner(step_fused)
+        _, wall_f = time_region(run_f, 10, 2)
+        gbps = (bytes_step + args.layers * M * 11008 * 2) / (wall_f / 10 * 1e-3) / 1e9
+        other[f"decode_w4a16_m{M}_grouped_qkv_and_glu"] = {
+            "ms_per_step": round(wall_f / 10, 4), "gbps": round(gbps, 1),
+            "launches_per_step": 6 * args.layers,
+            "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
         del layers
         torch.cuda.empty_cache()
         result["secondary"] = {**other, **secondary(L, _lib, torch, dev, args)}

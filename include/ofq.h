@@ -206,6 +206,52 @@ int ofq_groupwise_quantize(void* stream, const void* x, void* q, void* scale, vo
                            int64_t group_size, int64_t n, int64_t k);
 
 /*
+ * grouped linear with groupwise-quantised weights: `count` (<= 64) independent problems
+ *   outs[i][m_i, n_i] = fused_linear_with_groupwise_quantized_weight(xs[i], ws[i], ...)
+ * in one call, the quantised counterpart of grouped_matmul_bias
+ * (oneflow/user/kernels/grouped_matmul_bias.cu:153-204; functional signature
+ * oneflow/core/functional/functional_api.yaml:2759-2760: TensorTuple xs, weights, biases -> ys).
+ * As there, problems are grouped by shape: those of equal (m, k) with m <= 16 run as ONE launch
+ * (any n_i; e.g. the q, k and v projections, or gate and up, of a decode step), the rest one
+ * after the other.  All problems share the dtypes and the quantisation attributes.
+ * xs, ws, w_scales, w_zeros, bs, outs: HOST arrays of `count` device pointers (w_zeros NULL iff
+ * symmetric; bs NULL or with NULL entries for "no bias"); ms, ns, ks: HOST arrays.
+ */
+int ofq_grouped_linear_gq(void* stream, int count, const void* const* xs, const void* const* ws,
+                          const void* const* w_scales, const void* const* w_zeros,
+                          const void* const* bs, void* const* outs, const int64_t* ms,
+                          const int64_t* ns, const int64_t* ks, int w_dtype, int t_dtype,
+                          int num_bits, int symmetric, int group_dim, int64_t group_size);
+
+/*
+ * fused_glu with groupwise-quantised weights, the quantised counterpart of fused_glu
+ * (oneflow/user/kernels/fused_glu_kernel.cu:303-347 for the gating, :566-770 for Compute;
+ * functional signature oneflow/core/functional/functional_api.yaml:774-775 and the argument
+ * rules of oneflow/core/functional/impl/nn_functor.cpp:3724-3800):
+ *   matmul_wx = x w~^T + b, matmul_vx = x v~^T + c      (outputs, t_dtype [m, n])
+ *   y = matmul_wx * act(matmul_vx)                       (act in fp32 on the widened gate,
+ *                                                         rounded to t_dtype; product rounded)
+ * Split mode (v != NULL): w and v are [n, k*bits/8] with their own scales / zeros, c NULL iff b
+ * NULL.  Otherwise w is [2n, k*bits/8] (hidden-state rows first, gate rows second), b [2n] or
+ * NULL, matmul_wx is [m, 2n] and v, v_scale, v_zero, c, matmul_vx are NULL.
+ * activation: OFQ_ACT_*.  For m <= 16 the two linears of split mode are one launch.
+ */
+enum {
+  OFQ_ACT_NONE = 0,
+  OFQ_ACT_SIGMOID = 1,
+  OFQ_ACT_RELU = 2,
+  OFQ_ACT_GELU = 3,
+  OFQ_ACT_FAST_GELU = 4,
+  OFQ_ACT_SILU = 5
+};
+int ofq_fused_glu_gq(void* stream, const void* x, const void* w, const void* w_scale,
+                     const void* w_zero, const void* b, const void* v, const void* v_scale,
+                     const void* v_zero, const void* c, void* y, void* matmul_wx,
+                     void* matmul_vx, int activation, int w_dtype, int t_dtype, int num_bits,
+                     int symmetric, int group_dim, int64_t group_size, int64_t m, int64_t n,
+                     int64_t k);
+
+/*
  * matmul_quant
  * The op is named by the task but absent from the reference tree (only the env-var name
  * ONEFLOW_MLIR_GROUP_MATMUL_QUANT, python/oneflow/framework/infer_compiler/with_fx_graph.py:63);

@@ -42,6 +42,9 @@ SIGNATURES = {
     "ofq_fused_skip_layer_norm_min_max_observer": (_i, [_vp, _vp, _vp, _vp, ctypes.c_double, _vp,
                                                         _vp, _vp, _vp, _vp, _i, _i64, _i64,
                                                         ctypes.c_double, _i, _vp, _sz]),
+    "ofq_grouped_linear_gq": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
+                                   _i, _i, _i64]),
+    "ofq_fused_glu_gq": (_i, [_vp] * 13 + [_i, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64]),
     "ofq_groupwise_quantize": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64]),
     "ofq_matmul_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64]),
 }

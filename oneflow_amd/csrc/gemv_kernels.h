@@ -494,11 +494,11 @@ constexpr int kW4pMaxTiles = 4;
 //   bell-shaped ones).  x is staged in the k-order of unpack4_pairs, one MFMA per code word.
 template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
          int ZMODE = kZeroNone>
-__global__ void __launch_bounds__(NWAVES * 64)
-gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
-             const f16* __restrict__ scale, const f16* __restrict__ zero,
-             const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
-             int group_size, int cpg_shift, int rows_per_block) {
+__device__ __forceinline__ void
+gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
+              const f16* __restrict__ scale, const f16* __restrict__ zero,
+              const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
+              int group_size, int cpg_shift, int rows_per_block) {
   static_assert(EXACT || (SIGNED && ZMODE == kZeroNone), "the unrounded path has no zero term");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
@@ -510,7 +510,7 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15;
   const int kb = lane >> 4;
-  const int row0 = blockIdx.x * rows_per_block;
+  const int row0 = block * rows_per_block;
   int rows_blk = N - row0;
   if (rows_blk > rows_per_block) rows_blk = rows_per_block;
   if (rows_blk <= 0) return;
@@ -793,6 +793,74 @@ gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
       out[(int64_t)m * N + row0 + row_l] = (f16)(sum + (float)bias_at_end(bias_raw));
     }
   }
+}
+
+template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
+         int ZMODE = kZeroNone>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+             const f16* __restrict__ scale, const f16* __restrict__ zero,
+             const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
+             int group_size, int cpg_shift, int rows_per_block) {
+  gemv_w4p_body<NWAVES, kW4pDepth, EXACT, SIGNED, ZMODE>(blockIdx.x, x, w, scale, zero, bias, out,
+                                                         M, N, K, group_size, cpg_shift,
+                                                         rows_per_block);
+}
+
+// Several problems of equal m, k and quantisation in one launch: the grid is the concatenation
+// of the problems' blocks; a block finds its problem in the table.
+constexpr int kGemvMaxProblems = 8;
+struct GemvProblem {
+  const void* x;
+  const uint8_t* w;
+  const void* scale;
+  const void* zero;
+  const void* bias;
+  void* out;
+  int N;
+  int first_block;  // of the grid
+};
+struct GemvGroup {
+  GemvProblem p[kGemvMaxProblems];
+  int count;
+};
+// (every field is selected with a chain of scalar selects over the table entries: indexing the
+// argument struct with a run-time value, or copying an entry as a whole, moves the table to
+// scratch memory)
+__device__ __forceinline__ GemvProblem select_problem(const GemvGroup& g, int block) {
+  int i = 0;
+#pragma unroll
+  for (int j = 1; j < kGemvMaxProblems; ++j) {
+    if (j < g.count && block >= g.p[j].first_block) i = j;
+  }
+  GemvProblem pr;
+#define OFQ_SEL(field)                                   \
+  pr.field = g.p[0].field;                               \
+  _Pragma("unroll") for (int j = 1; j < kGemvMaxProblems; ++j) { \
+    if (i == j) pr.field = g.p[j].field;                 \
+  }
+  OFQ_SEL(x)
+  OFQ_SEL(w)
+  OFQ_SEL(scale)
+  OFQ_SEL(zero)
+  OFQ_SEL(bias)
+  OFQ_SEL(out)
+  OFQ_SEL(N)
+  OFQ_SEL(first_block)
+#undef OFQ_SEL
+  return pr;
+}
+
+template<int NWAVES, bool EXACT, bool SIGNED, int ZMODE>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_w4p_f16_grouped(GemvGroup g, int M, int K, int group_size, int cpg_shift,
+                     int rows_per_block) {
+  const GemvProblem pr = select_problem(g, (int)blockIdx.x);
+  gemv_w4p_body<NWAVES, 1, EXACT, SIGNED, ZMODE>(
+      (int)blockIdx.x - pr.first_block, static_cast<const f16*>(pr.x), pr.w,
+      static_cast<const f16*>(pr.scale), static_cast<const f16*>(pr.zero),
+      static_cast<const f16*>(pr.bias), static_cast<f16*>(pr.out), M, pr.N, K, group_size,
+      cpg_shift, rows_per_block);
 }
 
 inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,

@@ -13,6 +13,7 @@
 #pragma once
 
 #include "dequant_regs.h"
+#include "gemv_kernels.h"
 #include "ofq_device.h"
 
 namespace ofq {
@@ -55,11 +56,11 @@ __device__ __forceinline__ float raw16_at_end(uint16_t raw) {
 // Either way a wave takes chunk pairs p = wave, wave + NWAVES, ... and walks all tiles of the
 // block for each, so x is fetched once per pair and the per-tile sums stay in registers.
 template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, bool STAGED>
-__global__ void __launch_bounds__(NWAVES * 64)
-gemv_rows(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
-          const uint16_t* __restrict__ scale, const uint16_t* __restrict__ zero,
-          const uint16_t* __restrict__ bias, uint16_t* __restrict__ out, int M, int N, int K,
-          int group_size, int gs_shift, int rows_per_block) {
+__device__ __forceinline__ void
+gemv_rows_body(int block, const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
+               const uint16_t* __restrict__ scale, const uint16_t* __restrict__ zero,
+               const uint16_t* __restrict__ bias, uint16_t* __restrict__ out, int M, int N, int K,
+               int group_size, int gs_shift, int rows_per_block) {
   typedef typename TT<T>::storage S;
   static_assert(sizeof(S) == 2, "16-bit element types");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -76,7 +77,7 @@ gemv_rows(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15;
   const int kb = lane >> 4;
-  const int row0 = blockIdx.x * rows_per_block;
+  const int row0 = block * rows_per_block;
   int rows_blk = N - row0;
   if (rows_blk > rows_per_block) rows_blk = rows_per_block;
   if (rows_blk <= 0) return;
@@ -280,6 +281,31 @@ gemv_rows(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
       TT<T>::store(reinterpret_cast<S*>(out) + (int64_t)m * N + row0 + row_l, sum + bv);
     }
   }
+}
+
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, bool STAGED>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_rows(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
+          const uint16_t* __restrict__ scale, const uint16_t* __restrict__ zero,
+          const uint16_t* __restrict__ bias, uint16_t* __restrict__ out, int M, int N, int K,
+          int group_size, int gs_shift, int rows_per_block) {
+  gemv_rows_body<T, BITS, SIGNED, ZMODE, NWAVES, STAGED>(blockIdx.x, x, w, scale, zero, bias, out,
+                                                         M, N, K, group_size, gs_shift,
+                                                         rows_per_block);
+}
+
+// Several linears of the same m, k and quantisation in one launch (q/k/v, gate/up ...): the grid
+// is the concatenation of the problems' blocks, every problem cut into rows_per_block-row
+// blocks; a block finds its problem in the table and runs the single-problem body on it.
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, bool STAGED>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_rows_grouped(GemvGroup g, int M, int K, int group_size, int gs_shift, int rows_per_block) {
+  const GemvProblem pr = select_problem(g, (int)blockIdx.x);
+  gemv_rows_body<T, BITS, SIGNED, ZMODE, NWAVES, STAGED>(
+      (int)blockIdx.x - pr.first_block, static_cast<const uint16_t*>(pr.x), pr.w,
+      static_cast<const uint16_t*>(pr.scale), static_cast<const uint16_t*>(pr.zero),
+      static_cast<const uint16_t*>(pr.bias), static_cast<uint16_t*>(pr.out), M, pr.N, K,
+      group_size, gs_shift, rows_per_block);
 }
 
 inline size_t gemv_rows_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,

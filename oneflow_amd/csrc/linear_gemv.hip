@@ -327,7 +327,180 @@ int launch_gemv_variant(hipStream_t st, const LinearArgs& a) {
   return ofq_check_launch();
 }
 
+// ---- several problems, one launch -------------------------------------------------------------
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
+int launch_rows_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
+                             int group_size, int rows_per_block, size_t lds) {
+  auto kern = gemv_rows_grouped<T, BITS, SIGNED, ZMODE, NW, STAGED>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, NW * 64, lds, st>>>(g, m, k, group_size, ilog2_exact(group_size), rows_per_block);
+  return ofq_check_launch();
+}
+
+template<typename T, int NW, bool STAGED>
+int launch_rows_grouped_t(hipStream_t st, const LinearArgs& a, const GemvGroup& g, int grid,
+                          int rpb, size_t lds) {
+  const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
+#define OFQ_R(B, SG, ZM)                                                           \
+  if (a.bits == B && a.w_signed == SG && zmode == ZM)                              \
+    return launch_rows_grouped_inst<T, B, SG, ZM, NW, STAGED>(st, g, grid, (int)a.m, (int)a.k, \
+                                                              (int)a.group_size, rpb, lds);
+  OFQ_R(4, true, kZeroNone)
+  OFQ_R(4, false, kZeroSymU)
+  OFQ_R(4, false, kZeroAsym)
+  OFQ_R(8, true, kZeroNone)
+  OFQ_R(8, false, kZeroSymU)
+  OFQ_R(8, false, kZeroAsym)
+#undef OFQ_R
+  return OFQ_ERR_UNSUPPORTED;
+}
+
+template<int NW, bool EXACT, bool SIGNED, int ZMODE>
+int launch_w4p_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
+                            int group_size, int rows_per_block, size_t lds) {
+  auto kern = gemv_w4p_f16_grouped<NW, EXACT, SIGNED, ZMODE>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, NW * 64, lds, st>>>(g, m, k, group_size, ilog2_exact(group_size / 128),
+                                  rows_per_block);
+  return ofq_check_launch();
+}
+
+// the smallest common rows_per_block (>= 16, <= max_rows) whose blocks fit one resident round:
+// 256 blocks of 16 waves, else 512 of 8; returns the grid size
+int64_t grouped_split(const LinearArgs* pr, int count, int max_rows, int* rpb_out) {
+  constexpr int kCUs = 256;
+  int64_t n_total = 0;
+  for (int i = 0; i < count; ++i) n_total += pr[i].n;
+  auto blocks_at = [&](int rpb) {
+    int64_t b = 0;
+    for (int i = 0; i < count; ++i) b += (pr[i].n + rpb - 1) / rpb;
+    return b;
+  };
+  int rpb = (int)((n_total + kCUs - 1) / kCUs);
+  if (rpb < 16) rpb = 16;
+  while (rpb < max_rows && blocks_at(rpb) > kCUs) ++rpb;
+  if (rpb > max_rows || blocks_at(rpb) > kCUs) {
+    rpb = (int)((n_total + 2 * kCUs - 1) / (2 * kCUs));
+    if (rpb < 16) rpb = 16;
+    while (rpb < max_rows && blocks_at(rpb) > 2 * kCUs) ++rpb;
+  }
+  if (rpb > max_rows) rpb = max_rows;
+  *rpb_out = rpb;
+  return blocks_at(rpb);
+}
+
+void fill_group(GemvGroup& g, const LinearArgs* pr, int count, int rpb) {
+  g.count = count;
+  int first = 0;
+  for (int i = 0; i < count; ++i) {
+    g.p[i].x = pr[i].x;
+    g.p[i].w = static_cast<const uint8_t*>(pr[i].w);
+    g.p[i].scale = pr[i].scale;
+    g.p[i].zero = pr[i].zero;
+    g.p[i].bias = pr[i].bias;
+    g.p[i].out = pr[i].out;
+    g.p[i].N = (int)pr[i].n;
+    g.p[i].first_block = first;
+    first += (int)((pr[i].n + rpb - 1) / rpb);
+  }
+}
+
+// fp16, 4-bit codes, groups in multiples of 128: the kernel of the single-problem fast path
+int launch_w4p_grouped(hipStream_t st, const LinearArgs* pr, int count) {
+  const LinearArgs& a = pr[0];
+  int rpb = 0;
+  const int64_t grid = grouped_split(pr, count, 16 * kW4pMaxTiles, &rpb);
+  if (grid > 0x7FFFFFFF) return OFQ_ERR_UNSUPPORTED;
+  const bool two_per_cu = grid > 256;
+  const int nw = two_per_cu ? 8 : 16;
+  if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
+  if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) return OFQ_ERR_UNSUPPORTED;
+  const bool exact = !(a.symmetric && a.w_signed);
+  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                                        !a.symmetric);
+  if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
+  GemvGroup g{};
+  fill_group(g, pr, count, rpb);
+#define OFQ_W4PG(NWV)                                                                        \
+  if (nw == NWV) {                                                                           \
+    if (!exact)                                                                              \
+      return launch_w4p_grouped_inst<NWV, false, true, kZeroNone>(                           \
+          st, g, (int)grid, (int)a.m, (int)a.k, (int)a.group_size, rpb, lds);                \
+    if (a.symmetric)                                                                         \
+      return launch_w4p_grouped_inst<NWV, true, false, kZeroSymU>(                           \
+          st, g, (int)grid, (int)a.m, (int)a.k, (int)a.group_size, rpb, lds);                \
+    return launch_w4p_grouped_inst<NWV, true, false, kZeroAsym>(                             \
+        st, g, (int)grid, (int)a.m, (int)a.k, (int)a.group_size, rpb, lds);                  \
+  }
+  OFQ_W4PG(16) OFQ_W4PG(8)
+#undef OFQ_W4PG
+  return OFQ_ERR_UNSUPPORTED;
+}
+
 }  // namespace
+
+int launch_gemv_grouped(hipStream_t st, const LinearArgs* pr, int count) {
+  if (count < 1 || count > kGemvMaxProblems) return OFQ_ERR_UNSUPPORTED;
+  const LinearArgs& a = pr[0];
+  bool all_w4p = true;
+  for (int i = 0; i < count; ++i) {
+    const LinearArgs& b = pr[i];
+    if (!rows_supported(b)) return OFQ_ERR_UNSUPPORTED;
+    if (b.t_dtype != a.t_dtype || b.bits != a.bits || b.w_signed != a.w_signed
+        || b.symmetric != a.symmetric || b.group_size != a.group_size || b.m != a.m
+        || b.k != a.k) {
+      return OFQ_ERR_UNSUPPORTED;
+    }
+    all_w4p = all_w4p && w4p_supported(b);
+  }
+  if (all_w4p) {
+    const int rc = launch_w4p_grouped(st, pr, count);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
+  int rpb = 0;
+  const int64_t grid = grouped_split(pr, count, 16 * kRowsMaxTiles, &rpb);
+  if (grid > 0x7FFFFFFF) return OFQ_ERR_UNSUPPORTED;
+  const bool two_per_cu = grid > 256;
+  const int nw = two_per_cu ? 8 : 16;
+  const size_t cap = (two_per_cu ? 80u : 160u) * 1024u;
+  bool staged = a.m * a.k / 8 <= (int64_t)kRowsMaxUnits * nw * 64;
+  size_t lds = gemv_rows_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, !a.symmetric,
+                                   staged);
+  if (staged && lds > cap) {
+    staged = false;
+    lds = gemv_rows_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, !a.symmetric,
+                              false);
+  }
+  if (lds > cap) return OFQ_ERR_UNSUPPORTED;
+  GemvGroup g{};
+  fill_group(g, pr, count, rpb);
+#define OFQ_RG(TT_, NWV)                                                                   \
+  return staged ? launch_rows_grouped_t<TT_, NWV, true>(st, a, g, (int)grid, rpb, lds)     \
+                : launch_rows_grouped_t<TT_, NWV, false>(st, a, g, (int)grid, rpb, lds)
+  if (a.t_dtype == OFQ_BF16) {
+    if (nw == 16) { OFQ_RG(bf16, 16); }
+    OFQ_RG(bf16, 8);
+  }
+  if (nw == 16) { OFQ_RG(f16, 16); }
+  OFQ_RG(f16, 8);
+#undef OFQ_RG
+}
 
 bool gemv_wq_supported(const LinearArgs& a) {
   if (rows_supported(a)) return true;

@@ -13,6 +13,8 @@ One deliberate difference: the reference functor routes ``m > 8`` of the fused l
 ``groupwise_dequantize`` + matmul (quantization.cpp:341-350); here every ``m`` goes to the fused
 op, whose kernels cover both regimes.
 """
+import ctypes
+
 import torch
 
 from . import _lib
@@ -137,9 +139,11 @@ def groupwise_dequantize(in_, scale, *, zero=None, num_bits=8, symmetric=True, g
 # fused_linear_with_groupwise_quantized_weight:
 # FusedLinearWithGroupwiseQuantizedWeightFunctor, quantization.cpp:264-372
 # --------------------------------------------------------------------------------------------
-def fused_linear_with_groupwise_quantized_weight(x, w, w_scale, *, w_zero=None, b=None,
-                                                 num_bits=8, symmetric=True, group_dim=-1,
-                                                 group_size=-1):
+def _check_fused_linear_args(x, w, w_scale, w_zero, b, num_bits, symmetric, group_dim,
+                             group_size):
+    """The argument checks of FusedLinearWithGroupwiseQuantizedWeightFunctor
+    (oneflow/core/functional/impl/quantization.cpp:264-340); returns (m, n, k, group_dim,
+    group_size) with the negative defaults resolved."""
     _check(x.dim() >= 2,
            "The number of dimensions for tensor x should be greater than or equal to 2.")
     k = x.shape[-1]
@@ -195,6 +199,14 @@ def fused_linear_with_groupwise_quantized_weight(x, w, w_scale, *, w_zero=None, 
                "dimension of tensor w")
     _check(x.dtype in (torch.float16, torch.float32, torch.bfloat16),
            f"no fused_linear_with_groupwise_quantized_weight kernel for dtype {x.dtype}")
+    return m, n, k, gd, gs
+
+
+def fused_linear_with_groupwise_quantized_weight(x, w, w_scale, *, w_zero=None, b=None,
+                                                 num_bits=8, symmetric=True, group_dim=-1,
+                                                 group_size=-1):
+    m, n, k, gd, gs = _check_fused_linear_args(x, w, w_scale, w_zero, b, num_bits, symmetric,
+                                               group_dim, group_size)
     _require_gpu(x, w, w_scale, w_zero, b)
     x, w, w_scale, w_zero, b = map(_contig, (x, w, w_scale, w_zero, b))
     out = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=x.dtype, device=x.device)
@@ -207,6 +219,91 @@ def fused_linear_with_groupwise_quantized_weight(x, w, w_scale, *, w_zero=None, 
                                k, _ptr(ws), ws_bytes)
     _lib.check("ofq_fused_linear_gq", st)
     return out
+
+
+def grouped_linear_with_groupwise_quantized_weight(xs, ws, w_scales, *, w_zeros=None, bs=None,
+                                                   num_bits=8, symmetric=True, group_dim=-1,
+                                                   group_size=-1):
+    """``fused_linear_with_groupwise_quantized_weight`` over tuples of problems, the quantised
+    counterpart of ``grouped_matmul_bias(xs, weights, biases)`` (functional_api.yaml:2759-2760;
+    checks of GroupedMatmulBiasFunctor: equal tuple lengths).  Problems of equal (m, k) with
+    m <= 16 run as one launch.  Returns the list of outputs."""
+    count = len(xs)
+    _check(count > 0, "xs should not be empty")
+    _check(count <= 64, "at most 64 problems per call")
+    _check(len(ws) == count and len(w_scales) == count, "xs, ws and w_scales should have the same length")
+    _check(w_zeros is None or len(w_zeros) == count, "w_zeros should have the length of xs")
+    _check(bs is None or len(bs) == count, "bs should have the length of xs")
+    w_zeros = list(w_zeros) if w_zeros is not None else [None] * count
+    bs = list(bs) if bs is not None else [None] * count
+    dims = [_check_fused_linear_args(xs[i], ws[i], w_scales[i], w_zeros[i], bs[i], num_bits,
+                                     symmetric, group_dim, group_size) for i in range(count)]
+    _check(all(x.dtype == xs[0].dtype for x in xs) and all(w.dtype == ws[0].dtype for w in ws),
+           "all problems should share the dtypes of x and w")
+    _check(all(d[3] == dims[0][3] and d[4] == dims[0][4] for d in dims),
+           "all problems should share group_dim and group_size")
+    _require_gpu(*xs, *ws, *w_scales, *w_zeros, *bs)
+    xs, ws, w_scales = [list(map(_contig, t)) for t in (xs, ws, w_scales)]
+    w_zeros, bs = list(map(_contig, w_zeros)), list(map(_contig, bs))
+    outs = [torch.empty(tuple(x.shape[:-1]) + (d[1],), dtype=x.dtype, device=x.device)
+            for x, d in zip(xs, dims)]
+    arr = lambda ts: (ctypes.c_void_p * count)(*[_ptr(t) for t in ts])
+    i64 = lambda v: (ctypes.c_int64 * count)(*v)
+    L = _lib.lib()
+    st = L.ofq_grouped_linear_gq(
+        _stream(xs[0]), count, arr(xs), arr(ws), arr(w_scales), None if symmetric else arr(w_zeros),
+        arr(bs), arr(outs), i64([d[0] for d in dims]), i64([d[1] for d in dims]),
+        i64([d[2] for d in dims]), _dt(ws[0]), _dt(xs[0]), num_bits, int(symmetric), dims[0][3],
+        dims[0][4])
+    _lib.check("ofq_grouped_linear_gq", st)
+    return outs
+
+
+_ACTIVATIONS = {"none": 0, "sigmoid": 1, "relu": 2, "gelu": 3, "fast_gelu": 4, "silu": 5}
+
+
+def fused_glu_with_groupwise_quantized_weight(x, w, w_scale, *, w_zero=None, b=None, v=None,
+                                              v_scale=None, v_zero=None, c=None,
+                                              activation="none", num_bits=8, symmetric=True,
+                                              group_dim=-1, group_size=-1):
+    """``fused_glu(x, w, b, v, c, activation)`` (functional_api.yaml:774-775, checks of
+    FusedGluFunctor, nn_functor.cpp:3724-3800) with groupwise-quantised ``w`` / ``v``:
+    ``y = (x w~^T + b) * act(x v~^T + c)``; without ``v`` the 2n rows of ``w`` hold the
+    hidden-state rows first and the gate rows second."""
+    _check(activation in _ACTIVATIONS, f"unsupported activation {activation!r}")
+    split = v is not None
+    if b is not None:
+        if split:
+            _check(c is not None, "expected existance of c, when provide tensors w, v and b")
+    else:
+        _check(c is None, "expected existance of b while providing c")
+    m, n_w, k, gd, gs = _check_fused_linear_args(x, w, w_scale, w_zero, b, num_bits, symmetric,
+                                                 group_dim, group_size)
+    if split:
+        _check(v_scale is not None, "v_scale should be specified with v")
+        _check(tuple(v.shape) == tuple(w.shape) and v.dtype == w.dtype,
+               "v should have the shape and dtype of w")
+        _check_fused_linear_args(x, v, v_scale, v_zero, c, num_bits, symmetric, group_dim,
+                                 group_size)
+        n = n_w
+    else:
+        _check(v_scale is None and v_zero is None and c is None,
+               "v_scale, v_zero and c belong to v")
+        _check(n_w % 2 == 0, "dimension 0 of 'w' is not divisible by 2")
+        n = n_w // 2
+    _require_gpu(x, w, w_scale, w_zero, b, v, v_scale, v_zero, c)
+    x, w, w_scale, w_zero, b, v, v_scale, v_zero, c = map(
+        _contig, (x, w, w_scale, w_zero, b, v, v_scale, v_zero, c))
+    lead = tuple(x.shape[:-1])
+    y = torch.empty(lead + (n,), dtype=x.dtype, device=x.device)
+    matmul_wx = torch.empty(lead + (n_w,), dtype=x.dtype, device=x.device)
+    matmul_vx = torch.empty(lead + (n,), dtype=x.dtype, device=x.device) if split else None
+    st = _lib.lib().ofq_fused_glu_gq(
+        _stream(x), _ptr(x), _ptr(w), _ptr(w_scale), _ptr(w_zero), _ptr(b), _ptr(v), _ptr(v_scale),
+        _ptr(v_zero), _ptr(c), _ptr(y), _ptr(matmul_wx), _ptr(matmul_vx), _ACTIVATIONS[activation],
+        _dt(w), _dt(x), num_bits, int(symmetric), gd, gs, m, n, k)
+    _lib.check("ofq_fused_glu_gq", st)
+    return y
 
 
 # --------------------------------------------------------------------------------------------

@@ -561,6 +561,47 @@ int ofq_ref_skip_layer_norm_min_max_observer(const void* x, const void* bias, co
                                   rows, cols, eps, t, bits);
 }
 
+/* ------------------------------------------------------------------------------------------
+ * The gating of fused_glu (user/kernels/fused_glu_kernel.cu:303-347): per element
+ *   y = hidden_state * act(gate), hidden_state = matmul_wx[r*stride + c],
+ *   gate = matmul_vx[r*stride + c], both operations in T.  For the 16-bit types the activation
+ *   is the fp32 functor applied to the widened value and rounded back
+ *   (ep/cuda/primitive/unary_functor.cuh:449-464,522-570); fp32 forms:
+ *   ep/common/primitive/unary_functor.h:146-170,477-484 (relu, silu, sigmoid),
+ *   ep/cuda/primitive/unary_functor.cuh:31-58 (gelu, fast_gelu).  fast_gelu follows the generic
+ *   form for every T (the reference has an architecture-dependent fp16 variant, :100-136).
+ * act: 0 none, 1 sigmoid, 2 relu, 3 gelu, 4 fast_gelu, 5 silu.
+ * ---------------------------------------------------------------------------------------- */
+static float glu_activation(float v, int act) {
+  switch (act) {
+    case 1: return 1.0f / (1.0f + expf(-v));
+    case 2: return v <= 0.0f ? 0.0f : v;
+    case 3: return 0.5f * v * (1.0f + erff(0.70710678118654752440f * v));
+    case 4: {
+      const float alpha = 0.7978845608028654f;
+      const float beta = 0.044714998453855515f;
+      const float tanh_in = alpha * (v + beta * v * v * v);
+      return 0.5f * v * (1.0f + tanhf(tanh_in));
+    }
+    case 5: return v / (1.0f + expf(-v));
+    default: return v;
+  }
+}
+
+int ofq_ref_glu_gate(const void* matmul_wx, const void* matmul_vx, void* y, int64_t m, int64_t n,
+                     int64_t stride, int t, int act) {
+  if (act < 0 || act > 5) return 1;
+  for (int64_t r = 0; r < m; ++r) {
+    for (int64_t c = 0; c < n; ++c) {
+      const float h = t_load(matmul_wx, r * stride + c, t);
+      const float g = t_load(matmul_vx, r * stride + c, t);
+      const float a = t_round(glu_activation(g, act), t);
+      t_store(y, r * n + c, h * a, t);
+    }
+  }
+  return 0;
+}
+
 /* quantization with a low-precision input and int8 codes (the dynamic activation path): the
  * same rule as QuantizationPerLayerSymmetric (quantization_kernel.cpp:22-33) evaluated in fp32
  * on the widened input, codes narrowed to int8 (exact: the clamp keeps them in [-128,127]). */

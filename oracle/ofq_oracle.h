@@ -68,6 +68,8 @@ int ofq_ref_skip_layer_norm_min_max_observer(const void* x, const void* bias, co
                                              void* y, float* scale, float* zero_point,
                                              int64_t rows, int64_t cols, double eps, int t,
                                              int bits);
+int ofq_ref_glu_gate(const void* matmul_wx, const void* matmul_vx, void* y, int64_t m, int64_t n,
+                     int64_t stride, int t, int act);
 
 int ofq_ref_quantize_to_int8(const void* in, const float* scale, int8_t* out, int64_t elem_cnt,
                              int64_t scale_size, int64_t shape0, int t, int bits);

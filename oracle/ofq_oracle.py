@@ -268,6 +268,36 @@ def skip_layer_norm_min_max_observer(x, gamma, beta, bias=None, skip=None, eps=1
     return y, scale, zp
 
 
+ACTIVATIONS = {"none": 0, "sigmoid": 1, "relu": 2, "gelu": 3, "fast_gelu": 4, "silu": 5}
+
+
+def glu_gate(hidden, gate, activation="none"):
+    """y = hidden * act(gate) in T (fused_glu_kernel.cu:303-347); 2-D arrays of equal shape."""
+    hidden = _c(hidden)
+    gate = _c(gate)
+    m, n = hidden.shape
+    y = np.empty_like(hidden)
+    rc = lib().ofq_ref_glu_gate(_p(hidden), _p(gate), _p(y), _i64(m), _i64(n), _i64(n),
+                                t_code(hidden), ACTIVATIONS[activation])
+    assert rc == 0
+    return y
+
+
+def fused_glu(x, w, w_scale, w_zero=None, b=None, v=None, v_scale=None, v_zero=None, c=None,
+              activation="none", num_bits=8, symmetric=True, group_dim=-1, group_size=-1):
+    """fused_glu over groupwise-quantised weights: the op's two linears (rounded to T, as the
+    reference stores matmul_wx / matmul_vx) and the gating.  Returns (y, matmul_wx, matmul_vx)."""
+    wx = fused_linear(x, w, w_scale, w_zero, b, num_bits, symmetric, group_dim, group_size)
+    wx2 = wx.reshape(-1, wx.shape[-1])
+    if v is not None:
+        vx = fused_linear(x, v, v_scale, v_zero, c, num_bits, symmetric, group_dim, group_size)
+        y = glu_gate(wx2, vx.reshape(wx2.shape), activation)
+        return y.reshape(wx.shape), wx, vx
+    n = wx2.shape[1] // 2
+    y = glu_gate(np.ascontiguousarray(wx2[:, :n]), np.ascontiguousarray(wx2[:, n:]), activation)
+    return y.reshape(wx.shape[:-1] + (n,)), wx, None
+
+
 def quantize_to_int8(x, scale, quantization_bit=8):
     x = _c(x)
     scale = _c(scale, np.float32)

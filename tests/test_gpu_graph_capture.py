@@ -139,3 +139,36 @@ def test_moving_average_observer_in_a_graph():
         torch.cuda.synchronize()
         assert torch.equal(cap.moving_max, ref.moving_max) and torch.equal(cap.moving_min, ref.moving_min), i
         assert torch.equal(s, rs) and torch.equal(z, rz), i
+
+
+def test_grouped_glu_and_skip_layer_norm_in_a_graph():
+    """The decoder-block neighbours: q/k/v as one grouped call, the gated unit, and the residual
+    LayerNorm + observer, captured together."""
+    import oneflow_amd as flow
+    import torch
+    k, g = 512, 128
+    rng = H.rng_for(21, 0)
+    ws = []
+    for n in (512, 128, 128, 1376, 1376):
+        codes = rng.integers(0, 256, size=(n, k // 2)).astype(np.uint8)
+        sc = rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float16)
+        ze = rng.uniform(-0.08, -0.04, size=(n, k // g)).astype(np.float16)
+        ws.append((_t(codes), _t(sc), _t(ze)))
+    gamma = _t((1 + 0.1 * rng.standard_normal(k)).astype(np.float16))
+
+    def inputs(seed):
+        r = H.rng_for(22, seed)
+        return [_t(r.standard_normal((2, k)).astype(np.float16)),
+                _t(r.standard_normal((2, k)).astype(np.float16))]
+
+    def run(x, skip):
+        h, s, z = flow._C.fused_skip_layer_norm_min_max_observer(x, gamma, None, None, skip, 1e-5,
+                                                                 1.0, 8)
+        q, kk, v = flow._C.grouped_linear_with_groupwise_quantized_weight(
+            [h, h, h], [w[0] for w in ws[:3]], [w[1] for w in ws[:3]],
+            w_zeros=[w[2] for w in ws[:3]], num_bits=4, symmetric=False, group_dim=1, group_size=g)
+        y = flow._C.fused_glu_with_groupwise_quantized_weight(
+            h, ws[3][0], ws[3][1], w_zero=ws[3][2], v=ws[4][0], v_scale=ws[4][1], v_zero=ws[4][2],
+            activation="silu", num_bits=4, symmetric=False, group_dim=1, group_size=g)
+        return h, s, q, kk, v, y
+    _capture_and_check(inputs, run)

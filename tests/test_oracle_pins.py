@@ -344,6 +344,53 @@ def test_skip_layer_norm_observer_against_the_reference_composition():
         assert np.array_equal(a_, b_)
 
 
+def test_glu_gate_against_float64_forms():
+    """hidden * act(gate) in T.  'none' and 'relu' have exact closed forms; the smooth
+    activations are compared with float64 evaluations of the textbook formulas (scipy erf, numpy
+    exp / tanh): the activation must agree to a rounding of T, so a wrong constant, a swapped
+    operand (act applied to the hidden state) or a missing rounding of act(gate) shows."""
+    from scipy.special import erf
+    rng = np.random.default_rng(21)
+    h = rng.standard_normal((6, 40)).astype(np.float16)
+    g = (3 * rng.standard_normal((6, 40))).astype(np.float16)
+    assert np.array_equal(O.glu_gate(h, g, "none"), h * g)
+    assert np.array_equal(O.glu_gate(h, g, "relu"), h * np.maximum(g, np.float16(0)))
+    z = np.zeros_like(g)
+    assert np.array_equal(O.glu_gate(h, z, "sigmoid"), h * np.float16(0.5))
+    for name in ("silu", "gelu", "fast_gelu"):
+        assert np.all(O.glu_gate(h, z, name) == 0)
+    g64 = g.astype(np.float64)
+    forms = {
+        "sigmoid": 1 / (1 + np.exp(-g64)),
+        "silu": g64 / (1 + np.exp(-g64)),
+        "gelu": 0.5 * g64 * (1 + erf(g64 / np.sqrt(2.0))),
+        "fast_gelu": 0.5 * g64 * (1 + np.tanh(0.7978845608028654 * (g64 + 0.044714998453855515 * g64 ** 3))),
+    }
+    ones = np.ones_like(h)
+    for name, want in forms.items():
+        act = O.glu_gate(ones, g, name).astype(np.float64)  # 1 * act(gate): the activation itself
+        ulp = np.exp2(np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -14))) - 10)
+        # (1 + erf) and (1 + tanh) are formed in fp32, as in the reference: for very negative
+        # gates that sum cancels and carries an absolute error of one fp32 rounding of 1
+        slack = 0.5 * np.abs(g64) * 2.0 ** -23 if name in ("gelu", "fast_gelu") else 0.0
+        assert (np.abs(act - want) <= 0.501 * ulp + slack + 1e-12).all(), name
+        # and the product is one more rounding of hidden * that value
+        y = O.glu_gate(h, g, name)
+        assert np.array_equal(y, h * O.glu_gate(ones, g, name)), name
+    # fp32 keeps the fp32 evaluation
+    g32 = g.astype(np.float32)
+    y32 = O.glu_gate(np.ones_like(g32), g32, "silu")
+    assert np.allclose(y32, forms["silu"], rtol=3e-7, atol=1e-9)
+    # the split of the single-weight mode: hidden-state columns first, gate columns second
+    # (test_fused_glu.py:66-71, `matmul_wx_b.chunk(2, dim=-1)`)
+    x = rng.standard_normal((3, 64)).astype(np.float16)
+    codes = rng.integers(-100, 100, size=(16, 64)).astype(np.int8)
+    sc = rng.uniform(1e-3, 1e-2, size=(16, 1)).astype(np.float16)
+    y, wx, _ = O.fused_glu(x, codes, sc, activation="relu", num_bits=8, symmetric=True,
+                           group_dim=1, group_size=64)
+    assert np.array_equal(y, wx[:, :8] * np.maximum(wx[:, 8:], np.float16(0)))
+
+
 def test_matmul_quant_exact_integer_accumulation():
     rng = np.random.default_rng(4)
     m, n, k = 7, 19, 4096
