@@ -492,14 +492,46 @@ constexpr int kW4pMaxTiles = 4;
 //   three roundings are relative to those, and leaving them out moves the result by ~1e-3
 //   relative to the dequantize->matmul composition (measured 6e-4 on uniform codes, more on
 //   bell-shaped ones).  x is staged in the k-order of unpack4_pairs, one MFMA per code word.
+// GLU mode: the block also owns the SAME rows of a second weight (the gate), as further tiles,
+// and its last step forms y = T(hidden * T(act(gate))) from the two rounded sums
+// (oneflow/user/kernels/fused_glu_kernel.cu:303-347); both sums are stored as well.
+struct GluArgs {
+  const uint8_t* w2;
+  const f16* scale2;
+  const f16* zero2;
+  const f16* bias2;
+  f16* out2;
+  f16* y;
+  int act;  // 0 none, 1 sigmoid, 2 relu, 3 gelu, 4 fast_gelu, 5 silu
+};
+
+// fp32 forms of oneflow/core/ep/common/primitive/unary_functor.h:146-170,477-484 and
+// oneflow/core/ep/cuda/primitive/unary_functor.cuh:31-58
+__device__ __forceinline__ float glu_activation(float v, int act) {
+  switch (act) {
+    case 1: return 1.0f / (1.0f + expf(-v));
+    case 2: return v <= 0.0f ? 0.0f : v;
+    case 3: return 0.5f * v * (1.0f + erff(0.70710678118654752440f * v));
+    case 4: {
+      const float alpha = 0.7978845608028654f;
+      const float beta = 0.044714998453855515f;
+      const float tanh_in = alpha * (v + beta * v * v * v);
+      return 0.5f * v * (1.0f + tanhf(tanh_in));
+    }
+    case 5: return v / (1.0f + expf(-v));
+    default: return v;
+  }
+}
+
 template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
-         int ZMODE = kZeroNone>
+         int ZMODE = kZeroNone, bool GLU = false>
 __device__ __forceinline__ void
 gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
               const f16* __restrict__ scale, const f16* __restrict__ zero,
               const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
-              int group_size, int cpg_shift, int rows_per_block) {
+              int group_size, int cpg_shift, int rows_per_block, GluArgs glu = GluArgs()) {
   static_assert(EXACT || (SIGNED && ZMODE == kZeroNone), "the unrounded path has no zero term");
+  constexpr int NMAT = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
   const int nchunks = K >> 7;
@@ -514,15 +546,20 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   int rows_blk = N - row0;
   if (rows_blk > rows_per_block) rows_blk = rows_per_block;
   if (rows_blk <= 0) return;
-  const int ntiles = (rows_blk + 15) >> 4;
+  const int ntiles = (rows_blk + 15) >> 4;  // per weight
+  const int nvt = NMAT * ntiles;            // tiles the block walks: the gate's follow the first's
   const bool has_x = r < M;
+  // tile vt -> its weight (0 / 1), its first row within the block, its row of the scale tiles
+  auto mat_of = [&](int vt) { return GLU && vt >= ntiles ? 1 : 0; };
+  auto trow_of = [&](int vt) { return (GLU && vt >= ntiles ? vt - ntiles : vt) * 16; };
+  auto srow_of = [&](int vt) { return (GLU && vt >= ntiles ? rows_per_block : 0) + trow_of(vt); };
 
-  // LDS: [red ntiles*NWAVES*M*16 f32][scales rows_per_block*G halves, padded to 16 B]
+  // LDS: [red ntiles*NWAVES*M*16 f32][scales NMAT*rows_per_block*G halves, padded to 16 B]
   //      [zeros, same size (asymmetric only)][corr nchunks*16 f32 (unrounded path only)]
   //      [64 zero bytes][x records M*nchunks*256 B]
   float* red = reinterpret_cast<float*>(smem);
   const int red_floats = kW4pMaxTiles * NWAVES * M * 16;
-  const int tile_bytes = (rows_per_block * G * 2 + 15) & ~15;
+  const int tile_bytes = (NMAT * rows_per_block * G * 2 + 15) & ~15;
   f16* sl = reinterpret_cast<f16*>(smem + (size_t)red_floats * 4);
   f16* zl = reinterpret_cast<f16*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
   float* corr_l = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(sl)
@@ -555,14 +592,27 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     sreg = *reinterpret_cast<const u32x4*>(stile + se);
     if (ZMODE == kZeroAsym) zreg = *reinterpret_cast<const u32x4*>(ztile + se);
   }
+  // the gate's scales (GLU): same rows of the second weight, hence the same alignment
+  const f16* stile2 = GLU ? glu.scale2 + (int64_t)row0 * G : stile;
+  const f16* ztile2 = GLU && ZMODE == kZeroAsym ? glu.zero2 + (int64_t)row0 * G : stile2;
+  const bool s_aligned2 = ((reinterpret_cast<uintptr_t>(stile2)) & 15u) == 0;
+  const bool s_vec2 = GLU && s_aligned2 && se + 8 <= tile_halves;
+  u32x4 sreg2, zreg2;
+  if (GLU && s_vec2) {
+    sreg2 = *reinterpret_cast<const u32x4*>(stile2 + se);
+    if (ZMODE == kZeroAsym) zreg2 = *reinterpret_cast<const u32x4*>(ztile2 + se);
+  }
   // bias of the output this thread folds at the end: tid = (tile * M + m) * 16 + n
   // (kept as raw bits: widening it here would wait for every load issued so far)
-  uint16_t bias_raw = 0;
+  uint16_t bias_raw = 0, bias_raw2 = 0;
   {
     const int t = tid / (M * 16);
     const int n = row0 + t * 16 + (tid & 15);
     if (bias != nullptr && t < ntiles && (t * 16 + (tid & 15)) < rows_blk) {
       bias_raw = reinterpret_cast<const uint16_t*>(bias)[n];
+    }
+    if (GLU && glu.bias2 != nullptr && t < ntiles && (t * 16 + (tid & 15)) < rows_blk) {
+      bias_raw2 = reinterpret_cast<const uint16_t*>(glu.bias2)[n];
     }
   }
 
@@ -570,14 +620,15 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   // kW4pDepth of them are requested now, before anything is waited for (for the usual shapes
   // that is all of them: the block's whole share of the weights is in flight at once)
   const uint8_t* wbase = w + (int64_t)row0 * (K >> 1) + kb * 16;
+  const uint8_t* wbase2 = GLU ? glu.w2 + (int64_t)row0 * (K >> 1) + kb * 16 : wbase;
   // Straight-line on purpose: a load under a branch (even a uniform one) makes the compiler
   // wait for everything in flight at the first LDS fill.  A slot without an item (live = false)
   // reads one and the same 16 bytes in every lane, a single cached request; lanes past the
   // block's rows re-read its first row (their outputs are never stored).
   auto issue = [&](int tile, int pair, u32x4 (&dst)[2], bool live) {
-    const int row_l = tile * 16 + r;
+    const int row_l = trow_of(tile) + r;
     const bool ok = row_l < rows_blk;
-    const uint8_t* p = wbase + (int64_t)(ok ? row_l : 0) * (K >> 1);
+    const uint8_t* p = (mat_of(tile) ? wbase2 : wbase) + (int64_t)(ok ? row_l : 0) * (K >> 1);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c = 2 * pair + u;
@@ -603,7 +654,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     // unconditional, so that the wait counts stay exact: a slot without an item reads one and
     // the same 16 bytes in every lane (a single cached request)
     {
-      const bool live = it_tile[d] < ntiles;
+      const bool live = it_tile[d] < nvt;
       issue(live ? it_tile[d] : 0, live ? it_pair[d] : 0, wq[d], live);
     }
   }
@@ -622,6 +673,35 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   for (int e = (s_aligned ? NT * 8 : 0) + tid; e < tile_halves; e += NT) {
     sl[e] = stile[e];
     if (ZMODE == kZeroAsym) zl[e] = ztile[e];
+  }
+  if (GLU) {
+    f16* sl2 = sl + rows_per_block * G;
+    f16* zl2 = zl + rows_per_block * G;
+    // (rows_per_block * G halves may leave sl2 off a 16-byte boundary: vector stores only
+    // when it is on one)
+    const bool lds_vec = ((rows_per_block * G) & 7) == 0;
+    if (s_vec2 && lds_vec) {
+      *reinterpret_cast<u32x4*>(sl2 + se) = sreg2;
+      if (ZMODE == kZeroAsym) *reinterpret_cast<u32x4*>(zl2 + se) = zreg2;
+    } else if (s_vec2) {
+      const f16x8 sv = __builtin_bit_cast(f16x8, sreg2);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sl2[se + j] = sv[j];
+      if (ZMODE == kZeroAsym) {
+        const f16x8 zv = __builtin_bit_cast(f16x8, zreg2);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) zl2[se + j] = zv[j];
+      }
+    } else if (se < tile_halves && s_aligned2) {
+      for (int j = se; j < tile_halves && j < se + 8; ++j) {
+        sl2[j] = stile2[j];
+        if (ZMODE == kZeroAsym) zl2[j] = ztile2[j];
+      }
+    }
+    for (int e = (s_aligned2 ? NT * 8 : 0) + tid; e < tile_halves; e += NT) {
+      sl2[e] = stile2[e];
+      if (ZMODE == kZeroAsym) zl2[e] = ztile2[e];
+    }
   }
   if (tid < 16) reinterpret_cast<uint32_t*>(zrec)[tid] = 0u;
 #pragma unroll
@@ -673,7 +753,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
 
   // one item = the chunk pair `pair` of tile `tile`, codes in slot d
   auto process = [&](int d, int tile, int pair) {
-    const f16* slr = sl + (tile * 16 + r) * G;
+    const f16* slr = sl + (srow_of(tile) + r) * G;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c = 2 * pair + u;
@@ -686,7 +766,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
         if (EXACT) {
           const f16 sh = slr[grp];
           f16 zh = (f16)0.0f;
-          if (ZMODE == kZeroAsym) zh = zl[(tile * 16 + r) * G + grp];
+          if (ZMODE == kZeroAsym) zh = zl[(srow_of(tile) + r) * G + grp];
           if (ZMODE == kZeroSymU) zh = (f16)(-7.0f) * sh;
           const f16x2 s2 = {sh, sh};
           const f16x2 z2 = {zh, zh};
@@ -745,7 +825,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     }
   };
   // items of this wave: wave, wave + NWAVES, ... < nitems
-  const int nitems = ntiles * npairs;
+  const int nitems = nvt * npairs;
   int left = nitems > wave ? (nitems - wave + NWAVES - 1) / NWAVES : 0;
   // steady state: every slot is consumed and refilled unconditionally, so the compiler's wait
   // before each slot is exact (the 2 * (kW4pDepth - 1) younger loads stay in flight)
@@ -789,7 +869,19 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     for (int wv = 0; wv < NWAVES; ++wv) sum += red[(t * NWAVES + wv) * M * 16 + rem];
     const int m = rem >> 4;
     const int row_l = t * 16 + (rem & 15);
-    if (row_l < rows_blk) {
+    if (GLU) {
+      float sum2 = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < NWAVES; ++wv) sum2 += red[((t + ntiles) * NWAVES + wv) * M * 16 + rem];
+      if (row_l < rows_blk) {
+        const int64_t o = (int64_t)m * N + row0 + row_l;
+        const f16 hidden = (f16)(sum + (float)bias_at_end(bias_raw));
+        const f16 gate = (f16)(sum2 + (float)bias_at_end(bias_raw2));
+        out[o] = hidden;
+        glu.out2[o] = gate;
+        glu.y[o] = hidden * (f16)glu_activation((float)gate, glu.act);
+      }
+    } else if (row_l < rows_blk) {
       out[(int64_t)m * N + row0 + row_l] = (f16)(sum + (float)bias_at_end(bias_raw));
     }
   }
@@ -863,11 +955,23 @@ gemv_w4p_f16_grouped(GemvGroup g, int M, int K, int group_size, int cpg_shift,
       cpg_shift, rows_per_block);
 }
 
+// two weights of equal shape (hidden state, gate), every block the same rows of both
+template<int NWAVES, bool EXACT, bool SIGNED, int ZMODE>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_w4p_f16_glu(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+                 const f16* __restrict__ scale, const f16* __restrict__ zero,
+                 const f16* __restrict__ bias, f16* __restrict__ out, GluArgs glu, int M, int N,
+                 int K, int group_size, int cpg_shift, int rows_per_block) {
+  gemv_w4p_body<NWAVES, 1, EXACT, SIGNED, ZMODE, true>(blockIdx.x, x, w, scale, zero, bias, out,
+                                                       M, N, K, group_size, cpg_shift,
+                                                       rows_per_block, glu);
+}
+
 inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,
-                                 bool exact, bool asym) {
+                                 bool exact, bool asym, int nmat = 1) {
   const int G = K / group_size;
   return (size_t)kW4pMaxTiles * nwaves * M * 16 * 4
-         + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15)
+         + (size_t)(asym ? 2 : 1) * ((nmat * rows_per_block * G * 2 + 15) & ~15)
          + (exact ? 0 : (size_t)(K >> 7) * 64) + 64 + (size_t)M * (K * 2 + 16);
 }
 

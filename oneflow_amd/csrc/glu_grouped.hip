@@ -256,6 +256,12 @@ extern "C" int ofq_fused_glu_gq(void* stream, const void* x, const void* w, cons
     a[1].zero = v_zero;
     a[1].bias = c;
     a[1].out = matmul_vx;
+    // decode, fp16, 4-bit codes: both linears and the gating as one launch
+    if (m <= 16 && t_dtype == OFQ_F16 && decode_args_ok(a[0]) && decode_args_ok(a[1])
+        && ofq_aligned16(y)) {
+      rc = launch_gemv_glu(st, a[0], a[1], y, activation);
+      if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+    }
     rc = run_group(stream, a, 2);
   } else {
     rc = run_single(stream, a[0]);

@@ -270,8 +270,10 @@ int launch_w4s(hipStream_t st, const LinearArgs& a) {
   const int cpg_shift = ilog2_exact(a.group_size / 128);
   // waves per block: as many as still let every block be resident at once (<= 24 waves per CU on
   // 256 CUs), so the kernel runs as a single round of blocks; never more than there are pairs
+  // and never fewer than fold the block's m * 16 outputs with one thread each
+  const int nw_min = a.m > 8 ? 4 : 2;
   int nw = 16;
-  while (nw > 2 && (tiles * nw > 6144 || nw > npairs)) nw >>= 1;
+  while (nw > nw_min && (tiles * nw > 6144 || nw > npairs)) nw >>= 1;
   const int nt = nw * 64;
   const int64_t nunits = a.m * a.k / 16;
   bool staged = nunits <= (int64_t)kGemvMaxUnits * nt;
@@ -453,7 +455,70 @@ int launch_w4p_grouped(hipStream_t st, const LinearArgs* pr, int count) {
   return OFQ_ERR_UNSUPPORTED;
 }
 
+template<int NW, bool EXACT, bool SIGNED, int ZMODE>
+int launch_w4p_glu_inst(hipStream_t st, const LinearArgs& a, const GluArgs& glu, int grid,
+                        int rows_per_block, size_t lds) {
+  auto kern = gemv_w4p_f16_glu<NW, EXACT, SIGNED, ZMODE>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
+                                  static_cast<const f16*>(a.scale),
+                                  static_cast<const f16*>(a.zero),
+                                  static_cast<const f16*>(a.bias), static_cast<f16*>(a.out), glu,
+                                  (int)a.m, (int)a.n, (int)a.k, (int)a.group_size,
+                                  ilog2_exact(a.group_size / 128), rows_per_block);
+  return ofq_check_launch();
+}
+
 }  // namespace
+
+int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act) {
+  if (!w4p_supported(a) || !w4p_supported(g)) return OFQ_ERR_UNSUPPORTED;
+  if (g.n != a.n || g.k != a.k || g.m != a.m || g.x != a.x) return OFQ_ERR_UNSUPPORTED;
+  constexpr int kCUs = 256;
+  // a block walks the same rows of both weights: half the tiles per weight
+  const int64_t max_rows = 16 * (kW4pMaxTiles / 2);
+  int64_t grid = kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
+  int rpb = (int)((a.n + grid - 1) / grid);
+  if (rpb < 16) rpb = 16;
+  grid = (a.n + rpb - 1) / rpb;
+  const bool two_per_cu = grid > kCUs;
+  const int nw = two_per_cu ? 8 : 16;
+  if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
+  if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) return OFQ_ERR_UNSUPPORTED;
+  const bool exact = !(a.symmetric && a.w_signed);
+  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                                        !a.symmetric, 2);
+  if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
+  GluArgs glu;
+  glu.w2 = static_cast<const uint8_t*>(g.w);
+  glu.scale2 = static_cast<const f16*>(g.scale);
+  glu.zero2 = static_cast<const f16*>(g.zero);
+  glu.bias2 = static_cast<const f16*>(g.bias);
+  glu.out2 = static_cast<f16*>(g.out);
+  glu.y = static_cast<f16*>(y);
+  glu.act = act;
+#define OFQ_W4PGLU(NWV)                                                                        \
+  if (nw == NWV) {                                                                             \
+    if (!exact)                                                                                \
+      return launch_w4p_glu_inst<NWV, false, true, kZeroNone>(st, a, glu, (int)grid, rpb, lds); \
+    if (a.symmetric)                                                                           \
+      return launch_w4p_glu_inst<NWV, true, false, kZeroSymU>(st, a, glu, (int)grid, rpb, lds); \
+    return launch_w4p_glu_inst<NWV, true, false, kZeroAsym>(st, a, glu, (int)grid, rpb, lds);  \
+  }
+  OFQ_W4PGLU(16) OFQ_W4PGLU(8)
+#undef OFQ_W4PGLU
+  return OFQ_ERR_UNSUPPORTED;
+}
 
 int launch_gemv_grouped(hipStream_t st, const LinearArgs* pr, int count) {
   if (count < 1 || count > kGemvMaxProblems) return OFQ_ERR_UNSUPPORTED;

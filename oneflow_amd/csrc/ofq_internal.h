@@ -40,6 +40,12 @@ int launch_gemv_wq(hipStream_t st, const LinearArgs& a);
 // OFQ_ERR_UNSUPPORTED when the shapes do not fit it (caller launches the problems one by one).
 int launch_gemv_grouped(hipStream_t st, const LinearArgs* problems, int count);
 
+// fused_glu in split mode for decode: hidden = x w~^T + b -> a.out, gate = x v~^T + c -> g.out,
+// y = hidden * act(gate), all in ONE launch (every block owns the same rows of both weights).
+// a and g differ in w / scale / zero / bias / out only.  OFQ_ERR_UNSUPPORTED when the shapes do
+// not fit (caller runs the linears and the gating separately).
+int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act);
+
 // Any shape / grouping; one wave per output element.
 int launch_linear_generic(hipStream_t st, const LinearArgs& a);
 

@@ -86,16 +86,18 @@ def _glu_call(L, _lib, torch, x, w, ws, wz, b, v, vs, vz, c, act, wcode, tcode, 
 
 
 @pytest.mark.parametrize("t", ["f16", "bf16", "f32"])
-@pytest.mark.parametrize("m,n,k", [(1, 1024, 512), (16, 344, 256), (40, 136, 256), (5, 37, 128)])
+@pytest.mark.parametrize("m,n,k", [(1, 1024, 512), (16, 344, 256), (40, 136, 256), (5, 37, 128),
+                                   (2, 9000, 256)])
 @pytest.mark.parametrize("split", [True, False])
-def test_glu_all_activations(t, m, n, k, split):
+@pytest.mark.parametrize("g", [64, 128])
+def test_glu_all_activations(t, m, n, k, split, g):
     import torch
     from oneflow_amd import _lib
     L = _lib.lib()
     tcode = {"f16": _lib.F16, "bf16": _lib.BF16, "f32": _lib.F32}[t]
     rng = np.random.Generator(np.random.PCG64(m + n + k))
-    bits, g = 4, 64
-    for symmetric, qdt in ((True, np.int8), (False, np.uint8)):
+    bits = 4
+    for symmetric, qdt in ((True, np.int8), (True, np.uint8), (False, np.uint8)):
         wcode = _lib.I8 if qdt == np.int8 else _lib.U8
         rows = n if split else 2 * n
         x, w, ws, wz, b = _problem(rng, m, rows, k, bits, symmetric, qdt, g, t)

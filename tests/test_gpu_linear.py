@@ -72,7 +72,8 @@ def test_decode_w4a16_llama_shapes(m, n, k, container):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 5000, 256), (3, 4099, 384), (16, 6000, 128), (2, 40000, 256),
-                                   (5, 33000, 128), (8, 4112, 1024)])
+                                   (5, 33000, 128), (8, 4112, 1024), (16, 688, 256), (12, 100, 128),
+                                   (9, 2048, 128)])
 @pytest.mark.parametrize("container", [np.int8, np.uint8])
 def test_decode_w4a16_row_balanced_shapes(m, n, k, container):
     """n large enough that a block owns more than one 16-row tile, with row counts per block
