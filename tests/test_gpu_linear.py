@@ -288,3 +288,52 @@ def test_midsize_m_split_k(m, n, k, num_bits):
             for got in outs:
                 H.assert_linear_parity(got, ref, t, f"m={m} n={n} k={k} {t} {symmetric} {qdt}")
             assert H.rel_l2(O.to_f32(outs[0]), O.to_f32(outs[1])) < 1e-3
+
+
+def test_decode_random_shape_sweep():
+    """Seeded sweep over the decode dispatch: m 1..16, ragged n, k from one chunk to many, group
+    sizes from one lane's load to the whole row, both code widths, all containers, fp16 and bf16:
+    every kernel variant and wave count the launchers can pick, each against the oracle."""
+    rng = np.random.Generator(np.random.PCG64(20240229))
+    n_cases = 0
+    for _ in range(90):
+        t = ("f16", "bf16")[int(rng.integers(0, 2))]
+        num_bits = (4, 8)[int(rng.integers(0, 2))]
+        m = int(rng.integers(1, 17))
+        ck = 128 if num_bits == 4 else 64
+        k = ck * int(rng.choice([1, 2, 3, 4, 8, 16, 32]))
+        n = int(rng.choice([1, 15, 16, 17, 100, 688, 1000, 2049, 4100]))
+        divisors = [g for g in (16, 32, 64, 128, 256, 512, k) if k % g == 0 and g % (ck // 4) == 0]
+        g = int(rng.choice(divisors))
+        symmetric, qdt = VARIANTS[int(rng.integers(0, 3))]
+        x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), t)
+        wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+        b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), t) if rng.integers(0, 2) else None
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, g, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        H.assert_linear_parity(got, ref, t, f"{t} b{num_bits} m={m} n={n} k={k} g={g} {symmetric} {qdt}")
+        n_cases += 1
+    assert n_cases == 90
+
+
+def test_prefill_random_shape_sweep():
+    """The same for m > 16 (tile shapes, K slices with a workspace, ragged edges)."""
+    rng = np.random.Generator(np.random.PCG64(777))
+    for _ in range(40):
+        t = ("f16", "bf16")[int(rng.integers(0, 2))]
+        num_bits = (4, 8)[int(rng.integers(0, 2))]
+        m = int(rng.choice([17, 31, 64, 129, 200, 257, 300]))
+        k = 64 * int(rng.choice([1, 2, 3, 8, 16, 24, 40]))
+        n = int(rng.choice([1, 31, 33, 127, 130, 353, 500]))
+        lane_k = 32 if num_bits == 4 else 16
+        divisors = [g for g in (16, 32, 64, 128, k) if k % g == 0 and g % lane_k == 0]
+        g = int(rng.choice(divisors))
+        symmetric, qdt = VARIANTS[int(rng.integers(0, 3))]
+        x = H.as_T((rng.standard_normal((m, k)) / 4).astype(np.float32), t)
+        wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+        b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), t) if rng.integers(0, 2) else None
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, g, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        H.assert_linear_parity(got, ref, t, f"{t} b{num_bits} m={m} n={n} k={k} g={g} {symmetric} {qdt}")
