@@ -308,6 +308,164 @@ gemv_rows_grouped(GemvGroup g, int M, int K, int group_size, int gs_shift, int r
       group_size, gs_shift, rows_per_block);
 }
 
+// ---------------------------------------------------------------------------------------------
+// 16 < m <= 64: the same row split with MT = 2 or 4 sixteen-row tiles of x per MFMA group.  A
+// weight tile is expanded once per chunk and meets all MT tiles of x, which come straight from
+// L2 (x is far too large for LDS here: m * k * 2 bytes per block); a wave walks chunks
+// c = wave, wave + NWAVES, ... and, per chunk, every 16-row weight tile of the block, with the
+// codes of the next (tile, chunk) requested before the current ones are used.  Sums stay in
+// registers (kRowsMaxTiles * MT accumulators) and are folded through LDS one weight tile at a
+// time.  No barrier inside the k loop, unlike the tiled GEMM, whose per-k-tile cost does not
+// shrink with m.
+// ---------------------------------------------------------------------------------------------
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, int MT>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_rows_mt(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
+             const uint16_t* __restrict__ scale, const uint16_t* __restrict__ zero,
+             const uint16_t* __restrict__ bias, uint16_t* __restrict__ out, int M, int N, int K,
+             int group_size, int gs_shift, int rows_per_block) {
+  typedef typename TT<T>::storage S;
+  static_assert(sizeof(S) == 2, "16-bit element types");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NT = NWAVES * 64;
+  constexpr int CK = BITS == 4 ? 128 : 64;
+  constexpr int LK = CK / 4;
+  constexpr int XV = LK / 8;
+  const int nchunks = K / CK;
+  const int row_bytes = nchunks * 64;
+  const int G = K / group_size;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15;
+  const int kb = lane >> 4;
+  const int row0 = blockIdx.x * rows_per_block;
+  int rows_blk = N - row0;
+  if (rows_blk > rows_per_block) rows_blk = rows_per_block;
+  if (rows_blk <= 0) return;
+  const int ntiles = (rows_blk + 15) >> 4;
+
+  // LDS: [red NWAVES*MT*256 f32][scales rows_per_block*G, padded to 16 B][zeros (asymmetric)]
+  float* red = reinterpret_cast<float*>(smem);
+  const int tile_bytes = (rows_per_block * G * 2 + 15) & ~15;
+  uint16_t* sl = reinterpret_cast<uint16_t*>(smem + (size_t)NWAVES * MT * 256 * 4);
+  uint16_t* zl = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
+
+  const uint8_t* wbase = w + (int64_t)row0 * row_bytes + kb * 16;
+  auto issue = [&](int tile, int c, bool live) {
+    const int row_l = tile * 16 + r;
+    const bool ok = row_l < rows_blk;
+    const uint8_t* q = wbase + (int64_t)(ok ? row_l : 0) * row_bytes + (int64_t)c * 64;
+    return __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4*>(live ? q : w + (int64_t)row0 * row_bytes));
+  };
+  int c = wave;
+  u32x4 cur = issue(0, c < nchunks ? c : 0, c < nchunks);
+
+  const int tile_halves = rows_blk * G;
+  const uint16_t* stile = scale + (int64_t)row0 * G;
+  const uint16_t* ztile = ZMODE == kZeroAsym ? zero + (int64_t)row0 * G : stile;
+  for (int e = tid; e < tile_halves; e += NT) {
+    sl[e] = stile[e];
+    if (ZMODE == kZeroAsym) zl[e] = ztile[e];
+  }
+  __syncthreads();
+
+  // this lane's rows of x: row mt*16 + r of every tile (rows >= M feed outputs never stored and
+  // re-read row 0), k-slot kb
+  const uint8_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int row = mt * 16 + r;
+    xrow[mt] = reinterpret_cast<const uint8_t*>(x) + ((size_t)(row < M ? row : 0) * K + kb * LK) * 2;
+  }
+  f32x4 acc[kRowsMaxTiles][MT];
+#pragma unroll
+  for (int t = 0; t < kRowsMaxTiles; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  while (c < nchunks) {
+    u32x4 xa[MT][XV];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const u32x4* xp = reinterpret_cast<const u32x4*>(xrow[mt] + (size_t)c * (CK * 2));
+#pragma unroll
+      for (int j = 0; j < XV; ++j) xa[mt][j] = xp[j];
+    }
+    const int k0 = c * CK + kb * LK;
+    const int grp = gs_shift >= 0 ? (k0 >> gs_shift) : (k0 / group_size);
+#pragma unroll
+    for (int t = 0; t < kRowsMaxTiles; ++t) {
+      if (t < ntiles) {
+        // codes of the next item first: the next tile of this chunk, else tile 0 of the wave's
+        // next chunk
+        const bool last_t = t + 1 >= ntiles;
+        const int nc = last_t ? c + NWAVES : c;
+        const bool live = nc < nchunks;
+        const u32x4 nxt = issue(last_t ? 0 : t + 1, live ? nc : 0, live);
+        const int srow = (t * 16 + r) * G;
+        const float s = TT<T>::load(reinterpret_cast<const S*>(sl) + srow + grp);
+        float z = 0.f;
+        if (ZMODE == kZeroAsym) z = TT<T>::load(reinterpret_cast<const S*>(zl) + srow + grp);
+        if (ZMODE == kZeroSymU) z = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * s);
+        if constexpr (BITS == 4) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u32x4 b = dequant8_b4<T, SIGNED, ZMODE>(cur[j], s, z);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[t][mt] = MfmaK32<T>::mma(xa[mt][j], b, acc[t][mt]);
+          }
+        } else {
+          u32x4 b0, b1;
+          dequant16_b8<T, SIGNED, ZMODE>(cur, s, z, b0, b1);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            acc[t][mt] = MfmaK32<T>::mma(xa[mt][0], b0, acc[t][mt]);
+            acc[t][mt] = MfmaK32<T>::mma(xa[mt][1], b1, acc[t][mt]);
+          }
+        }
+        cur = nxt;
+      }
+    }
+    c += NWAVES;
+  }
+
+  // fold, one weight tile at a time: red[wave][m (MT*16)][n (16)]
+#pragma unroll
+  for (int t = 0; t < kRowsMaxTiles; ++t) {
+    if (t < ntiles) {
+      if (t > 0) __syncthreads();  // the previous tile's sums have been read
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int m = mt * 16 + 4 * kb + v;
+          red[(wave * (MT * 16) + m) * 16 + r] = acc[t][mt][v];
+        }
+      __syncthreads();
+      for (int o = tid; o < M * 16; o += NT) {
+        float sum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < NWAVES; ++wv) sum += red[wv * (MT * 256) + o];
+        const int m = o >> 4;
+        const int row_l = t * 16 + (o & 15);
+        if (row_l < rows_blk) {
+          if (bias != nullptr) sum += TT<T>::load(reinterpret_cast<const S*>(bias) + row0 + row_l);
+          TT<T>::store(reinterpret_cast<S*>(out) + (int64_t)m * N + row0 + row_l, sum);
+        }
+      }
+    }
+  }
+}
+
+inline size_t gemv_rows_mt_lds_bytes(int nwaves, int mt, int K, int group_size,
+                                     int rows_per_block, bool asym) {
+  const int G = K / group_size;
+  return (size_t)nwaves * mt * 256 * 4
+         + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15);
+}
+
 inline size_t gemv_rows_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,
                                   bool asym, bool staged) {
   const int G = K / group_size;

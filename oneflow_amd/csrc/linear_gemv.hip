@@ -329,6 +329,70 @@ int launch_gemv_variant(hipStream_t st, const LinearArgs& a) {
   return ofq_check_launch();
 }
 
+// ---- 16 < m <= 128: several tiles of x per weight tile ----------------------------------------
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT>
+int launch_rows_mt_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m,
+                        int grid, int rows_per_block, size_t lds) {
+  auto kern = gemv_rows_mt<T, BITS, SIGNED, ZMODE, NW, MT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, NW * 64, lds, st>>>(
+      static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(a.w),
+      static_cast<const uint16_t*>(a.scale), static_cast<const uint16_t*>(a.zero),
+      static_cast<const uint16_t*>(a.bias), static_cast<uint16_t*>(out), m, (int)a.n, (int)a.k,
+      (int)a.group_size, ilog2_exact(a.group_size), rows_per_block);
+  return ofq_check_launch();
+}
+
+template<typename T, int NW, int MT>
+int launch_rows_mt_t(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m,
+                     int grid, int rpb, size_t lds) {
+  const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
+#define OFQ_R(B, SG, ZM)                                              \
+  if (a.bits == B && a.w_signed == SG && zmode == ZM)                 \
+    return launch_rows_mt_inst<T, B, SG, ZM, NW, MT>(st, a, x, out, m, grid, rpb, lds);
+  OFQ_R(4, true, kZeroNone)
+  OFQ_R(4, false, kZeroSymU)
+  OFQ_R(4, false, kZeroAsym)
+  OFQ_R(8, true, kZeroNone)
+  OFQ_R(8, false, kZeroSymU)
+  OFQ_R(8, false, kZeroAsym)
+#undef OFQ_R
+  return OFQ_ERR_UNSUPPORTED;
+}
+
+// rows [m0, m0 + m) of x, m <= 64
+int launch_rows_mt_part(hipStream_t st, const LinearArgs& a, int64_t m0, int m) {
+  constexpr int kCUs = 256;
+  const int64_t max_rows = 16 * kRowsMaxTiles;
+  int64_t grid = kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
+  int rpb = (int)((a.n + grid - 1) / grid);
+  if (rpb < 16) rpb = 16;
+  grid = (a.n + rpb - 1) / rpb;
+  const int mt = m <= 32 ? 2 : 4;
+  const int nw = mt == 2 ? 16 : 8;
+  const size_t lds =
+      gemv_rows_mt_lds_bytes(nw, mt, (int)a.k, (int)a.group_size, rpb, !a.symmetric);
+  if (lds > 160u * 1024u) return OFQ_ERR_UNSUPPORTED;
+  const size_t esz = 2;
+  const void* x = static_cast<const char*>(a.x) + (size_t)m0 * a.k * esz;
+  void* out = static_cast<char*>(a.out) + (size_t)m0 * a.n * esz;
+  if (a.t_dtype == OFQ_BF16) {
+    return mt == 2 ? launch_rows_mt_t<bf16, 16, 2>(st, a, x, out, m, (int)grid, rpb, lds)
+                   : launch_rows_mt_t<bf16, 8, 4>(st, a, x, out, m, (int)grid, rpb, lds);
+  }
+  return mt == 2 ? launch_rows_mt_t<f16, 16, 2>(st, a, x, out, m, (int)grid, rpb, lds)
+                 : launch_rows_mt_t<f16, 8, 4>(st, a, x, out, m, (int)grid, rpb, lds);
+}
+
 // ---- several problems, one launch -------------------------------------------------------------
 template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
 int launch_rows_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
@@ -567,6 +631,23 @@ int launch_gemv_grouped(hipStream_t st, const LinearArgs* pr, int count) {
 #undef OFQ_RG
 }
 
+bool gemv_mt_supported(const LinearArgs& a) {
+  // beyond 64 rows the weights would be walked twice and the tiled GEMM with K slices is faster
+  if (a.m <= 16 || a.m > 64) return false;
+  LinearArgs b = a;
+  b.m = 16;  // the same shape rules as the decode kernel
+  return rows_supported(b) && a.n * a.k <= 0x7FFFFFFFLL * 8;
+}
+
+int launch_gemv_mt(hipStream_t st, const LinearArgs& a) {
+  for (int64_t m0 = 0; m0 < a.m; m0 += 64) {
+    const int m = (int)(a.m - m0 < 64 ? a.m - m0 : 64);
+    const int rc = launch_rows_mt_part(st, a, m0, m);
+    if (rc != OFQ_OK) return rc;  // OFQ_ERR_UNSUPPORTED can only come from the first part
+  }
+  return OFQ_OK;
+}
+
 bool gemv_wq_supported(const LinearArgs& a) {
   if (rows_supported(a)) return true;
   if (a.t_dtype != OFQ_F16 || a.group_dim != 1 || a.m > 16 || a.m < 1) return false;
@@ -637,7 +718,7 @@ extern "C" size_t ofq_fused_linear_gq_workspace_bytes(int w_dtype, int t_dtype, 
   a.m = m;
   a.n = n;
   a.k = k;
-  if (gemv_wq_supported(a)) return 0;
+  if (gemv_wq_supported(a) || gemv_mt_supported(a)) return 0;
   return gemm_wq_workspace_bytes(a);  // 0 for every path but the two-pass GEMM at large m
 }
 
@@ -690,6 +771,10 @@ extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
   if (gemv_wq_supported(a)) {
     const int rc = launch_gemv_wq(st, a);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;  // e.g. bf16 with an x too large to stage
+  }
+  if (gemv_mt_supported(a)) {
+    const int rc = launch_gemv_mt(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
   }
   if (gemm_wq_supported(a)) return launch_gemm_wq(st, a, workspace, workspace_bytes);
   return launch_linear_generic(st, a);

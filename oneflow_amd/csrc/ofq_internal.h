@@ -35,6 +35,11 @@ int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t 
 bool gemv_wq_supported(const LinearArgs& a);
 int launch_gemv_wq(hipStream_t st, const LinearArgs& a);
 
+// 16 < m <= 64 without a workspace: the decode kernel's row split with several 16-row tiles of x
+// per weight tile.
+bool gemv_mt_supported(const LinearArgs& a);
+int launch_gemv_mt(hipStream_t st, const LinearArgs& a);
+
 // Up to 8 decode linears that share m, k, dtype and quantisation attributes (x, w, scale, zero,
 // bias, out and n per problem) as ONE launch of the natural-order decode kernel.
 // OFQ_ERR_UNSUPPORTED when the shapes do not fit it (caller launches the problems one by one).

@@ -248,11 +248,37 @@ def test_prefill_with_and_without_workspace():
         assert H.rel_l2(O.to_f32(outs[0]), O.to_f32(outs[1])) < 1e-3
 
 
-@pytest.mark.parametrize("m,n,k", [(17, 300, 1024), (100, 203, 1536), (130, 520, 2048),
-                                   (128, 1000, 4096), (300, 384, 1024)])
+@pytest.mark.parametrize("m,n,k,g", [(17, 300, 1024, 64), (32, 203, 1536, 128), (33, 4100, 512, 32),
+                                     (64, 1000, 4096, 128), (48, 129, 256, 64), (50, 2049, 384, 64),
+                                     (63, 700, 2048, 256)])
+@pytest.mark.parametrize("num_bits", [4, 8])
+@pytest.mark.parametrize("t", ["f16", "bf16"])
+def test_small_batch_multi_tile_kernel(m, n, k, g, num_bits, t):
+    """16 < m <= 64: the decode kernel's row split with 2 or 4 tiles of x per weight tile; needs
+    no workspace.  Ragged m, n, partial last blocks and tiles."""
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    rng = np.random.Generator(np.random.PCG64(m * 13 + n + num_bits))
+    x = H.as_T((rng.standard_normal((m, k)) / 4).astype(np.float32), t)
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), t)
+    tcode = _lib.F16 if t == "f16" else _lib.BF16
+    for symmetric, qdt in VARIANTS:
+        wcode = _lib.I8 if qdt == np.int8 else _lib.U8
+        assert L.ofq_fused_linear_gq_workspace_bytes(wcode, tcode, num_bits, int(symmetric), 1, g,
+                                                     m, n, k) == 0
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, g, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        r, e = H.assert_linear_parity(got, ref, t, f"{t} b{num_bits} m={m} n={n} k={k} {symmetric} {qdt}")
+        assert r < (3e-3 if t == "bf16" else 1e-4)
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 300, 1024), (128, 1000, 4096), (130, 520, 2048),
+                                   (300, 384, 1024), (257, 203, 1536)])
 @pytest.mark.parametrize("num_bits", [4, 8])
 def test_midsize_m_split_k(m, n, k, num_bits):
-    """16 < m < 1024 with few output tiles: given the workspace the op cuts K into slices that run
+    """64 < m < 1024 with few output tiles: given the workspace the op cuts K into slices that run
     as separate blocks and folds their fp32 partial sums; without it one block walks all of K.
     Both meet the contract and agree with each other up to summation order.  n not a multiple of
     4 takes the scalar fold."""

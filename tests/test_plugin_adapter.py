@@ -62,6 +62,7 @@ def test_registrations(plugin):
     assert tmp(K_BFLOAT16, K_UINT8, 2048, 11008, 4096, 8, 0, 1, 64) == 11008 * 4096 * 2
     assert tmp(K_FLOAT16, K_INT8, 1, 4096, 4096, 4, 1, 1, 128) == 0
     assert tmp(K_FLOAT16, K_INT8, 128, 4096, 4096, 4, 1, 1, 128) == 8 * 128 * 4096 * 4
+    assert tmp(K_FLOAT16, K_INT8, 64, 4096, 4096, 4, 1, 1, 128) == 0
     assert tmp(K_FLOAT16, K_INT8, 16, 4096, 4096, 4, 1, 1, 128) == 0
     assert tmp(K_FLOAT, K_UINT8, 2048, 4096, 4096, 8, 0, 1, 64) == 0
 
