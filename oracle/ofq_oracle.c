@@ -25,6 +25,17 @@
  *       the reference holds no such op (only the env-var name ONEFLOW_MLIR_GROUP_MATMUL_QUANT);
  *       semantics are defined by composition of reference rules and pinned by closed forms and an
  *       exact int64 GEMM.  PARITY WITH THE REFERENCE UNPINNED for these two.
+ *   groupwise_quantize, moving_average_min_max_observer:
+ *       pinned against an independent numpy restatement of the reference test's quantiser and
+ *       closed forms / hand-written fp32 step sequences.
+ *   skip_layer_norm input (skip_layer_norm_min_max_observer):
+ *       pinned bit for bit on the reference test's own composition (add bias, add skip*alpha,
+ *       layer_norm) evaluated in T with numpy and fed to the LayerNorm oracle above.
+ *   glu_gate:
+ *       'none' / 'relu' / sigmoid(0) exact closed forms; sigmoid, silu, gelu, fast_gelu against
+ *       float64 evaluations (scipy erf, numpy exp / tanh) to one rounding of T.  The reference's
+ *       architecture-dependent fp16 fast_gelu (tanh approximation instruction) is not restated:
+ *       PARITY UNPINNED for fast_gelu in fp16 against that variant.
  *   double precision observer/quantization paths and the "cambricon" formula:
  *       same code as f32 through a macro; cambricon pinned only by closed-form powers of two.
  */
