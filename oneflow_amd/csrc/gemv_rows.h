@@ -459,6 +459,157 @@ gemv_rows_mt(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// fp32 activations (the reference registers float next to half,
+// groupwise_quantization_kernels.cu:844-851): the same row split on v_mfma_f32_16x16x4_f32, one
+// fp32 value of x and one of w~ per lane and MFMA.  w~ = (float(q) * s) + z, both operations
+// rounded to fp32 as in the reference; products and sums are fp32 inside the matrix core.
+// x (m <= 16 rows) comes from L2.  Structure of gemv_rows_mt with a single tile of x.
+// ---------------------------------------------------------------------------------------------
+template<int BITS, bool SIGNED, int ZMODE, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64)
+gemv_rows_f32(const float* __restrict__ x, const uint8_t* __restrict__ w,
+              const float* __restrict__ scale, const float* __restrict__ zero,
+              const float* __restrict__ bias, float* __restrict__ out, int M, int N, int K,
+              int group_size, int gs_shift, int rows_per_block) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NT = NWAVES * 64;
+  constexpr int CK = BITS == 4 ? 128 : 64;
+  constexpr int LK = CK / 4;   // elements per lane and chunk
+  constexpr int XV = LK / 4;   // 16-byte pieces of x per lane and chunk
+  const int nchunks = K / CK;
+  const int row_bytes = nchunks * 64;
+  const int G = K / group_size;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15;
+  const int kb = lane >> 4;
+  const int row0 = blockIdx.x * rows_per_block;
+  int rows_blk = N - row0;
+  if (rows_blk > rows_per_block) rows_blk = rows_per_block;
+  if (rows_blk <= 0) return;
+  const int ntiles = (rows_blk + 15) >> 4;
+
+  // LDS: [red NWAVES*256 f32][scales rows_per_block*G f32][zeros (asymmetric)]
+  float* red = reinterpret_cast<float*>(smem);
+  float* sl = red + NWAVES * 256;
+  float* zl = sl + rows_per_block * G;
+
+  const uint8_t* wbase = w + (int64_t)row0 * row_bytes + kb * 16;
+  auto issue = [&](int tile, int c, bool live) {
+    const int row_l = tile * 16 + r;
+    const bool ok = row_l < rows_blk;
+    const uint8_t* q = wbase + (int64_t)(ok ? row_l : 0) * row_bytes + (int64_t)c * 64;
+    return __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4*>(live ? q : w + (int64_t)row0 * row_bytes));
+  };
+  int c = wave;
+  u32x4 cur = issue(0, c < nchunks ? c : 0, c < nchunks);
+
+  const int tile_elems = rows_blk * G;
+  const float* stile = scale + (int64_t)row0 * G;
+  const float* ztile = ZMODE == kZeroAsym ? zero + (int64_t)row0 * G : stile;
+  for (int e = tid; e < tile_elems; e += NT) {
+    sl[e] = stile[e];
+    if (ZMODE == kZeroAsym) zl[e] = ztile[e];
+  }
+  __syncthreads();
+
+  const float* xrow = x + (size_t)(r < M ? r : 0) * K + kb * LK;
+  f32x4 acc[kRowsMaxTiles];
+#pragma unroll
+  for (int t = 0; t < kRowsMaxTiles; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  while (c < nchunks) {
+    f32x4 xa[XV];
+#pragma unroll
+    for (int j = 0; j < XV; ++j) xa[j] = reinterpret_cast<const f32x4*>(xrow + (size_t)c * CK)[j];
+    const int k0 = c * CK + kb * LK;
+    const int grp = gs_shift >= 0 ? (k0 >> gs_shift) : (k0 / group_size);
+#pragma unroll
+    for (int t = 0; t < kRowsMaxTiles; ++t) {
+      if (t < ntiles) {
+        const bool last_t = t + 1 >= ntiles;
+        const int nc = last_t ? c + NWAVES : c;
+        const bool live = nc < nchunks;
+        const u32x4 nxt = issue(last_t ? 0 : t + 1, live ? nc : 0, live);
+        const int srow = (t * 16 + r) * G;
+        const float s = sl[srow + grp];
+        float z = 0.f;
+        if (ZMODE == kZeroAsym) z = zl[srow + grp];
+        if (ZMODE == kZeroSymU) z = -(float)((1 << (BITS - 1)) - 1) * s;
+        // a signed container is read as offset binary; the offset leaves inside the fused
+        // multiply-add (u * s - off * s is exact before its single rounding)
+        const float off = SIGNED ? -(float)(1 << (BITS - 1)) * s : 0.f;
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+          uint32_t word = cur[wd];
+          if (SIGNED) word ^= (BITS == 4 ? 0x88888888u : 0x80808080u);
+          if constexpr (BITS == 4) {
+            const uint32_t hi = (word >> 4) & 0x0F0F0F0Fu;  // elements 0, 2, 4, 6 of the word
+            const uint32_t lo = word & 0x0F0F0F0Fu;         // elements 1, 3, 5, 7
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              const float u0 = (float)((hi >> (8 * b)) & 0xFFu);
+              const float u1 = (float)((lo >> (8 * b)) & 0xFFu);
+              float w0 = SIGNED ? __builtin_fmaf(u0, s, off) : u0 * s;
+              float w1 = SIGNED ? __builtin_fmaf(u1, s, off) : u1 * s;
+              if (ZMODE != kZeroNone) {
+                w0 = w0 + z;
+                w1 = w1 + z;
+              }
+              // element 8*wd + 2*b (+1) of the lane's 32: piece 2*wd + b/2 of x, component 2*(b%2)
+              acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[2 * wd + (b >> 1)][2 * (b & 1)], w0,
+                                                            acc[t], 0, 0, 0);
+              acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[2 * wd + (b >> 1)][2 * (b & 1) + 1],
+                                                            w1, acc[t], 0, 0, 0);
+            }
+          } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              const float u0 = (float)((word >> (8 * b)) & 0xFFu);
+              float w0 = SIGNED ? __builtin_fmaf(u0, s, off) : u0 * s;
+              if (ZMODE != kZeroNone) w0 = w0 + z;
+              acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[wd][b], w0, acc[t], 0, 0, 0);
+            }
+          }
+        }
+        cur = nxt;
+      }
+    }
+    c += NWAVES;
+  }
+
+  // fold, one weight tile at a time: red[wave][m (16)][n (16)]
+#pragma unroll
+  for (int t = 0; t < kRowsMaxTiles; ++t) {
+    if (t < ntiles) {
+      if (t > 0) __syncthreads();
+#pragma unroll
+      for (int v = 0; v < 4; ++v) red[(wave * 16 + 4 * kb + v) * 16 + r] = acc[t][v];
+      __syncthreads();
+      for (int o = tid; o < M * 16; o += NT) {
+        float sum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < NWAVES; ++wv) sum += red[wv * 256 + o];
+        const int m = o >> 4;
+        const int row_l = t * 16 + (o & 15);
+        if (row_l < rows_blk) {
+          if (bias != nullptr) sum += bias[row0 + row_l];
+          out[(int64_t)m * N + row0 + row_l] = sum;
+        }
+      }
+    }
+  }
+}
+
+inline size_t gemv_rows_f32_lds_bytes(int nwaves, int K, int group_size, int rows_per_block,
+                                      bool asym) {
+  const int G = K / group_size;
+  return (size_t)nwaves * 256 * 4 + (size_t)(asym ? 2 : 1) * rows_per_block * G * 4;
+}
+
 inline size_t gemv_rows_mt_lds_bytes(int nwaves, int mt, int K, int group_size,
                                      int rows_per_block, bool asym) {
   const int G = K / group_size;

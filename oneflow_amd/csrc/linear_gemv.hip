@@ -393,6 +393,68 @@ int launch_rows_mt_part(hipStream_t st, const LinearArgs& a, int64_t m0, int m) 
                  : launch_rows_mt_t<f16, 8, 4>(st, a, x, out, m, (int)grid, rpb, lds);
 }
 
+// ---- fp32 activations -------------------------------------------------------------------------
+template<int BITS, bool SIGNED, int ZMODE>
+int launch_rows_f32_inst(hipStream_t st, const LinearArgs& a, const float* x, float* out, int m,
+                         int grid, int rows_per_block, size_t lds) {
+  auto kern = gemv_rows_f32<BITS, SIGNED, ZMODE, 16>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, 16 * 64, lds, st>>>(x, static_cast<const uint8_t*>(a.w),
+                                  static_cast<const float*>(a.scale),
+                                  static_cast<const float*>(a.zero),
+                                  static_cast<const float*>(a.bias), out, m, (int)a.n, (int)a.k,
+                                  (int)a.group_size, ilog2_exact(a.group_size), rows_per_block);
+  return ofq_check_launch();
+}
+
+bool rows_f32_supported(const LinearArgs& a) {
+  if (a.t_dtype != OFQ_F32 || (a.bits != 4 && a.bits != 8)) return false;
+  const int ck = a.bits == 4 ? 128 : 64;
+  return a.group_dim == 1 && a.m >= 1 && a.k % ck == 0 && a.group_size % (ck / 4) == 0
+         && a.k <= (1 << 20) && a.n <= 0x7FFFFFFF - 16 && (a.symmetric || !a.w_signed);
+}
+
+// any m: 16 rows of x per pass over the weights
+int launch_rows_f32(hipStream_t st, const LinearArgs& a) {
+  constexpr int kCUs = 256;
+  const int64_t max_rows = 16 * kRowsMaxTiles;
+  int64_t grid = kCUs;
+  if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
+  int rpb = (int)((a.n + grid - 1) / grid);
+  if (rpb < 16) rpb = 16;
+  grid = (a.n + rpb - 1) / rpb;
+  const size_t lds =
+      gemv_rows_f32_lds_bytes(16, (int)a.k, (int)a.group_size, rpb, !a.symmetric);
+  if (lds > 160u * 1024u) return OFQ_ERR_UNSUPPORTED;
+  const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
+  for (int64_t m0 = 0; m0 < a.m; m0 += 16) {
+    const int m = (int)(a.m - m0 < 16 ? a.m - m0 : 16);
+    const float* x = static_cast<const float*>(a.x) + m0 * a.k;
+    float* out = static_cast<float*>(a.out) + m0 * a.n;
+    int rc = OFQ_ERR_UNSUPPORTED;
+#define OFQ_R(B, SG, ZM)                                              \
+  if (a.bits == B && a.w_signed == SG && zmode == ZM)                 \
+    rc = launch_rows_f32_inst<B, SG, ZM>(st, a, x, out, m, (int)grid, rpb, lds);
+    OFQ_R(4, true, kZeroNone)
+    OFQ_R(4, false, kZeroSymU)
+    OFQ_R(4, false, kZeroAsym)
+    OFQ_R(8, true, kZeroNone)
+    OFQ_R(8, false, kZeroSymU)
+    OFQ_R(8, false, kZeroAsym)
+#undef OFQ_R
+    if (rc != OFQ_OK) return rc;
+  }
+  return OFQ_OK;
+}
+
 // ---- several problems, one launch -------------------------------------------------------------
 template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
 int launch_rows_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
@@ -690,6 +752,10 @@ int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
 }
 
 int launch_linear_generic(hipStream_t st, const LinearArgs& a) {
+  if (rows_f32_supported(a)) {
+    const int rc = launch_rows_f32(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   if (a.m > 65535) return OFQ_ERR_UNSUPPORTED;
   switch (a.t_dtype) {
     case OFQ_F16: return launch_generic_t<f16>(st, a);

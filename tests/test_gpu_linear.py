@@ -363,3 +363,24 @@ def test_prefill_random_shape_sweep():
         ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
         got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
         H.assert_linear_parity(got, ref, t, f"{t} b{num_bits} m={m} n={n} k={k} g={g} {symmetric} {qdt}")
+
+
+@pytest.mark.parametrize("m,n,k,g", [(1, 4096, 4096, 128), (7, 1000, 512, 64), (16, 4100, 256, 32),
+                                     (17, 300, 1024, 16), (40, 129, 128, 128), (3, 20000, 128, 64)])
+@pytest.mark.parametrize("num_bits", [4, 8])
+def test_fp32_activations(m, n, k, g, num_bits):
+    """T = float (registered by the reference next to half): the fp32 MFMA kernel, 16 rows of x
+    per pass over the weights; fp32 products and sums, so only the summation order differs from
+    the oracle."""
+    if num_bits == 4 and g % 32 != 0:
+        g = 32
+    rng = np.random.Generator(np.random.PCG64(m * 3 + n + num_bits))
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    b = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    for symmetric, qdt in VARIANTS:
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, g, qdt, "f32")
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        assert H.rel_l2(got, ref) < 2e-6, (symmetric, qdt)
+        assert np.allclose(got, ref, rtol=1e-4, atol=1e-4)
