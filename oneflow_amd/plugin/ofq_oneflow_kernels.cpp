@@ -13,6 +13,12 @@
 //   moving_average_min_max_observer               moving_average_min_max_observer_kernel.cu:306-314
 //   quantization                                  quantization_kernel.cu:149-156
 //   fake_quantization                             fake_quantization_kernel.cu:150-157
+// Added registrations (ops without a kernel in the reference tree; their op definitions would sit
+// next to OneFlowUserOps.td:8248-8387 with the argument names used here):
+//   fused_layer_norm_min_max_observer      x, [gamma], [beta], [bias], [skip] -> y, scale, zero_point
+//   matmul_quant                           a, b, a_scale, b_scale, [bias] -> out
+//   fused_glu_with_groupwise_quantized_weight      arguments of fused_glu + the weights' scales / zeros
+//   grouped_linear_with_groupwise_quantized_weight variadic xs, ws, w_scales, [w_zeros], [bs] -> ys
 // bf16 variants are added; kernels carry kKernelPriorityOptimized so that they win over stock
 // kernels registered for the same (op, device, dtype)
 // (oneflow/core/framework/user_op_registry_manager.cpp:95-114).
@@ -315,6 +321,249 @@ REGISTER_OFQ_QUANTIZATION("quantization", false, DataType::kDouble);
 REGISTER_OFQ_QUANTIZATION("fake_quantization", true, DataType::kFloat);
 REGISTER_OFQ_QUANTIZATION("fake_quantization", true, DataType::kDouble);
 
+// ---- fused_layer_norm_min_max_observer: x, [gamma], [beta], [bias], [skip] -> y, scale,
+//      zero_point (+ tmp_buffer); attrs epsilon, alpha (double), quantization_bit.  With bias /
+//      skip the normalised row is that of skip_layer_norm (skip_layer_norm_kernel.cu:36-67). ----
+class OfqLayerNormObserverKernel final : public user_op::OpKernel, public user_op::CudaGraphSupport {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx, user_op::OpKernelState*,
+               const user_op::OpKernelCache*) const override {
+    auto opt = [&](const char* name) -> const user_op::Tensor* {
+      return ctx->has_input(name, 0) ? ctx->Tensor4ArgNameAndIndex(name, 0) : nullptr;
+    };
+    const user_op::Tensor* x = ctx->Tensor4ArgNameAndIndex("x", 0);
+    const user_op::Tensor* gamma = opt("gamma");
+    const user_op::Tensor* beta = opt("beta");
+    const user_op::Tensor* bias = opt("bias");
+    const user_op::Tensor* skip = opt("skip");
+    user_op::Tensor* y = ctx->Tensor4ArgNameAndIndex("y", 0);
+    user_op::Tensor* scale = ctx->Tensor4ArgNameAndIndex("scale", 0);
+    user_op::Tensor* zero_point = ctx->Tensor4ArgNameAndIndex("zero_point", 0);
+    user_op::Tensor* tmp = ctx->Tensor4ArgNameAndIndex("tmp_buffer", 0);
+    CHECK_GE(x->shape_view().NumAxes(), 2);
+    const int64_t cols = x->shape_view().At(x->shape_view().NumAxes() - 1);
+    const int64_t rows = x->shape_view().elem_cnt() / cols;
+    if (gamma != nullptr) { CHECK_EQ(gamma->shape_view().elem_cnt(), cols); }
+    if (beta != nullptr) { CHECK_EQ(beta->shape_view().elem_cnt(), cols); }
+    if (bias != nullptr) { CHECK_EQ(bias->shape_view().elem_cnt(), cols); }
+    if (skip != nullptr) { CHECK(skip->shape_view() == x->shape_view()); }
+    CHECK_EQ(scale->data_type(), DataType::kFloat);
+    CHECK(tmp != nullptr);
+    const size_t tmp_bytes = (size_t)tmp->shape_view().elem_cnt();
+    const int dt = ToOfq(x->data_type());
+    if (bias != nullptr || skip != nullptr) {
+      CheckOk(ofq_fused_skip_layer_norm_min_max_observer(
+                  RawStream(ctx), x->dptr(), bias ? bias->dptr() : nullptr,
+                  skip ? skip->dptr() : nullptr, ctx->Attr<double>("alpha"),
+                  gamma ? gamma->dptr() : nullptr, beta ? beta->dptr() : nullptr, y->mut_dptr(),
+                  scale->mut_dptr<float>(), zero_point->mut_dptr<float>(), dt, rows, cols,
+                  ctx->Attr<double>("epsilon"), ctx->Attr<int32_t>("quantization_bit"),
+                  tmp->mut_dptr(), tmp_bytes),
+              "fused_skip_layer_norm_min_max_observer");
+    } else {
+      CheckOk(ofq_fused_layer_norm_min_max_observer(
+                  RawStream(ctx), x->dptr(), gamma ? gamma->dptr() : nullptr,
+                  beta ? beta->dptr() : nullptr, y->mut_dptr(), scale->mut_dptr<float>(),
+                  zero_point->mut_dptr<float>(), dt, rows, cols, ctx->Attr<double>("epsilon"),
+                  ctx->Attr<int32_t>("quantization_bit"), tmp->mut_dptr(), tmp_bytes),
+              "fused_layer_norm_min_max_observer");
+    }
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_LN_OBSERVER(dtype)                                                       \
+  REGISTER_USER_KERNEL("fused_layer_norm_min_max_observer")                                   \
+      .SetCreateFn<OfqLayerNormObserverKernel>()                                              \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)                        \
+                       && (user_op::HobDataType("y", 0) == dtype))                            \
+      .SetInferTmpSizeFn([](user_op::InferContext* ctx) -> size_t {                           \
+        const ShapeView xs = ctx->InputShape("x", 0);                                         \
+        const int64_t cols = xs.At(xs.NumAxes() - 1);                                         \
+        return ofq_fused_layer_norm_min_max_observer_workspace_bytes(ToOfq(dtype),            \
+                                                                     xs.elem_cnt() / cols,    \
+                                                                     cols);                   \
+      })                                                                                      \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_LN_OBSERVER(DataType::kFloat16);
+REGISTER_OFQ_LN_OBSERVER(DataType::kBFloat16);
+REGISTER_OFQ_LN_OBSERVER(DataType::kFloat);
+
+// ---- matmul_quant: a [m,k] int8, b [n,k] int8, a_scale [1] float, b_scale [n] float, [bias]
+//      -> out [m,n] (operand layout of fused_matmul_bias, OneFlowUserOps.td:5615-5633) ----------
+class OfqMatmulQuantKernel final : public user_op::OpKernel, public user_op::CudaGraphSupport {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx, user_op::OpKernelState*,
+               const user_op::OpKernelCache*) const override {
+    const user_op::Tensor* a = ctx->Tensor4ArgNameAndIndex("a", 0);
+    const user_op::Tensor* b = ctx->Tensor4ArgNameAndIndex("b", 0);
+    const user_op::Tensor* a_scale = ctx->Tensor4ArgNameAndIndex("a_scale", 0);
+    const user_op::Tensor* b_scale = ctx->Tensor4ArgNameAndIndex("b_scale", 0);
+    const user_op::Tensor* bias =
+        ctx->has_input("bias", 0) ? ctx->Tensor4ArgNameAndIndex("bias", 0) : nullptr;
+    user_op::Tensor* out = ctx->Tensor4ArgNameAndIndex("out", 0);
+    CHECK_EQ(a->data_type(), DataType::kInt8);
+    CHECK_EQ(b->data_type(), DataType::kInt8);
+    CHECK_EQ(a_scale->data_type(), DataType::kFloat);
+    CHECK_EQ(b_scale->data_type(), DataType::kFloat);
+    CHECK_GE(a->shape_view().NumAxes(), 2);
+    CHECK_EQ(b->shape_view().NumAxes(), 2);
+    const int64_t k = a->shape_view().At(a->shape_view().NumAxes() - 1);
+    const int64_t m = a->shape_view().elem_cnt() / k;
+    const int64_t n = b->shape_view().At(0);
+    CHECK_EQ(b->shape_view().At(1), k);
+    CHECK_EQ(a_scale->shape_view().elem_cnt(), 1);
+    CHECK_EQ(b_scale->shape_view().elem_cnt(), n);
+    if (bias != nullptr) {
+      CHECK_EQ(bias->shape_view().elem_cnt(), n);
+      CHECK_EQ(bias->data_type(), out->data_type());
+    }
+    CheckOk(ofq_matmul_quant(RawStream(ctx), a->dptr(), b->dptr(), a_scale->dptr<float>(),
+                             b_scale->dptr<float>(), bias ? bias->dptr() : nullptr,
+                             out->mut_dptr(), ToOfq(out->data_type()), m, n, k),
+            "matmul_quant");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_MATMUL_QUANT(dtype)                                    \
+  REGISTER_USER_KERNEL("matmul_quant")                                      \
+      .SetCreateFn<OfqMatmulQuantKernel>()                                  \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)      \
+                       && (user_op::HobDataType("out", 0) == dtype))        \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_MATMUL_QUANT(DataType::kFloat16);
+REGISTER_OFQ_MATMUL_QUANT(DataType::kBFloat16);
+REGISTER_OFQ_MATMUL_QUANT(DataType::kFloat);
+
+// ---- fused_glu_with_groupwise_quantized_weight: the arguments of fused_glu
+//      (x, w, [b], [v], [c] -> y, matmul_wx, [matmul_vx]; attr activation,
+//      fused_glu_kernel.cu:566-600) plus w_scale, [w_zero], [v_scale], [v_zero] and the
+//      quantisation attrs of the fused linear ----------------------------------------------------
+class OfqFusedGluKernel final : public user_op::OpKernel, public user_op::CudaGraphSupport {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx, user_op::OpKernelState*,
+               const user_op::OpKernelCache*) const override {
+    auto opt = [&](const char* name) -> const user_op::Tensor* {
+      return ctx->has_input(name, 0) ? ctx->Tensor4ArgNameAndIndex(name, 0) : nullptr;
+    };
+    auto ptr = [](const user_op::Tensor* t) -> const void* { return t ? t->dptr() : nullptr; };
+    const user_op::Tensor* x = ctx->Tensor4ArgNameAndIndex("x", 0);
+    const user_op::Tensor* w = ctx->Tensor4ArgNameAndIndex("w", 0);
+    const user_op::Tensor* w_scale = ctx->Tensor4ArgNameAndIndex("w_scale", 0);
+    const user_op::Tensor* v = opt("v");
+    user_op::Tensor* y = ctx->Tensor4ArgNameAndIndex("y", 0);
+    user_op::Tensor* matmul_wx = ctx->Tensor4ArgNameAndIndex("matmul_wx", 0);
+    user_op::Tensor* matmul_vx = ctx->Tensor4ArgNameAndIndex("matmul_vx", 0);
+    const std::string act = ctx->Attr<std::string>("activation");
+    int act_code = -1;
+    const char* names[] = {"none", "sigmoid", "relu", "gelu", "fast_gelu", "silu"};
+    for (int i = 0; i < 6; ++i) {
+      if (act == names[i]) act_code = i;
+    }
+    CHECK_GE(act_code, 0);
+    const int32_t num_bits = ctx->Attr<int32_t>("num_bits");
+    CHECK_GE(x->shape_view().NumAxes(), 2);
+    const int64_t k = x->shape_view().At(x->shape_view().NumAxes() - 1);
+    const int64_t m = x->shape_view().elem_cnt() / k;
+    CHECK_EQ(w->shape_view().NumAxes(), 2);
+    CHECK_EQ(w->shape_view().At(1) * (8 / num_bits), k);
+    const int64_t n = v != nullptr ? w->shape_view().At(0) : w->shape_view().At(0) / 2;
+    if (v != nullptr) {
+      CHECK(v->shape_view() == w->shape_view());
+      CHECK(matmul_vx != nullptr);
+    }
+    CHECK_EQ(y->shape_view().At(y->shape_view().NumAxes() - 1), n);
+    CheckOk(ofq_fused_glu_gq(RawStream(ctx), x->dptr(), w->dptr(), w_scale->dptr(),
+                             ptr(opt("w_zero")), ptr(opt("b")), ptr(v), ptr(opt("v_scale")),
+                             ptr(opt("v_zero")), ptr(opt("c")), y->mut_dptr(),
+                             matmul_wx->mut_dptr(), matmul_vx ? matmul_vx->mut_dptr() : nullptr,
+                             act_code, ToOfq(w->data_type()), ToOfq(x->data_type()), num_bits,
+                             ctx->Attr<bool>("symmetric") ? 1 : 0,
+                             (int)ctx->Attr<int64_t>("group_dim"),
+                             ctx->Attr<int64_t>("group_size"), m, n, k),
+            "fused_glu_with_groupwise_quantized_weight");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_FUSED_GLU(dtype)                                       \
+  REGISTER_USER_KERNEL("fused_glu_with_groupwise_quantized_weight")         \
+      .SetCreateFn<OfqFusedGluKernel>()                                     \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)      \
+                       && (user_op::HobDataType("y", 0) == dtype))          \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_FUSED_GLU(DataType::kFloat16);
+REGISTER_OFQ_FUSED_GLU(DataType::kBFloat16);
+REGISTER_OFQ_FUSED_GLU(DataType::kFloat);
+
+// ---- grouped_linear_with_groupwise_quantized_weight: variadic xs, ws, w_scales, [w_zeros],
+//      [bs] -> ys, walked like GroupedMatmulBiasKernel::Compute walks its tuples
+//      (grouped_matmul_bias.cu:153-190) ----------------------------------------------------------
+class OfqGroupedLinearKernel final : public user_op::OpKernel, public user_op::CudaGraphSupport {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx, user_op::OpKernelState*,
+               const user_op::OpKernelCache*) const override {
+    const int32_t count = ctx->input_size("xs");
+    CHECK_GE(count, 1);
+    CHECK_LE(count, 64);
+    CHECK_EQ(ctx->input_size("ws"), count);
+    CHECK_EQ(ctx->input_size("w_scales"), count);
+    const bool has_zeros = ctx->has_input("w_zeros", 0);
+    const bool has_biases = ctx->has_input("bs", 0);
+    if (has_zeros) { CHECK_EQ(ctx->input_size("w_zeros"), count); }
+    if (has_biases) { CHECK_EQ(ctx->input_size("bs"), count); }
+    const int32_t num_bits = ctx->Attr<int32_t>("num_bits");
+    const void* xs[64];
+    const void* ws[64];
+    const void* scales[64];
+    const void* zeros[64];
+    const void* bs[64];
+    void* ys[64];
+    int64_t ms[64], ns[64], ks[64];
+    for (int32_t i = 0; i < count; ++i) {
+      const user_op::Tensor* x = ctx->Tensor4ArgNameAndIndex("xs", i);
+      const user_op::Tensor* w = ctx->Tensor4ArgNameAndIndex("ws", i);
+      CHECK_GE(x->shape_view().NumAxes(), 2);
+      ks[i] = x->shape_view().At(x->shape_view().NumAxes() - 1);
+      ms[i] = x->shape_view().elem_cnt() / ks[i];
+      CHECK_EQ(w->shape_view().NumAxes(), 2);
+      CHECK_EQ(w->shape_view().At(1) * (8 / num_bits), ks[i]);
+      ns[i] = w->shape_view().At(0);
+      xs[i] = x->dptr();
+      ws[i] = w->dptr();
+      scales[i] = ctx->Tensor4ArgNameAndIndex("w_scales", i)->dptr();
+      zeros[i] = has_zeros ? ctx->Tensor4ArgNameAndIndex("w_zeros", i)->dptr() : nullptr;
+      bs[i] = has_biases ? ctx->Tensor4ArgNameAndIndex("bs", i)->dptr() : nullptr;
+      ys[i] = ctx->Tensor4ArgNameAndIndex("ys", i)->mut_dptr();
+    }
+    const user_op::Tensor* x0 = ctx->Tensor4ArgNameAndIndex("xs", 0);
+    const user_op::Tensor* w0 = ctx->Tensor4ArgNameAndIndex("ws", 0);
+    CheckOk(ofq_grouped_linear_gq(RawStream(ctx), count, xs, ws, scales,
+                                  has_zeros ? zeros : nullptr, has_biases ? bs : nullptr, ys, ms,
+                                  ns, ks, ToOfq(w0->data_type()), ToOfq(x0->data_type()), num_bits,
+                                  ctx->Attr<bool>("symmetric") ? 1 : 0,
+                                  (int)ctx->Attr<int64_t>("group_dim"),
+                                  ctx->Attr<int64_t>("group_size")),
+            "grouped_linear_with_groupwise_quantized_weight");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_GROUPED_LINEAR(dtype)                                  \
+  REGISTER_USER_KERNEL("grouped_linear_with_groupwise_quantized_weight")    \
+      .SetCreateFn<OfqGroupedLinearKernel>()                                \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)      \
+                       && (user_op::HobDataType("ys", 0) == dtype))         \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_GROUPED_LINEAR(DataType::kFloat16);
+REGISTER_OFQ_GROUPED_LINEAR(DataType::kBFloat16);
+REGISTER_OFQ_GROUPED_LINEAR(DataType::kFloat);
+
 }  // namespace oneflow
 
 #ifdef OFQ_PLUGIN_STANDALONE
@@ -431,6 +680,90 @@ extern "C" int ofq_plugin_run_fused_linear(void* stream, void* x, void* w, void*
   ctx.attrs["num_bits"].i = num_bits;
   ctx.attrs["symmetric"].b = symmetric != 0;
   ctx.attrs["group_dim"].i = group_dim;
+  ctx.attrs["group_size"].i = group_size;
+  auto kernel = r->create();
+  kernel->Compute(&ctx, nullptr, nullptr);
+  return 0;
+}
+// Runs the registered dynamic-int8 front end (LayerNorm + observer, with the optional residual
+// inputs) through a KernelComputeContext.
+extern "C" int ofq_plugin_run_layer_norm_observer(void* stream, void* x, void* gamma, void* beta,
+                                                  void* bias, void* skip, double alpha, void* y,
+                                                  void* scale, void* zero_point, void* tmp,
+                                                  long long tmp_bytes, int t_dtype, long long rows,
+                                                  long long cols, double epsilon, int bits) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["y"] = (DataType)t_dtype;
+  const auto* r = Lookup("fused_layer_norm_min_max_observer", c);
+  if (r == nullptr) return -1;
+  RawStreamHolder st(stream);
+  user_op::KernelComputeContext ctx;
+  ctx.stream_ = &st;
+  const DataType T = (DataType)t_dtype;
+  ctx.AddTensor("x", {rows, cols}, T, x);
+  if (gamma) ctx.AddTensor("gamma", {cols}, T, gamma);
+  if (beta) ctx.AddTensor("beta", {cols}, T, beta);
+  if (bias) ctx.AddTensor("bias", {cols}, T, bias);
+  if (skip) ctx.AddTensor("skip", {rows, cols}, T, skip);
+  ctx.AddTensor("y", {rows, cols}, T, y);
+  ctx.AddTensor("scale", {1}, DataType::kFloat, scale);
+  ctx.AddTensor("zero_point", {1}, DataType::kFloat, zero_point);
+  ctx.AddTensor("tmp_buffer", {tmp_bytes}, DataType::kUInt8, tmp);
+  ctx.attrs["epsilon"].f = epsilon;
+  ctx.attrs["alpha"].f = alpha;
+  ctx.attrs["quantization_bit"].i = bits;
+  auto kernel = r->create();
+  kernel->Compute(&ctx, nullptr, nullptr);
+  return 0;
+}
+
+extern "C" int ofq_plugin_run_matmul_quant(void* stream, void* a, void* b, void* a_scale,
+                                           void* b_scale, void* bias, void* out, int out_dtype,
+                                           long long m, long long n, long long k) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["out"] = (DataType)out_dtype;
+  const auto* r = Lookup("matmul_quant", c);
+  if (r == nullptr) return -1;
+  RawStreamHolder st(stream);
+  user_op::KernelComputeContext ctx;
+  ctx.stream_ = &st;
+  ctx.AddTensor("a", {m, k}, DataType::kInt8, a);
+  ctx.AddTensor("b", {n, k}, DataType::kInt8, b);
+  ctx.AddTensor("a_scale", {1}, DataType::kFloat, a_scale);
+  ctx.AddTensor("b_scale", {n}, DataType::kFloat, b_scale);
+  if (bias) ctx.AddTensor("bias", {n}, (DataType)out_dtype, bias);
+  ctx.AddTensor("out", {m, n}, (DataType)out_dtype, out);
+  auto kernel = r->create();
+  kernel->Compute(&ctx, nullptr, nullptr);
+  return 0;
+}
+
+// q/k/v-style grouped call: `count` problems sharing x ([m,k]) with weights [ns[i], k*bits/8]
+// (symmetric, groups along K), outputs ys[i] [m, ns[i]]
+extern "C" int ofq_plugin_run_grouped_linear(void* stream, int count, void* x, void** ws,
+                                             void** scales, void** ys, const long long* ns,
+                                             int t_dtype, int w_dtype, long long m, long long k,
+                                             int num_bits, long long group_size) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["ys"] = (DataType)t_dtype;
+  const auto* r = Lookup("grouped_linear_with_groupwise_quantized_weight", c);
+  if (r == nullptr) return -1;
+  RawStreamHolder st(stream);
+  user_op::KernelComputeContext ctx;
+  ctx.stream_ = &st;
+  const DataType T = (DataType)t_dtype;
+  for (int i = 0; i < count; ++i) {
+    ctx.AddTensor("xs", {m, k}, T, x, i);
+    ctx.AddTensor("ws", {ns[i], k * num_bits / 8}, (DataType)w_dtype, ws[i], i);
+    ctx.AddTensor("w_scales", {ns[i], k / group_size}, T, scales[i], i);
+    ctx.AddTensor("ys", {m, ns[i]}, T, ys[i], i);
+  }
+  ctx.attrs["num_bits"].i = num_bits;
+  ctx.attrs["symmetric"].b = true;
+  ctx.attrs["group_dim"].i = 1;
   ctx.attrs["group_size"].i = group_size;
   auto kernel = r->create();
   kernel->Compute(&ctx, nullptr, nullptr);

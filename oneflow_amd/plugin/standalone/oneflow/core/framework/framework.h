@@ -106,9 +106,17 @@ class KernelComputeContext {
   T Attr(const std::string& name) const;
   ep::Stream* stream() { return stream_; }
 
+  // number of tensors bound to a variadic argument (user_op::KernelComputeContext::input_size)
+  int32_t input_size(const std::string& name) const {
+    int32_t n = 0;
+    while (tensors_.count({name, n}) != 0) ++n;
+    return n;
+  }
+
   // test-side helpers
-  void AddTensor(const std::string& name, std::vector<int64_t> shape, DataType dt, void* ptr) {
-    tensors_[{name, 0}] = std::make_unique<Tensor>(std::move(shape), dt, ptr);
+  void AddTensor(const std::string& name, std::vector<int64_t> shape, DataType dt, void* ptr,
+                 int32_t index = 0) {
+    tensors_[{name, index}] = std::make_unique<Tensor>(std::move(shape), dt, ptr);
   }
   std::map<std::string, AttrValue> attrs;
   ep::Stream* stream_ = nullptr;

@@ -31,7 +31,15 @@ def test_registrations(plugin):
         seen.setdefault(name.value.decode(), []).append((prio.value, tmp.value))
     assert set(seen) == {"groupwise_dequantize", "fused_linear_with_groupwise_quantized_weight",
                          "min_max_observer", "moving_average_min_max_observer", "quantization",
-                         "fake_quantization"}
+                         "fake_quantization", "fused_layer_norm_min_max_observer", "matmul_quant",
+                         "fused_glu_with_groupwise_quantized_weight",
+                         "grouped_linear_with_groupwise_quantized_weight"}
+    for name in ("fused_layer_norm_min_max_observer", "matmul_quant",
+                 "fused_glu_with_groupwise_quantized_weight",
+                 "grouped_linear_with_groupwise_quantized_weight"):
+        assert len(seen[name]) == 3  # half, bfloat16, float
+    assert all(t == 1 for _, t in seen["fused_layer_norm_min_max_observer"])
+    assert all(t == 0 for _, t in seen["matmul_quant"])
     assert len(seen["groupwise_dequantize"]) == 3 and len(seen["min_max_observer"]) == 2
     assert len(seen["moving_average_min_max_observer"]) == 2
     # every kernel outranks a stock registration (priority 0); the observers and the fused linear
@@ -49,6 +57,10 @@ def test_registrations(plugin):
     assert has(b"quantization", K_CUDA, b"in", K_DOUBLE) == 1
     assert has(b"quantization", K_CUDA, b"in", K_FLOAT16) == 0
     assert has(b"matmul", K_CUDA, b"out", K_FLOAT16) == 0
+    assert has(b"matmul_quant", K_CUDA, b"out", K_FLOAT16) == 1
+    assert has(b"matmul_quant", K_CUDA, b"out", K_DOUBLE) == 0
+    assert has(b"fused_layer_norm_min_max_observer", K_CUDA, b"y", K_BFLOAT16) == 1
+    assert has(b"grouped_linear_with_groupwise_quantized_weight", K_CPU, b"ys", K_FLOAT16) == 0
     plugin.ofq_plugin_observer_tmp_bytes.restype = ctypes.c_longlong
     shape = (ctypes.c_longlong * 2)(4096, 4096)
     assert plugin.ofq_plugin_observer_tmp_bytes(K_FLOAT, shape, 2, 0) == 4096 * 2 * 4
@@ -90,3 +102,76 @@ def test_fused_linear_through_the_adapter(plugin):
     assert rc == 0
     torch.cuda.synchronize()
     assert torch.equal(out, direct)
+
+
+@pytest.mark.gpu
+def test_dynamic_int8_ops_through_the_adapter(plugin):
+    """fused_layer_norm_min_max_observer (plain and with the skip_layer_norm inputs) and
+    matmul_quant looked up from the registry and run through a KernelComputeContext: the same bits
+    as the direct calls."""
+    import torch
+    import helpers as H
+    import oneflow_amd as flow
+    rng = np.random.default_rng(12)
+    rows, cols = 64, 1024
+    x = H.to_torch(rng.standard_normal((rows, cols)).astype(np.float16))
+    skip = H.to_torch(rng.standard_normal((rows, cols)).astype(np.float16))
+    gamma = H.to_torch((1 + 0.1 * rng.standard_normal(cols)).astype(np.float16))
+    beta = H.to_torch((0.1 * rng.standard_normal(cols)).astype(np.float16))
+    vp, ll, dbl, ci = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_double, ctypes.c_int
+    run = plugin.ofq_plugin_run_layer_norm_observer
+    run.argtypes = [vp] * 6 + [dbl] + [vp] * 4 + [ll, ci, ll, ll, dbl, ci]
+    stream = torch.cuda.current_stream().cuda_stream
+    for sk in (None, skip):
+        if sk is None:
+            want = flow._C.fused_layer_norm_min_max_observer(x, gamma, beta, 1e-5, 8)
+        else:
+            want = flow._C.fused_skip_layer_norm_min_max_observer(x, gamma, beta, None, sk, 1e-5, 0.5, 8)
+        y = torch.empty_like(x)
+        s = torch.empty(1, dtype=torch.float32, device="cuda")
+        z = torch.empty(1, dtype=torch.float32, device="cuda")
+        tmp = torch.empty(rows * 4, dtype=torch.uint8, device="cuda")
+        rc = run(stream, x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), None,
+                 sk.data_ptr() if sk is not None else None, 0.5, y.data_ptr(), s.data_ptr(),
+                 z.data_ptr(), tmp.data_ptr(), rows * 4, K_FLOAT16, rows, cols, 1e-5, 8)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[0]) and torch.equal(s, want[1]) and torch.equal(z, want[2])
+    m, n, k = 48, 200, 256
+    a = H.to_torch(rng.integers(-128, 128, size=(m, k)).astype(np.int8))
+    b = H.to_torch(rng.integers(-127, 128, size=(n, k)).astype(np.int8))
+    a_s = H.to_torch(np.array([0.02], np.float32))
+    b_s = H.to_torch(rng.uniform(1e-3, 1e-2, size=n).astype(np.float32))
+    want = flow._C.matmul_quant(a, b, a_s, b_s, None, torch.float16)
+    out = torch.empty_like(want)
+    mq = plugin.ofq_plugin_run_matmul_quant
+    mq.argtypes = [vp] * 7 + [ci, ll, ll, ll]
+    assert mq(stream, a.data_ptr(), b.data_ptr(), a_s.data_ptr(), b_s.data_ptr(), None,
+              out.data_ptr(), K_FLOAT16, m, n, k) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+
+
+@pytest.mark.gpu
+def test_grouped_linear_through_the_adapter(plugin):
+    import torch
+    import helpers as H
+    import oneflow_amd as flow
+    rng = np.random.default_rng(13)
+    m, k, g, ns = 2, 512, 128, (256, 64, 64)
+    x = H.to_torch(rng.standard_normal((m, k)).astype(np.float16))
+    ws = [H.to_torch(rng.integers(-128, 128, size=(n, k // 2)).astype(np.int8)) for n in ns]
+    scs = [H.to_torch(rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float16)) for n in ns]
+    want = flow._C.grouped_linear_with_groupwise_quantized_weight(
+        [x] * 3, ws, scs, num_bits=4, symmetric=True, group_dim=1, group_size=g)
+    outs = [torch.empty_like(w) for w in want]
+    vp, ll, ci = ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int
+    arr = lambda ts: (vp * 3)(*[t.data_ptr() for t in ts])
+    run = plugin.ofq_plugin_run_grouped_linear
+    run.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ll, ll, ci, ll]
+    rc = run(torch.cuda.current_stream().cuda_stream, 3, x.data_ptr(), arr(ws), arr(scs), arr(outs),
+             (ll * 3)(*ns), K_FLOAT16, K_INT8, m, k, 4, g)
+    assert rc == 0
+    torch.cuda.synchronize()
+    for o, w in zip(outs, want):
+        assert torch.equal(o, w)
