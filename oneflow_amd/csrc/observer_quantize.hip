@@ -26,8 +26,55 @@ __host__ __device__ inline int64_t obs_splits(int64_t inner) {
 }
 
 template<typename T>
+__device__ __forceinline__ T t_rint(T v);
+template<>
+__device__ __forceinline__ float t_rint<float>(float v) {
+  return __builtin_rintf(v);
+}
+template<>
+__device__ __forceinline__ double t_rint<double>(double v) {
+  return __builtin_rint(v);
+}
+template<typename T>
+__device__ __forceinline__ T t_abs(T v) {
+  return v < 0 ? -v : (v == 0 ? (T)0 : v);
+}
+
+// scale / zero point of one channel from its extremes
+// (oneflow/user/kernels/min_max_observer_kernel.cpp:22-58)
+template<typename T>
+__device__ __forceinline__ void observer_channel(T vmax, T vmin, int bits, int scheme, int formula,
+                                                 T* __restrict__ scale,
+                                                 T* __restrict__ zero_point) {
+  if (formula == OFQ_FORMULA_CAMBRICON) {
+    const T a = t_abs(vmax), b = t_abs(vmin);
+    const T m = a < b ? b : a;
+    // floor(log2(m)) with log2 evaluated in double and rounded to T, which is what a correctly
+    // rounded libm log2 of the CPU kernel returns (min_max_observer_kernel.cpp:55)
+    const T lg = (T)log2((double)m);
+    *scale = floor(lg) - (T)(bits - 2);
+    *zero_point = 0;
+  } else if (scheme == OFQ_SCHEME_SYMMETRIC) {
+    const T a = t_abs(vmax), b = t_abs(vmin);
+    const T m = a < b ? b : a;
+    const T denominator = (T)(1 << (bits - 1)) - 1;
+    *scale = m / denominator;
+    *zero_point = 0;
+  } else {
+    const T denominator = (T)(1 << bits) - 1;
+    const T s = (vmax - vmin) / denominator;
+    *scale = s;
+    *zero_point = -t_rint<T>(vmin / s);
+  }
+}
+
+// DIRECT: a channel is a single slice (splits == 1), so the block that reduced it writes its
+// scale and zero point itself and no second launch is needed.
+template<typename T, bool DIRECT>
 __global__ void __launch_bounds__(kObsBlock)
-observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, T* __restrict__ part) {
+observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, T* __restrict__ part,
+                 int bits, int scheme, int formula, T* __restrict__ scale,
+                 T* __restrict__ zero_point) {
   __shared__ T smem[kObsBlock / kWave];
   const int64_t c = blockIdx.x / splits;
   const int64_t sp = blockIdx.x % splits;
@@ -73,24 +120,14 @@ observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, T* __r
   vmax = block_reduce(vmax, OpMax(), smem);
   vmin = block_reduce(vmin, OpMin(), smem);
   if (threadIdx.x == 0) {
-    part[2 * blockIdx.x] = vmax;
-    part[2 * blockIdx.x + 1] = vmin;
+    if (DIRECT) {
+      observer_channel<T>(vmax, vmin, bits, scheme, formula, scale + blockIdx.x,
+                          zero_point + blockIdx.x);
+    } else {
+      part[2 * blockIdx.x] = vmax;
+      part[2 * blockIdx.x + 1] = vmin;
+    }
   }
-}
-
-template<typename T>
-__device__ __forceinline__ T t_rint(T v);
-template<>
-__device__ __forceinline__ float t_rint<float>(float v) {
-  return __builtin_rintf(v);
-}
-template<>
-__device__ __forceinline__ double t_rint<double>(double v) {
-  return __builtin_rint(v);
-}
-template<typename T>
-__device__ __forceinline__ T t_abs(T v) {
-  return v < 0 ? -v : (v == 0 ? (T)0 : v);
 }
 
 template<typename T>
@@ -105,26 +142,7 @@ observer_finalize(const T* __restrict__ part, int64_t channels, int64_t splits, 
     vmax = OpMax()(vmax, part[2 * (c * splits + s)]);
     vmin = OpMin()(vmin, part[2 * (c * splits + s) + 1]);
   }
-  if (formula == OFQ_FORMULA_CAMBRICON) {
-    const T a = t_abs(vmax), b = t_abs(vmin);
-    const T m = a < b ? b : a;
-    // floor(log2(m)) with log2 evaluated in double and rounded to T, which is what a correctly
-    // rounded libm log2 of the CPU kernel returns (min_max_observer_kernel.cpp:55)
-    const T lg = (T)log2((double)m);
-    scale[c] = floor(lg) - (T)(bits - 2);
-    zero_point[c] = 0;
-  } else if (scheme == OFQ_SCHEME_SYMMETRIC) {
-    const T a = t_abs(vmax), b = t_abs(vmin);
-    const T m = a < b ? b : a;
-    const T denominator = (T)(1 << (bits - 1)) - 1;
-    scale[c] = m / denominator;
-    zero_point[c] = 0;
-  } else {
-    const T denominator = (T)(1 << bits) - 1;
-    const T s = (vmax - vmin) / denominator;
-    scale[c] = s;
-    zero_point[c] = -t_rint<T>(vmin / s);
-  }
+  observer_channel<T>(vmax, vmin, bits, scheme, formula, scale + c, zero_point + c);
 }
 
 // ---- moving_average_min_max_observer ------------------------------------------------------------
@@ -412,6 +430,27 @@ int check_quant_args(const void* in, const void* scale, const void* zero_point, 
 }
 
 }  // namespace
+template<typename T>
+int launch_observer(hipStream_t st, const void* in, void* workspace, void* scale,
+                    void* zero_point, int64_t channels, int64_t inner, int64_t splits, int bits,
+                    int scheme, int formula) {
+  const T* src = static_cast<const T*>(in);
+  T* sc = static_cast<T*>(scale);
+  T* zp = static_cast<T*>(zero_point);
+  if (splits == 1) {
+    observer_partial<T, true><<<(int)channels, kObsBlock, 0, st>>>(src, inner, 1, nullptr, bits,
+                                                                  scheme, formula, sc, zp);
+    return ofq_check_launch();
+  }
+  T* part = static_cast<T*>(workspace);
+  observer_partial<T, false><<<(int)(channels * splits), kObsBlock, 0, st>>>(
+      src, inner, splits, part, bits, scheme, formula, nullptr, nullptr);
+  const int fin_grid = (int)((channels + kObsBlock - 1) / kObsBlock);
+  observer_finalize<T><<<fin_grid, kObsBlock, 0, st>>>(part, channels, splits, bits, scheme,
+                                                       formula, sc, zp);
+  return ofq_check_launch();
+}
+
 }  // namespace ofq
 
 using namespace ofq;
@@ -445,21 +484,12 @@ extern "C" int ofq_min_max_observer(void* stream, const void* in, void* scale, v
   const int64_t splits = obs_splits(inner);
   OFQ_RETURN_IF(channels * splits > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const int fin_grid = (int)((channels + kObsBlock - 1) / kObsBlock);
   if (in_dtype == OFQ_F32) {
-    observer_partial<float><<<(int)(channels * splits), kObsBlock, 0, st>>>(
-        static_cast<const float*>(in), inner, splits, static_cast<float*>(workspace));
-    observer_finalize<float><<<fin_grid, kObsBlock, 0, st>>>(
-        static_cast<const float*>(workspace), channels, splits, quantization_bit, scheme, formula,
-        static_cast<float*>(scale), static_cast<float*>(zero_point));
-  } else {
-    observer_partial<double><<<(int)(channels * splits), kObsBlock, 0, st>>>(
-        static_cast<const double*>(in), inner, splits, static_cast<double*>(workspace));
-    observer_finalize<double><<<fin_grid, kObsBlock, 0, st>>>(
-        static_cast<const double*>(workspace), channels, splits, quantization_bit, scheme, formula,
-        static_cast<double*>(scale), static_cast<double*>(zero_point));
+    return launch_observer<float>(st, in, workspace, scale, zero_point, channels, inner, splits,
+                                  quantization_bit, scheme, formula);
   }
-  return ofq_check_launch();
+  return launch_observer<double>(st, in, workspace, scale, zero_point, channels, inner, splits,
+                                 quantization_bit, scheme, formula);
 }
 
 extern "C" size_t ofq_moving_average_min_max_observer_workspace_bytes(int in_dtype,
@@ -492,16 +522,18 @@ extern "C" int ofq_moving_average_min_max_observer(
   // The extremes are reduced whether or not this step updates the moving values: whether it does
   // is known on the device only.
   if (in_dtype == OFQ_F32) {
-    observer_partial<float><<<(int)splits, kObsBlock, 0, st>>>(
-        static_cast<const float*>(in), elem_cnt, splits, static_cast<float*>(workspace));
+    observer_partial<float, false><<<(int)splits, kObsBlock, 0, st>>>(
+        static_cast<const float*>(in), elem_cnt, splits, static_cast<float*>(workspace), 0, 0, 0,
+        nullptr, nullptr);
     moving_average_finalize<float><<<1, kWave, 0, st>>>(
         static_cast<const float*>(workspace), splits, current_train_step, stop_update_after_iters,
         training, momentum, quantization_bit, scheme, formula, static_cast<float*>(moving_max),
         static_cast<float*>(moving_min), static_cast<float*>(scale),
         static_cast<float*>(zero_point));
   } else {
-    observer_partial<double><<<(int)splits, kObsBlock, 0, st>>>(
-        static_cast<const double*>(in), elem_cnt, splits, static_cast<double*>(workspace));
+    observer_partial<double, false><<<(int)splits, kObsBlock, 0, st>>>(
+        static_cast<const double*>(in), elem_cnt, splits, static_cast<double*>(workspace), 0, 0,
+        0, nullptr, nullptr);
     moving_average_finalize<double><<<1, kWave, 0, st>>>(
         static_cast<const double*>(workspace), splits, current_train_step,
         stop_update_after_iters, training, momentum, quantization_bit, scheme, formula,
