@@ -135,3 +135,57 @@ class QuantizedLinear(torch.nn.Module):
     def extra_repr(self):
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
                 f"num_bits={self.num_bits}, symmetric={self.symmetric}, group_size={self.group_size}")
+
+
+class QuantizedGLU(torch.nn.Module):
+    """``y = (x W^T + b) * act(x V^T + c)`` over two ``QuantizedLinear`` weights of equal shape
+    (``hidden`` = W, b and ``gate`` = V, c) through ``_C.fused_glu_with_groupwise_quantized_weight``
+    -- a Llama MLP's ``up_proj`` / ``gate_proj`` pair with ``activation="silu"``."""
+
+    def __init__(self, hidden, gate, activation="silu"):
+        super().__init__()
+        for a in ("in_features", "out_features", "num_bits", "symmetric", "group_size"):
+            if getattr(hidden, a) != getattr(gate, a):
+                raise ValueError(f"hidden and gate differ in {a}")
+        if (hidden.bias is None) != (gate.bias is None):
+            raise ValueError("hidden and gate should both have a bias or neither")
+        self.hidden, self.gate, self.activation = hidden, gate, activation
+
+    @classmethod
+    def from_float(cls, hidden_linear, gate_linear, activation="silu", **quant_args):
+        return cls(QuantizedLinear.from_float(hidden_linear, **quant_args),
+                   QuantizedLinear.from_float(gate_linear, **quant_args), activation)
+
+    def forward(self, x):
+        h, g = self.hidden, self.gate
+        return _C.fused_glu_with_groupwise_quantized_weight(
+            x, h.weight, h.weight_scale, w_zero=h.weight_zero, b=h.bias, v=g.weight,
+            v_scale=g.weight_scale, v_zero=g.weight_zero, c=g.bias, activation=self.activation,
+            num_bits=h.num_bits, symmetric=h.symmetric, group_dim=1, group_size=h.group_size)
+
+
+class GroupedQuantizedLinear(torch.nn.Module):
+    """Several ``QuantizedLinear`` modules applied to the same input in one call (the q, k and v
+    projections of an attention block) through
+    ``_C.grouped_linear_with_groupwise_quantized_weight``; returns the tuple of outputs."""
+
+    def __init__(self, linears):
+        super().__init__()
+        linears = list(linears)
+        for a in ("in_features", "num_bits", "symmetric", "group_size"):
+            if any(getattr(m, a) != getattr(linears[0], a) for m in linears):
+                raise ValueError(f"the linears differ in {a}")
+        self.linears = torch.nn.ModuleList(linears)
+
+    def forward(self, x):
+        ls = list(self.linears)
+        biases = [m.bias for m in ls]
+        if any(b is None for b in biases):
+            if not all(b is None for b in biases):
+                raise ValueError("either every linear has a bias or none")
+            biases = None
+        return tuple(_C.grouped_linear_with_groupwise_quantized_weight(
+            [x] * len(ls), [m.weight for m in ls], [m.weight_scale for m in ls],
+            w_zeros=None if ls[0].symmetric else [m.weight_zero for m in ls], bs=biases,
+            num_bits=ls[0].num_bits, symmetric=ls[0].symmetric, group_dim=1,
+            group_size=ls[0].group_size))

@@ -162,3 +162,25 @@ def test_glu_functional_matches_reference_style_composition():
     assert H.rel_l2(got, want) < 2e-3
     with pytest.raises(flow.CheckFailedError):
         flow._C.fused_glu_with_groupwise_quantized_weight(tt(x), tt(w), tt(ws), c=tt(x[0]))
+
+
+def test_module_wrappers():
+    """nn.QuantizedGLU and nn.GroupedQuantizedLinear give what their QuantizedLinear parts give
+    one by one (the linears agree up to summation order, the gating is then applied to them)."""
+    import torch
+    import oneflow_amd as flow
+    torch.manual_seed(3)
+    k, n = 512, 384
+    lin = [torch.nn.Linear(k, nn_, bias=True).half().cuda() for nn_ in (n, n, 128)]
+    x = torch.randn(3, k, dtype=torch.float16, device="cuda")
+    q = [flow.nn.QuantizedLinear.from_float(l, num_bits=4, symmetric=False, group_size=128,
+                                            quant_type=torch.uint8) for l in lin]
+    outs = flow.nn.GroupedQuantizedLinear(q)(x)
+    for o, m in zip(outs, q):
+        assert H.rel_l2(H.to_numpy(o), H.to_numpy(m(x))) < 1e-3
+    glu = flow.nn.QuantizedGLU(q[0], q[1], activation="silu")
+    y = glu(x)
+    ref = O.glu_gate(H.to_numpy(q[0](x)), H.to_numpy(q[1](x)), "silu")
+    assert H.rel_l2(H.to_numpy(y), ref) < 2e-3
+    with pytest.raises(ValueError):
+        flow.nn.QuantizedGLU(q[0], q[2])
