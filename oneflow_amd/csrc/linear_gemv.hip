@@ -377,20 +377,24 @@ int launch_rows_mt_part(hipStream_t st, const LinearArgs& a, int64_t m0, int m) 
   int rpb = (int)((a.n + grid - 1) / grid);
   if (rpb < 16) rpb = 16;
   grid = (a.n + rpb - 1) / rpb;
-  const int mt = m <= 32 ? 2 : 4;
-  const int nw = mt == 2 ? 16 : 8;
+  const int mt = (m + 15) / 16;  // 2, 3 or 4 tiles of x
+  // 16 waves while the registers allow four waves per SIMD, 12 beyond
+  const int nw = mt == 2 ? 16 : 12;
   const size_t lds =
       gemv_rows_mt_lds_bytes(nw, mt, (int)a.k, (int)a.group_size, rpb, !a.symmetric);
   if (lds > 160u * 1024u) return OFQ_ERR_UNSUPPORTED;
   const size_t esz = 2;
   const void* x = static_cast<const char*>(a.x) + (size_t)m0 * a.k * esz;
   void* out = static_cast<char*>(a.out) + (size_t)m0 * a.n * esz;
-  if (a.t_dtype == OFQ_BF16) {
-    return mt == 2 ? launch_rows_mt_t<bf16, 16, 2>(st, a, x, out, m, (int)grid, rpb, lds)
-                   : launch_rows_mt_t<bf16, 8, 4>(st, a, x, out, m, (int)grid, rpb, lds);
+#define OFQ_MT(TT_)                                                                        \
+  switch (mt) {                                                                            \
+    case 2: return launch_rows_mt_t<TT_, 16, 2>(st, a, x, out, m, (int)grid, rpb, lds);    \
+    case 3: return launch_rows_mt_t<TT_, 12, 3>(st, a, x, out, m, (int)grid, rpb, lds);    \
+    default: return launch_rows_mt_t<TT_, 12, 4>(st, a, x, out, m, (int)grid, rpb, lds);   \
   }
-  return mt == 2 ? launch_rows_mt_t<f16, 16, 2>(st, a, x, out, m, (int)grid, rpb, lds)
-                 : launch_rows_mt_t<f16, 8, 4>(st, a, x, out, m, (int)grid, rpb, lds);
+  if (a.t_dtype == OFQ_BF16) { OFQ_MT(bf16) }
+  OFQ_MT(f16)
+#undef OFQ_MT
 }
 
 // ---- fp32 activations -------------------------------------------------------------------------
