@@ -101,3 +101,39 @@ def test_module_wrappers_keep_reference_signatures():
     sig = inspect.signature(flow._C.groupwise_dequantize)
     kw = [n for n, p in sig.parameters.items() if p.kind == p.KEYWORD_ONLY]
     assert kw == ["zero", "num_bits", "symmetric", "group_dim", "group_size"]
+
+
+def test_glu_grouped_and_skip_layer_norm_checks():
+    """The argument rules of FusedGluFunctor (nn_functor.cpp:3724-3800), of the grouped tuples
+    (GroupedMatmulBiasFunctor: equal lengths) and of skip_layer_norm's inputs."""
+    x = torch.zeros((2, 64), dtype=torch.float16)
+    s = torch.ones((8, 1), dtype=torch.float16)
+    glu = flow._C.fused_glu_with_groupwise_quantized_weight
+    with pytest.raises(CheckFailedError, match="unsupported activation"):
+        glu(x, _w(), s, activation="tanh")
+    with pytest.raises(CheckFailedError, match="expected existance of b while providing c"):
+        glu(x, _w(), s, c=torch.zeros(8, dtype=torch.float16))
+    with pytest.raises(CheckFailedError, match="expected existance of c, when provide tensors w, v and b"):
+        glu(x, _w(), s, b=torch.zeros(8, dtype=torch.float16), v=_w(), v_scale=s)
+    with pytest.raises(CheckFailedError, match="v should have the shape and dtype of w"):
+        glu(x, _w(), s, v=_w(n=4), v_scale=torch.ones((4, 1), dtype=torch.float16))
+    with pytest.raises(CheckFailedError, match="not divisible by 2"):
+        glu(x, _w(n=7), torch.ones((7, 1), dtype=torch.float16))
+    with pytest.raises(CheckFailedError, match="tensors must live on the GPU"):
+        glu(x, _w(), s, v=_w(), v_scale=s, activation="silu")
+    grp = flow._C.grouped_linear_with_groupwise_quantized_weight
+    with pytest.raises(CheckFailedError, match="should have the same length"):
+        grp([x, x], [_w()], [s])
+    with pytest.raises(CheckFailedError, match="bs should have the length of xs"):
+        grp([x], [_w()], [s], bs=[None, None])
+    with pytest.raises(CheckFailedError, match="The size of second dimension of tensor w"):
+        grp([x], [_w(k=32)], [s])
+    with pytest.raises(CheckFailedError, match="tensors must live on the GPU"):
+        grp([x, x], [_w(), _w(n=4)], [s, torch.ones((4, 1), dtype=torch.float16)])
+    sln = flow._C.fused_skip_layer_norm_min_max_observer
+    with pytest.raises(CheckFailedError, match="skip should have the shape and dtype of x"):
+        sln(x, skip=torch.zeros((2, 32), dtype=torch.float16))
+    with pytest.raises(CheckFailedError, match="bias should be 1-D"):
+        sln(x, bias=torch.zeros((1, 64), dtype=torch.float16))
+    with pytest.raises(CheckFailedError, match=r"quantization_bit should be in range \(1, 8\]."):
+        sln(x, quantization_bit=9)
