@@ -18,14 +18,19 @@
 
 namespace ofq {
 
-// The copy-fed GEMMs are bound by the L2 -> LDS traffic per MFMA, which falls with the tile area,
-// so a 256x352 tile (one per CU, 8 waves side by side along M) beats 256x128 whenever its tiles
-// fill whole rounds of the 256 CUs reasonably well; with a poor fill the idle tail costs more
-// than the traffic saves.
-bool wide_tiles_pay(int64_t m, int64_t n) {
-  const int64_t tiles = ((m + 255) / 256) * ((n + 351) / 352);
-  const int64_t rounds = (tiles + 255) / 256;
-  return tiles * 100 >= rounds * 256 * 80;
+// Width of the weight tile under a 256-row tile of x.  The blocks run in rounds of one per CU;
+// a round costs about in proportion to the tile width, so the candidate with the smallest
+// (rounds x width) wins, the wider one on a tie (less L2 -> LDS traffic per MFMA).  352 is open
+// to the copy-fed GEMMs only (2048x11008: 8 x 32 = 256 tiles, exactly one round); 192 turns the
+// 258 or 344 tiles of m = 768 / 1024 at n = 11008 (two rounds of 128-wide tiles, the second
+// nearly empty) into one round of 174 / 232: 160 -> 115 us in-tile.
+int pick_tile_width(int64_t m, int64_t n, bool allow_352) {
+  const int64_t m_tiles = (m + 255) / 256;
+  auto cost = [&](int64_t bn) { return ((m_tiles * ((n + bn - 1) / bn) + 255) / 256) * bn; };
+  int best = 128;
+  if (cost(192) <= cost(best)) best = 192;
+  if (allow_352 && cost(352) <= cost(best)) best = 352;
+  return best;
 }
 
 namespace {
@@ -42,12 +47,17 @@ int launch_plain(hipStream_t st, const LinearArgs& a, const void* wt) {
   typename EP::Params ep;
   ep.bias = static_cast<const S*>(a.bias);
   ep.out = static_cast<S*>(a.out);
-  if (wide_tiles_pay(a.m, a.n)) {
-    return launch_core2<MF, B2Copy<352, 512>, EP, 256, 352, 8, 1>(st, a.x, a.k * 2, bp, ep, a.m,
-                                                                  a.n, a.k / 64);
+  switch (pick_tile_width(a.m, a.n, true)) {
+    case 352:
+      return launch_core2<MF, B2Copy<352, 512>, EP, 256, 352, 8, 1>(st, a.x, a.k * 2, bp, ep, a.m,
+                                                                    a.n, a.k / 64);
+    case 192:
+      return launch_core2<MF, B2Copy<192, 512>, EP, 256, 192, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
+                                                                    a.n, a.k / 64);
+    default:
+      return launch_core2<MF, B2Copy<128, 512>, EP, 256, 128, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
+                                                                    a.n, a.k / 64);
   }
-  return launch_core2<MF, B2Copy<128, 512>, EP, 256, 128, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m, a.n,
-                                                                a.k / 64);
 }
 
 // Few blocks (m small against the tile height, or few weight tiles): K is cut into `splits`
@@ -147,6 +157,10 @@ int launch_wq_variant(hipStream_t st, const LinearArgs& a, float* partials, int 
   }
   // 256x128 tiles on 8 waves when there are enough rows of x to fill them, else 128x128 on 4
   if (a.m > 128) {
+    if (pick_tile_width(a.m, a.n, false) == 192) {
+      return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 192, 512>, EP, 256, 192, 4, 2>(
+          st, a.x, a.k * 2, bp, ep, a.m, a.n, a.k / 64);
+    }
     return launch_core2<MF, B2Dequant<T, BITS, SIGNED, ZMODE, 128, 512>, EP, 256, 128, 4, 2>(
         st, a.x, a.k * 2, bp, ep, a.m, a.n, a.k / 64);
   }
@@ -253,8 +267,13 @@ extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, cons
     ep.b_scale = b_scale;                                                                      \
     ep.bias = static_cast<const TT<T>::storage*>(bias);                                        \
     ep.out = static_cast<TT<T>::storage*>(out);                                                \
-    if (m > 128 && wide_tiles_pay(m, n)) {                                                     \
+    const int bn = m > 128 ? pick_tile_width(m, n, true) : 128;                                \
+    if (bn == 352) {                                                                           \
       return launch_core2<MfmaI8, B2Copy<352, 512>, EP, 256, 352, 8, 1>(st, a, k, bp, ep, m,   \
+                                                                        n, k / 128);           \
+    }                                                                                          \
+    if (bn == 192) {                                                                           \
+      return launch_core2<MfmaI8, B2Copy<192, 512>, EP, 256, 192, 4, 2>(st, a, k, bp, ep, m,   \
                                                                         n, k / 128);           \
     }                                                                                          \
     if (m > 128) {                                                                             \

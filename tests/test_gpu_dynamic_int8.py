@@ -148,13 +148,14 @@ def test_matmul_quant_small_exact(m, n, k, t):
 
 
 @pytest.mark.parametrize("t", ["f32", "bf16"])
-def test_matmul_quant_wide_tiles_full_output(t):
-    """A shape that is dispatched to the 256x352 tiles with ragged last tiles in both m and n;
-    every output is checked.  The int32 accumulators come from a float64 matmul, which is exact
-    here (|sum| <= 128*128*256 < 2^53)."""
+@pytest.mark.parametrize("m,n", [(2053, 8196), (700, 11012)])
+def test_matmul_quant_wide_tiles_full_output(t, m, n):
+    """Shapes that are dispatched to the 256x352 and to the 256x192 tiles, with ragged last tiles
+    in both m and n; every output is checked.  The int32 accumulators come from a float64 matmul,
+    which is exact here (|sum| <= 128*128*256 < 2^53)."""
     import oneflow_amd as flow
     import torch
-    m, n, k = 2053, 8196, 256
+    k = 256
     rng = np.random.Generator(np.random.PCG64(99))
     a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
     b = rng.integers(-128, 128, size=(n, k)).astype(np.int8)

@@ -384,3 +384,34 @@ def test_fp32_activations(m, n, k, g, num_bits):
         got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
         assert H.rel_l2(got, ref) < 2e-6, (symmetric, qdt)
         assert np.allclose(got, ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("t", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n", [(700, 11012), (1030, 8300)])
+def test_prefill_192_wide_tiles(t, m, n):
+    """m and n for which three or four 256-row tiles of x times the 128-wide weight tiles spill
+    into a second, nearly empty round of blocks: the 192-wide tiles, in-tile (m < 1024) and
+    copy-fed behind the dequantised weight (m >= 1024, with the workspace); sampled rows."""
+    import torch
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    k, g = 256, 64
+    tcode = _lib.F16 if t == "f16" else _lib.BF16
+    rng = np.random.Generator(np.random.PCG64(m + n))
+    x = H.as_T((rng.standard_normal((m, k)) / 4).astype(np.float32), t)
+    w = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+    scale = H.as_T(rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float32), t)
+    zero = H.as_T(rng.uniform(-1.4, -1.1, size=(n, k // g)).astype(np.float32), t)
+    b = H.as_T(rng.standard_normal(n).astype(np.float32) / 10, t)
+    xt, wt, st, zt, bt = map(H.to_torch, (x, w, scale, zero, b))
+    need = L.ofq_fused_linear_gq_workspace_bytes(_lib.U8, tcode, 8, 0, 1, g, m, n, k)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    rows = np.unique(np.concatenate([np.arange(0, 3), np.arange(254, 258), np.arange(m - 3, m)]))
+    ref = O.fused_linear(x[rows], w, scale, zero, b, 8, False, 1, g)
+    for wptr, wbytes in ((ws.data_ptr(), need), (None, 0)):
+        out = torch.empty((m, n), dtype=xt.dtype, device="cuda")
+        rc = L.ofq_fused_linear_gq(torch.cuda.current_stream().cuda_stream, xt.data_ptr(),
+                                   wt.data_ptr(), st.data_ptr(), zt.data_ptr(), bt.data_ptr(),
+                                   out.data_ptr(), _lib.U8, tcode, 8, 0, 1, g, m, n, k, wptr, wbytes)
+        assert rc == 0
+        H.assert_linear_parity(H.to_numpy(out)[rows], ref, t, f"m={m} n={n} {t} ws={wbytes}")
