@@ -128,3 +128,27 @@ def test_layer_norm_and_matmul_quant_argument_errors(lib):
     assert mq(None, None, P, P, P, None, P, F16, 16, 16, 128) == NULLP
     assert mq(None, U, P, P, P, None, P, F16, 16, 16, 128) == MISALIGNED
     assert mq(None, P, P, P, P, None, P, F16, 0, 16, 128) == OK
+
+
+def test_grouped_and_glu_argument_errors(lib):
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
+    one = (vp * 1)(P.value)
+    n1 = (i64 * 1)(16)
+    g = lib.ofq_grouped_linear_gq
+    assert g(None, 0, None, None, None, None, None, None, None, None, None, I8, F16, 4, 1, 1, 128) == OK
+    assert g(None, 65, one, one, one, None, None, one, n1, n1, n1, I8, F16, 4, 1, 1, 128) == BAD_SHAPE
+    assert g(None, 1, None, one, one, None, None, one, n1, n1, n1, I8, F16, 4, 1, 1, 128) == NULLP
+    assert g(None, 1, one, one, one, None, None, one, n1, n1, n1, F16, F16, 4, 1, 1, 128) == BAD_DTYPE
+    assert g(None, 1, one, one, one, None, None, one, n1, n1, n1, U8, F16, 4, 0, 1, 128) == NULLP  # no zeros
+    # one problem goes through the single op's checks: num_bits 3 is rejected there
+    k128 = (i64 * 1)(128)
+    assert g(None, 1, one, one, one, None, None, one, n1, n1, k128, I8, F16, 3, 1, 1, 128) == BAD_ATTR
+    f = lib.ofq_fused_glu_gq
+    N = None
+    assert f(None, P, P, P, N, N, P, P, N, N, P, P, P, 6, I8, F16, 4, 1, 1, 128, 1, 16, 128) == BAD_ATTR
+    assert f(None, P, P, P, N, N, P, P, N, N, P, P, P, 5, F16, F16, 4, 1, 1, 128, 1, 16, 128) == BAD_DTYPE
+    assert f(None, P, P, P, N, N, P, P, N, N, P, P, P, 5, I8, F16, 4, 1, 1, 128, 0, 16, 128) == OK
+    assert f(None, P, P, P, N, N, P, P, N, N, N, P, P, 5, I8, F16, 4, 1, 1, 128, 1, 16, 128) == NULLP  # y
+    assert f(None, P, P, P, N, N, P, P, N, P, P, P, P, 5, I8, F16, 4, 1, 1, 128, 1, 16, 128) == NULLP  # c without b
+    assert f(None, P, P, P, N, P, P, P, N, N, P, P, P, 5, I8, F16, 4, 1, 1, 128, 1, 16, 128) == NULLP  # b without c
+    assert f(None, P, P, P, N, N, P, P, N, N, P, P, N, 5, I8, F16, 4, 1, 1, 128, 1, 16, 128) == NULLP  # matmul_vx
