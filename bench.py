@@ -66,6 +66,10 @@ def main():
                     help="for a `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` run: a few direct launches of "
                          "the hot path plus an elementwise kernel of known traffic (1 GiB read, "
                          "1 GiB written) to scale the counters by; prints no result line")
+    ap.add_argument("--pmc-gemm", action="store_true",
+                    help="for a `rocprofv3 --pmc` run on the MFMA kernels: three launches each of the "
+                         "prefill linear (with and without its workspace) and of matmul_quant at "
+                         "m=2048; prints no result line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU by design (the path has no collectives); "
@@ -84,6 +88,9 @@ def main():
     torch.cuda.set_device(dev)
     torch.manual_seed(1234)
     M = args.m
+    if args.pmc_gemm:
+        pmc_gemm(L, _lib, torch, dev)
+        return
 
     # ---- synthetic Llama-7B-shaped int4 weights, distinct per layer ----------------------------
     layers = []
@@ -265,6 +272,33 @@ def cpu_baseline(M):
     return {"value": round(total_bytes / t_total / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"{reps} Llama-7B decoder layers ({7 * reps} GEMVs, {total_bytes} algorithmic bytes, m={M}) "
                       f"through oracle/ofq_oracle.c in {t_total:.2f} s; host has {os.cpu_count()} cpus"}
+
+
+def pmc_gemm(L, _lib, torch, dev):
+    """BASELINE configurations 4 and 5 (the GEMM halves), a few direct launches each."""
+    cs = torch.cuda.current_stream().cuda_stream
+    m, n, k, g = 2048, 11008, 4096, 64
+    x = torch.randn((m, k), device=dev).to(torch.bfloat16)
+    w = torch.randint(0, 256, (n, k), dtype=torch.uint8, device=dev)
+    sc = torch.empty((n, k // g), device=dev).uniform_(1e-3, 1e-2).to(torch.bfloat16)
+    ze = torch.empty((n, k // g), device=dev).uniform_(120, 136).to(torch.bfloat16)
+    o = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    ws_bytes = L.ofq_fused_linear_gq_workspace_bytes(_lib.U8, _lib.BF16, 8, 0, 1, g, m, n, k)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    a8 = torch.randint(-128, 128, (m, k), dtype=torch.int8, device=dev)
+    w8 = torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev)
+    a_s = torch.full((1,), 0.01, dtype=torch.float32, device=dev)
+    b_s = torch.empty(n, dtype=torch.float32, device=dev).uniform_(1e-3, 1e-2)
+    o16 = torch.empty((m, n), dtype=torch.float16, device=dev)
+    for _ in range(3):
+        for wptr, wb in ((ws.data_ptr(), ws_bytes), (None, 0)):
+            st = L.ofq_fused_linear_gq(cs, x.data_ptr(), w.data_ptr(), sc.data_ptr(), ze.data_ptr(), None,
+                                       o.data_ptr(), _lib.U8, _lib.BF16, 8, 0, 1, g, m, n, k, wptr, wb)
+            assert st == 0, st
+        st = L.ofq_matmul_quant(cs, a8.data_ptr(), w8.data_ptr(), a_s.data_ptr(), b_s.data_ptr(), None,
+                                o16.data_ptr(), _lib.F16, m, n, k)
+        assert st == 0, st
+    torch.cuda.synchronize()
 
 
 def secondary(L, _lib, torch, dev, args):
