@@ -415,3 +415,24 @@ def test_prefill_192_wide_tiles(t, m, n):
                                    out.data_ptr(), _lib.U8, tcode, 8, 0, 1, g, m, n, k, wptr, wbytes)
         assert rc == 0
         H.assert_linear_parity(H.to_numpy(out)[rows], ref, t, f"m={m} n={n} {t} ws={wbytes}")
+
+
+@pytest.mark.parametrize("t", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("m", [1, 9, 20, 70])
+@pytest.mark.parametrize("num_bits,k,g", [(4, 384, 96), (4, 768, 192), (8, 192, 48), (8, 576, 96)])
+def test_group_sizes_that_are_not_powers_of_two(t, m, num_bits, k, g):
+    """Group sizes that are multiples of a lane's load but not powers of two (the kernels' group
+    index is then a division, not a shift), through every m regime."""
+    n = 200
+    rng = np.random.Generator(np.random.PCG64(m + k + g))
+    x = H.as_T((rng.standard_normal((m, k)) / 2).astype(np.float32), t)
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), t)
+    for symmetric, qdt in VARIANTS:
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, g, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, g)
+        if t == "f32":
+            assert np.allclose(got, ref, rtol=1e-4, atol=1e-4)
+        else:
+            H.assert_linear_parity(got, ref, t, f"{t} b{num_bits} m={m} k={k} g={g} {symmetric} {qdt}")
