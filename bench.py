@@ -510,6 +510,32 @@ def secondary(L, _lib, torch, dev, args):
                              "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
         del ws
 
+    # ---- the same decode kernel on a large weight: an int4 output layer, 128256 x 4096 ---------
+    # (263 MB per launch: the fixed cost per launch that bounds the 8-23 MB layer shapes is small
+    # here, so this shows what the kernel itself streams at)
+    n, k, g = 128256, 4096, 128
+    reps = 3
+    ws = [torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev) for _ in range(reps)]
+    sc = torch.empty((n, k // g), dtype=torch.float16, device=dev).uniform_(1e-3, 1e-2)
+    xx = torch.randn((1, k), device=dev).to(torch.float16)
+    oo = torch.empty((1, n), dtype=torch.float16, device=dev)
+    it[0] = 0
+
+    def head():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_fused_linear_gq(cs(), xx.data_ptr(), ws[i].data_ptr(), sc.data_ptr(), None, None,
+                                  oo.data_ptr(), _lib.I8, _lib.F16, 4, 1, 1, g, 1, n, k, None, 0),
+            "lm head")
+    us = timeit(head, iters=12)
+    nbytes = gemv_bytes(1, n, k) - n * 2  # no bias
+    gb = nbytes / (us * 1e-6) / 1e9
+    out["decode_w4a16_output_layer_128256x4096_m1"] = {
+        "us": round(us, 2), "gbps": round(gb, 1),
+        "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+    del ws
+
     # ---- weight quantise + pack: fp16 [11008,4096] -> symmetric int4, g=128 -------------------
     n, k, g = 11008, 4096, 128
     reps = 6  # 6 x 90 MB of distinct sources: beyond the caches

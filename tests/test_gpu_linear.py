@@ -436,3 +436,17 @@ def test_group_sizes_that_are_not_powers_of_two(t, m, num_bits, k, g):
             assert np.allclose(got, ref, rtol=1e-4, atol=1e-4)
         else:
             H.assert_linear_parity(got, ref, t, f"{t} b{num_bits} m={m} k={k} g={g} {symmetric} {qdt}")
+
+
+@pytest.mark.parametrize("t", ["f16", "bf16"])
+def test_decode_vocabulary_sized_n(t):
+    """An output layer: n = 128256 rows (more 64-row blocks than the chip holds at once)."""
+    m, n, k, g = 2, 128256, 512, 128
+    rng = np.random.Generator(np.random.PCG64(5))
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), t)
+    codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    w = H.pack_int4(codes)
+    scale = H.as_T(rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float32), t)
+    ref = O.fused_linear(x, w, scale, None, None, 4, True, 1, g)
+    got = _run(x, w, scale, None, None, 4, True, 1, g)
+    H.assert_linear_parity(got, ref, t, f"{t} lm head")
