@@ -439,9 +439,10 @@ def test_group_sizes_that_are_not_powers_of_two(t, m, num_bits, k, g):
 
 
 @pytest.mark.parametrize("t", ["f16", "bf16"])
-def test_decode_vocabulary_sized_n(t):
+@pytest.mark.parametrize("m", [2, 16])
+def test_decode_vocabulary_sized_n(t, m):
     """An output layer: n = 128256 rows (more 64-row blocks than the chip holds at once)."""
-    m, n, k, g = 2, 128256, 512, 128
+    n, k, g = 128256, 512, 128
     rng = np.random.Generator(np.random.PCG64(5))
     x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), t)
     codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
