@@ -264,7 +264,7 @@ def cpu_baseline(M):
     reps = 4  # about 10 s of scalar CPU work
     mt_bytes = 0
     t_mt = 0.0
-    mt_reps = 2
+    mt_reps = 8
     for name, n, k, cnt in LLAMA7B_LAYER:
         w = rng.integers(-128, 128, size=(n, k // 2), dtype=np.int8)
         scale = rng.uniform(1e-3, 1e-2, size=(n, k // 128)).astype(np.float16)
