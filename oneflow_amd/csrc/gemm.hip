@@ -235,6 +235,26 @@ int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t 
   return launch_wq_t<bf16, MfmaBF16>(st, a, nullptr, 1);
 }
 
+// Groups along N: nothing to gain from converting inside the GEMM (a k-tile of a weight row would
+// need 64 scales); above the streaming kernel's range the weight is dequantised once into the
+// workspace -- the reference functor's own decomposition for m > 8,
+// oneflow/core/functional/impl/quantization.cpp:341-350 -- and the copy-fed GEMM runs on it.
+size_t gemm_gn_workspace_bytes(const LinearArgs& a) {
+  if (a.group_dim != 0 || (a.t_dtype != OFQ_F16 && a.t_dtype != OFQ_BF16)) return 0;
+  if (a.m <= 64 || a.k % 64 != 0 || a.n % a.group_size != 0) return 0;
+  return (size_t)a.n * (size_t)a.k * 2;
+}
+
+int launch_gemm_gn(hipStream_t st, const LinearArgs& a, void* workspace) {
+  const int rc = ofq_groupwise_dequantize(st, a.w, a.scale, a.zero, workspace,
+                                          a.w_signed ? OFQ_I8 : OFQ_U8, a.t_dtype, a.bits,
+                                          a.symmetric ? 1 : 0, a.n / a.group_size, a.group_size,
+                                          a.k);
+  if (rc != OFQ_OK) return rc;
+  if (a.t_dtype == OFQ_F16) return launch_plain<f16, MfmaF16>(st, a, workspace);
+  return launch_plain<bf16, MfmaBF16>(st, a, workspace);
+}
+
 }  // namespace ofq
 
 using namespace ofq;

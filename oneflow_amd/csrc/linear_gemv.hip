@@ -789,6 +789,7 @@ extern "C" size_t ofq_fused_linear_gq_workspace_bytes(int w_dtype, int t_dtype, 
   a.n = n;
   a.k = k;
   if (gemv_wq_supported(a) || gemv_mt_supported(a)) return 0;
+  if (group_dim == 0) return gemm_gn_workspace_bytes(a);
   return gemm_wq_workspace_bytes(a);  // 0 for every path but the two-pass GEMM at large m
 }
 
@@ -847,5 +848,15 @@ extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
   }
   if (gemm_wq_supported(a)) return launch_gemm_wq(st, a, workspace, workspace_bytes);
+  if (a.group_dim == 0) {
+    const size_t need = gemm_gn_workspace_bytes(a);
+    if (need != 0 && workspace != nullptr && workspace_bytes >= need && ofq_aligned16(workspace)) {
+      return launch_gemm_gn(st, a, workspace);
+    }
+    if (gemv_gn_supported(a)) {
+      const int rc = launch_gemv_gn(st, a);
+      if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+    }
+  }
   return launch_linear_generic(st, a);
 }

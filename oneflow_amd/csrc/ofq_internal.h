@@ -40,6 +40,14 @@ int launch_gemv_wq(hipStream_t st, const LinearArgs& a);
 bool gemv_mt_supported(const LinearArgs& a);
 int launch_gemv_mt(hipStream_t st, const LinearArgs& a);
 
+// Groups along N (group_dim = 0), fp16 / bf16: the streaming kernel with one scale per k (any m,
+// 64 rows of x per pass over the weights), and for m > 64 with a workspace of
+// gemm_gn_workspace_bytes() the weight dequantised once plus a copy-fed GEMM.
+bool gemv_gn_supported(const LinearArgs& a);
+int launch_gemv_gn(hipStream_t st, const LinearArgs& a);
+size_t gemm_gn_workspace_bytes(const LinearArgs& a);
+int launch_gemm_gn(hipStream_t st, const LinearArgs& a, void* workspace);
+
 // Up to 8 decode linears that share m, k, dtype and quantisation attributes (x, w, scale, zero,
 // bias, out and n per problem) as ONE launch of the natural-order decode kernel.
 // OFQ_ERR_UNSUPPORTED when the shapes do not fit it (caller launches the problems one by one).

@@ -81,6 +81,9 @@ def test_fused_linear_argument_errors(lib):
     assert call(w=U) == MISALIGNED
     assert call(m=0) == OK
     assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 1, 128, 1, 4096, 4096) == 0
+    # groups along N: no workspace up to 64 rows of x, the dequantised weight beyond
+    assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 0, 128, 64, 4096, 4096) == 0
+    assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 0, 128, 65, 4096, 4096) == 4096 * 4096 * 2
 
 
 def test_observer_and_quantization_argument_errors(lib):
