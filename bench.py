@@ -532,6 +532,34 @@ def secondary(L, _lib, torch, dev, args):
                              "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
         del ws
 
+    # ---- groups along N (group_dim = 0, scale [n/g, k]): fp16 W4 symmetric g=128, m = 1 and 16 ---
+    n, k, g = 11008, 4096, 128
+    reps = 8
+    ws = [torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev) for _ in range(reps)]
+    sc = torch.empty((n // g, k), device=dev).uniform_(1e-3, 1e-2).to(torch.float16)
+    for m in (1, 16):
+        xx = torch.randn((m, k), device=dev).to(torch.float16)
+        oo = torch.empty((m, n), dtype=torch.float16, device=dev)
+
+        def dec_gn():
+            for i in range(reps):
+                chk(L.ofq_fused_linear_gq(cs(), xx.data_ptr(), ws[i].data_ptr(), sc.data_ptr(), None,
+                                          None, oo.data_ptr(), _lib.I8, _lib.F16, 4, 1, 0, g, m, n, k,
+                                          None, 0), "decode, groups along N")
+        dec_gn()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            dec_gn()
+        us = timeit(gr.replay, iters=10) / reps
+        nbytes = n * k // 2 + (n // g) * k * 2 + m * k * 2 + m * n * 2
+        gb = nbytes / (us * 1e-6) / 1e9
+        out[f"decode_f16_w4_groups_along_n_g128_11008x4096_m{m}"] = {
+            "us": round(us, 2), "gbps": round(gb, 1),
+            "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+    del ws
+
     # ---- the same decode kernel on a large weight: an int4 output layer, 128256 x 4096 ---------
     # (263 MB per launch: the fixed cost per launch that bounds the 8-23 MB layer shapes is small
     # here, so this shows what the kernel itself streams at)
