@@ -460,7 +460,32 @@ def secondary(L, _lib, torch, dev, args):
         "us": round(us, 2), "tops": round(tops, 1),
         "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": MFMA_PEAK_TFLOPS["i8"],
                      "unit": "TOP/s", "frac": round(tops / MFMA_PEAK_TFLOPS["i8"], 4)}}
-    del xs, ys, a8, wq, o
+    # the same op at decode (m = 1 and 16): the streaming int8 kernel; 6 weight sets cycled so that
+    # no launch finds its weight in the caches
+    reps_w = 6
+    wqs = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(reps_w)]
+    for md in (1, 16):
+        ad = torch.randint(-128, 128, (md, k), dtype=torch.int8, device=dev)
+        od = torch.empty((md, n), dtype=torch.float16, device=dev)
+
+        def mq_dec():
+            for i in range(reps_w):
+                chk(L.ofq_matmul_quant(cs(), ad.data_ptr(), wqs[i].data_ptr(), s.data_ptr(),
+                                       wsc.data_ptr(), None, od.data_ptr(), _lib.F16, md, n, k),
+                    "matmul_quant decode")
+        mq_dec()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            mq_dec()
+        us = timeit(gr.replay, iters=10) / reps_w
+        nbytes = n * k + n * 4 + md * k + md * n * 2
+        gb = nbytes / (us * 1e-6) / 1e9
+        out[f"matmul_quant_i8_decode_11008x4096_m{md}"] = {
+            "us": round(us, 2), "gbps": round(gb, 1),
+            "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
+    del xs, ys, a8, wq, o, wqs
 
     # ---- config 1: observer / quantization / fake_quantization of a 4096x4096 fp32 weight --------
     reps = 6

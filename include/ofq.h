@@ -260,6 +260,8 @@ int ofq_fused_glu_gq(void* stream, const void* x, const void* w, const void* w_s
  * a[m,k] int8, b[n,k] int8 (weight layout), exact int32 accumulation,
  * out[m,n] = T( float(acc) * (a_scale[0] * b_scale[n]) + float(bias[n]) ), out_dtype OFQ_F16 |
  * OFQ_BF16 | OFQ_F32; a_scale: one fp32 on the device; b_scale: fp32[n]; bias: out_dtype[n] or NULL.
+ * k has to be a multiple of 64.  m <= 64 streams the weights once (decode); larger m runs the
+ * tiled int8 MFMA GEMM (k a multiple of 128; else 64 rows of a per pass of the streaming kernel).
  */
 int ofq_matmul_quant(void* stream, const void* a, const void* b, const float* a_scale,
                      const float* b_scale, const void* bias, void* out, int out_dtype, int64_t m,

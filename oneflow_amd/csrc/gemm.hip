@@ -259,6 +259,9 @@ int launch_gemm_gn(hipStream_t st, const LinearArgs& a, void* workspace) {
 
 using namespace ofq;
 
+// rows of a up to which matmul_quant streams the weights instead of tiling them
+static constexpr int64_t kMatmulQuantRowsMaxM = 64;
+
 extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, const float* a_scale,
                                 const float* b_scale, const void* bias, void* out, int out_dtype,
                                 int64_t m, int64_t n, int64_t k) {
@@ -268,13 +271,18 @@ extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, cons
   if (m == 0 || n == 0) return OFQ_OK;
   const int64_t i32max = 0x7FFFFFFF;
   OFQ_RETURN_IF(m * k > i32max || n * k > i32max || m * n > i32max, OFQ_ERR_UNSUPPORTED);
-  // rows are consumed in 128-byte tiles of K
-  OFQ_RETURN_IF(k % 128 != 0, OFQ_ERR_UNSUPPORTED);
+  // rows are consumed in 64-byte chunks of K (streaming kernel) or 128-byte tiles (GEMM)
+  OFQ_RETURN_IF(k % 64 != 0, OFQ_ERR_UNSUPPORTED);
   OFQ_RETURN_IF(a == nullptr || b == nullptr || a_scale == nullptr || b_scale == nullptr
                     || out == nullptr,
                 OFQ_ERR_NULL_POINTER);
   OFQ_RETURN_IF(!ofq_aligned16(a) || !ofq_aligned16(b) || !ofq_aligned16(out), OFQ_ERR_MISALIGNED);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // few rows of a, or a K the GEMM's tiles do not divide: the weights stream once per 64 rows
+  if ((m <= kMatmulQuantRowsMaxM || k % 128 != 0) && matmul_quant_rows_supported(m, n, k)) {
+    return launch_matmul_quant_rows(st, a, b, a_scale, b_scale, bias, out, out_dtype, m, n, k);
+  }
+  OFQ_RETURN_IF(k % 128 != 0, OFQ_ERR_UNSUPPORTED);
   BCopyParams bp;
   bp.b = static_cast<const uint8_t*>(b);
   bp.ldb = k;

@@ -59,6 +59,13 @@ int launch_gemv_grouped(hipStream_t st, const LinearArgs* problems, int count);
 // not fit (caller runs the linears and the gating separately).
 int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act);
 
+// matmul_quant with few rows of a: int8 MFMA with the weights streamed once, 64 rows of a per
+// pass (any m; k a multiple of 64).
+bool matmul_quant_rows_supported(int64_t m, int64_t n, int64_t k);
+int launch_matmul_quant_rows(hipStream_t st, const void* a, const void* b, const float* a_scale,
+                             const float* b_scale, const void* bias, void* out, int out_dtype,
+                             int64_t m, int64_t n, int64_t k);
+
 // Any shape / grouping; one wave per output element.
 int launch_linear_generic(hipStream_t st, const LinearArgs& a);
 

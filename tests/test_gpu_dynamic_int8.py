@@ -179,3 +179,42 @@ def test_matmul_quant_wide_tiles_full_output(t, m, n):
                          {"f32": np.float32, "bf16": np.uint16}[t])
     view = np.uint32 if t == "f32" else np.uint16
     assert np.array_equal(got[np.ix_(rows, cols)].view(view), ref.view(view))
+
+
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (5, 1000, 192), (16, 37, 64), (17, 688, 1024),
+                                   (33, 2049, 448), (64, 300, 11008), (200, 130, 192)])
+def test_matmul_quant_few_rows_streaming(m, n, k, t):
+    """m <= 64 (and any m when k is a multiple of 64 but not of 128) runs the streaming int8 MFMA
+    kernel: 1, 2 and 4 tiles of a, ragged n, k from one chunk to many, several passes for
+    m = 200.  Bit-exact: int32 sums are order-free and the epilogue is the GEMM path's."""
+    import oneflow_amd as flow
+    import torch
+    rng = np.random.Generator(np.random.PCG64(m * 1000 + n + k))
+    a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, size=(n, k)).astype(np.int8)
+    a_scale = np.array([0.0317], np.float32)
+    b_scale = rng.uniform(1e-3, 1e-2, size=n).astype(np.float32)
+    bias = H.as_T(rng.standard_normal(n).astype(np.float32), t) if (m + n) % 2 else None
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[t]
+    got = H.to_numpy(flow._C.matmul_quant(H.to_torch(a), H.to_torch(b), H.to_torch(a_scale),
+                                          H.to_torch(b_scale), H.to_torch(bias), tdt))
+    acc = (a.astype(np.float64) @ b.astype(np.float64).T)
+    assert np.abs(acc).max() < 2**31
+    sc = (a_scale[0] * b_scale).astype(np.float32)
+    val = (acc.astype(np.float32) * sc[None, :]).astype(np.float32)
+    if bias is not None:
+        val = val + O.to_f32(bias)[None, :]
+    if t == "f32":
+        assert np.array_equal(got, val.astype(np.float32))
+    elif t == "bf16":
+        assert np.array_equal(got, O.f32_to_bf16_bits(val))
+    else:
+        assert np.array_equal(got, val.astype(np.float16))
+    # and the oracle on a corner
+    rows, cols = np.arange(max(0, m - 3), m), np.arange(max(0, n - 20), n)
+    ref = O.matmul_quant(a[rows], b[cols], a_scale, b_scale[cols],
+                         None if bias is None else bias[cols],
+                         {"f32": np.float32, "f16": np.float16, "bf16": np.uint16}[t])
+    view = np.uint32 if t == "f32" else np.uint16
+    assert np.array_equal(got[np.ix_(rows, cols)].view(view), ref.view(view))
