@@ -72,12 +72,14 @@ __device__ __forceinline__ void observer_channel(T vmax, T vmin, int bits, int s
 // scale and zero point itself and no second launch is needed.
 template<typename T, bool DIRECT>
 __global__ void __launch_bounds__(kObsBlock)
-observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, T* __restrict__ part,
-                 int bits, int scheme, int formula, T* __restrict__ scale,
+observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, int64_t total_slices,
+                 T* __restrict__ part, int bits, int scheme, int formula, T* __restrict__ scale,
                  T* __restrict__ zero_point) {
   __shared__ T smem[kObsBlock / kWave];
-  const int64_t c = blockIdx.x / splits;
-  const int64_t sp = blockIdx.x % splits;
+  // slice `blk` of channels * splits; the grid is capped, so a block may take several
+  for (int64_t blk = blockIdx.x; blk < total_slices; blk += gridDim.x) {
+  const int64_t c = blk / splits;
+  const int64_t sp = blk % splits;
   const int64_t begin = sp * kObsSliceElems;
   int64_t end = begin + kObsSliceElems;
   if (end > inner) end = inner;
@@ -121,12 +123,12 @@ observer_partial(const T* __restrict__ in, int64_t inner, int64_t splits, T* __r
   vmin = block_reduce(vmin, OpMin(), smem);
   if (threadIdx.x == 0) {
     if (DIRECT) {
-      observer_channel<T>(vmax, vmin, bits, scheme, formula, scale + blockIdx.x,
-                          zero_point + blockIdx.x);
+      observer_channel<T>(vmax, vmin, bits, scheme, formula, scale + blk, zero_point + blk);
     } else {
-      part[2 * blockIdx.x] = vmax;
-      part[2 * blockIdx.x + 1] = vmin;
+      part[2 * blk] = vmax;
+      part[2 * blk + 1] = vmin;
     }
+  }
   }
 }
 
@@ -143,6 +145,49 @@ observer_finalize(const T* __restrict__ part, int64_t channels, int64_t splits, 
     vmin = OpMin()(vmin, part[2 * (c * splits + s) + 1]);
   }
   observer_channel<T>(vmax, vmin, bits, scheme, formula, scale + c, zero_point + c);
+}
+
+// Channels of many slices (a per-layer observer is ONE channel of elem_cnt / 4096 slices): a block
+// per channel, the slices strided over its threads.  max / min do not depend on the order.
+template<typename T>
+__global__ void __launch_bounds__(kObsBlock)
+observer_finalize_wide(const T* __restrict__ part, int64_t splits, int bits, int scheme,
+                       int formula, T* __restrict__ scale, T* __restrict__ zero_point) {
+  __shared__ T smem[kObsBlock / kWave];
+  const int64_t c = blockIdx.x;
+  const T* p = part + 2 * c * splits;
+  T vmax = p[0];
+  T vmin = p[1];
+  for (int64_t s = threadIdx.x; s < splits; s += kObsBlock) {
+    vmax = OpMax()(vmax, p[2 * s]);
+    vmin = OpMin()(vmin, p[2 * s + 1]);
+  }
+  vmax = block_reduce(vmax, OpMax(), smem);
+  vmin = block_reduce(vmin, OpMin(), smem);
+  if (threadIdx.x == 0) {
+    observer_channel<T>(vmax, vmin, bits, scheme, formula, scale + c, zero_point + c);
+  }
+}
+
+// Very short channels (inner < kObsTinyInner elements, down to one): a thread per channel, so
+// that millions of channels do not become millions of blocks.
+constexpr int64_t kObsTinyInner = 64;
+template<typename T>
+__global__ void __launch_bounds__(kObsBlock)
+observer_tiny_channels(const T* __restrict__ in, int64_t channels, int64_t inner, int bits,
+                       int scheme, int formula, T* __restrict__ scale,
+                       T* __restrict__ zero_point) {
+  const int64_t step = (int64_t)gridDim.x * kObsBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kObsBlock + threadIdx.x; c < channels; c += step) {
+    const T* p = in + c * inner;
+    T vmax = p[0];
+    T vmin = vmax;
+    for (int64_t i = 1; i < inner; ++i) {
+      vmax = OpMax()(vmax, p[i]);
+      vmin = OpMin()(vmin, p[i]);
+    }
+    observer_channel<T>(vmax, vmin, bits, scheme, formula, scale + c, zero_point + c);
+  }
 }
 
 // ---- moving_average_min_max_observer ------------------------------------------------------------
@@ -437,17 +482,32 @@ int launch_observer(hipStream_t st, const void* in, void* workspace, void* scale
   const T* src = static_cast<const T*>(in);
   T* sc = static_cast<T*>(scale);
   T* zp = static_cast<T*>(zero_point);
+  constexpr int64_t kMaxGrid = 1 << 22;  // blocks; beyond, a block walks several slices
+  if (inner < kObsTinyInner) {
+    int64_t grid = (channels + kObsBlock - 1) / kObsBlock;
+    if (grid > kMaxGrid) grid = kMaxGrid;
+    observer_tiny_channels<T><<<(int)grid, kObsBlock, 0, st>>>(src, channels, inner, bits, scheme,
+                                                              formula, sc, zp);
+    return ofq_check_launch();
+  }
+  const int64_t total = channels * splits;
+  const int grid = (int)(total < kMaxGrid ? total : kMaxGrid);
   if (splits == 1) {
-    observer_partial<T, true><<<(int)channels, kObsBlock, 0, st>>>(src, inner, 1, nullptr, bits,
-                                                                  scheme, formula, sc, zp);
+    observer_partial<T, true><<<grid, kObsBlock, 0, st>>>(src, inner, 1, total, nullptr, bits,
+                                                         scheme, formula, sc, zp);
     return ofq_check_launch();
   }
   T* part = static_cast<T*>(workspace);
-  observer_partial<T, false><<<(int)(channels * splits), kObsBlock, 0, st>>>(
-      src, inner, splits, part, bits, scheme, formula, nullptr, nullptr);
-  const int fin_grid = (int)((channels + kObsBlock - 1) / kObsBlock);
-  observer_finalize<T><<<fin_grid, kObsBlock, 0, st>>>(part, channels, splits, bits, scheme,
-                                                       formula, sc, zp);
+  observer_partial<T, false><<<grid, kObsBlock, 0, st>>>(src, inner, splits, total, part, bits,
+                                                        scheme, formula, nullptr, nullptr);
+  if (splits > 32 && channels <= kMaxGrid) {
+    observer_finalize_wide<T><<<(int)channels, kObsBlock, 0, st>>>(part, splits, bits, scheme,
+                                                                  formula, sc, zp);
+  } else {
+    const int fin_grid = (int)((channels + kObsBlock - 1) / kObsBlock);
+    observer_finalize<T><<<fin_grid, kObsBlock, 0, st>>>(part, channels, splits, bits, scheme,
+                                                         formula, sc, zp);
+  }
   return ofq_check_launch();
 }
 
@@ -523,8 +583,8 @@ extern "C" int ofq_moving_average_min_max_observer(
   // is known on the device only.
   if (in_dtype == OFQ_F32) {
     observer_partial<float, false><<<(int)splits, kObsBlock, 0, st>>>(
-        static_cast<const float*>(in), elem_cnt, splits, static_cast<float*>(workspace), 0, 0, 0,
-        nullptr, nullptr);
+        static_cast<const float*>(in), elem_cnt, splits, splits, static_cast<float*>(workspace), 0,
+        0, 0, nullptr, nullptr);
     moving_average_finalize<float><<<1, kWave, 0, st>>>(
         static_cast<const float*>(workspace), splits, current_train_step, stop_update_after_iters,
         training, momentum, quantization_bit, scheme, formula, static_cast<float*>(moving_max),
@@ -532,8 +592,8 @@ extern "C" int ofq_moving_average_min_max_observer(
         static_cast<float*>(zero_point));
   } else {
     observer_partial<double, false><<<(int)splits, kObsBlock, 0, st>>>(
-        static_cast<const double*>(in), elem_cnt, splits, static_cast<double*>(workspace), 0, 0,
-        0, nullptr, nullptr);
+        static_cast<const double*>(in), elem_cnt, splits, splits, static_cast<double*>(workspace),
+        0, 0, 0, nullptr, nullptr);
     moving_average_finalize<double><<<1, kWave, 0, st>>>(
         static_cast<const double*>(workspace), splits, current_train_step,
         stop_update_after_iters, training, momentum, quantization_bit, scheme, formula,

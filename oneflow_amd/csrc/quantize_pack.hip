@@ -100,6 +100,72 @@ quantize_pack_rows(const typename TT<T>::storage* __restrict__ x, uint8_t* __res
   }
 }
 
+// groups along K of any length that is a multiple of 8 (a whole row per group = per-channel
+// quantisation, or lengths the sub-group kernel above does not take): a block per group, 64 to
+// 256 threads, two sweeps over the group -- extremes, then codes; the second sweep finds the
+// group in cache.  Same arithmetic per element, and max / min do not depend on the order.
+template<typename T, bool SYM, bool SIGNED, int BITS>
+__global__ void __launch_bounds__(256)
+quantize_pack_long_rows(const typename TT<T>::storage* __restrict__ x, uint8_t* __restrict__ q,
+                        typename TT<T>::storage* __restrict__ scale,
+                        typename TT<T>::storage* __restrict__ zero, int64_t g) {
+  typedef typename TT<T>::storage S;
+  __shared__ float smem[256 / kWave];
+  const int64_t grp = blockIdx.x;
+  const S* xg = x + grp * g;
+  const int64_t pieces = g >> 3;
+  auto load8 = [&](int64_t p, float (&v)[8]) {
+    S raw[8];
+    if (sizeof(S) == 2) {
+      *reinterpret_cast<u32x4*>(raw) = *reinterpret_cast<const u32x4*>(xg + p * 8);
+    } else {
+      reinterpret_cast<u32x4*>(raw)[0] = reinterpret_cast<const u32x4*>(xg + p * 8)[0];
+      reinterpret_cast<u32x4*>(raw)[1] = reinterpret_cast<const u32x4*>(xg + p * 8)[1];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = TT<T>::load(&raw[e]);
+  };
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int64_t p = threadIdx.x; p < pieces; p += blockDim.x) {
+    float v[8];
+    load8(p, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      mn = fminf(mn, v[e]);
+      mx = fmaxf(mx, v[e]);
+    }
+  }
+  mn = block_reduce(mn, OpMin(), smem);
+  mx = block_reduce(mx, OpMax(), smem);
+  const float amax = fmaxf(fabsf(mn), fabsf(mx));
+  const float sc = group_scale<SYM, BITS>(mn, mx, amax);
+  if (threadIdx.x == 0) {
+    TT<T>::store(&scale[grp], sc);
+    if (!SYM) TT<T>::store(&zero[grp], mn);
+  }
+  const int64_t base = grp * g;
+  for (int64_t p = threadIdx.x; p < pieces; p += blockDim.x) {
+    float v[8];
+    load8(p, v);
+    uint32_t c[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) c[e] = (uint32_t)quant_code<SYM, SIGNED, BITS>(v[e], sc, mn);
+    if (BITS == 8) {
+      u32x2 w;
+      w[0] = (c[0] & 0xFF) | ((c[1] & 0xFF) << 8) | ((c[2] & 0xFF) << 16) | (c[3] << 24);
+      w[1] = (c[4] & 0xFF) | ((c[5] & 0xFF) << 8) | ((c[6] & 0xFF) << 16) | (c[7] << 24);
+      *reinterpret_cast<u32x2*>(q + base + p * 8) = w;
+    } else {
+      uint32_t w = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        w |= ((((c[2 * b] & 0xF) << 4) | (c[2 * b + 1] & 0xF)) << (8 * b));
+      }
+      *reinterpret_cast<uint32_t*>(q + ((base + p * 8) >> 1)) = w;
+    }
+  }
+}
+
 // any grouping: x viewed as [outer][groups][g][inner]; one thread per (outer, group, column) for
 // 8-bit codes, per (outer, group, column pair) for 4-bit codes packed along the inner axis, per
 // (outer, group) when inner == 1 (pairs then lie inside the group, g is even)
@@ -174,6 +240,11 @@ int launch_variant(hipStream_t st, const void* x, void* q, void* scale, void* ze
     const int64_t grid = (slots + 255) / 256;
     if (grid > 0x7FFFFFFF) return OFQ_ERR_UNSUPPORTED;
     quantize_pack_rows<T, SYM, SIGNED, BITS><<<(int)grid, 256, 0, st>>>(xs, qs, ss, zs, og, (int)L);
+  } else if (group_dim == 1 && g % 8 == 0 && ofq_aligned16(x)
+             && ((reinterpret_cast<uintptr_t>(q) & 7u) == 0) && og <= 0x7FFFFFFF) {
+    int threads = (int)((L + 63) / 64 * 64);
+    if (threads > 256) threads = 256;
+    quantize_pack_long_rows<T, SYM, SIGNED, BITS><<<(int)og, threads, 0, st>>>(xs, qs, ss, zs, g);
   } else {
     const int64_t threads = og * (inner / ((BITS == 4 && inner > 1) ? 2 : 1));
     const int64_t grid = (threads + 255) / 256;

@@ -27,13 +27,16 @@ def _same_values_and_nan(a, b):
 
 
 # shapes/attribute grid of the reference tests (test_min_max_observer.py:137-148)
-@pytest.mark.parametrize("shape", [(9, 40, 20, 10), (4096, 64), (3, 5)])
+@pytest.mark.parametrize("shape", [(9, 40, 20, 10), (4096, 64), (3, 5), (300001,), (2, 700000), (70000, 3)])
 @pytest.mark.parametrize("bits", [8, 4, 2])
 @pytest.mark.parametrize("scheme", ["symmetric", "affine"])
 @pytest.mark.parametrize("per_layer", [True, False])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_observer_quantize_fake(shape, bits, scheme, per_layer, dtype):
     import oneflow_amd as flow
+    if len(shape) == 1 and not per_layer and scheme == "affine":
+        pytest.skip("one-element channels: the affine scale is (max - min) / .. = 0, and what "
+                    "follows is 0/0 in the reference too")
     rng = np.random.Generator(np.random.PCG64(hash((shape, bits, scheme, per_layer)) % 2**32))
     x = (rng.random(shape) - 0.5).astype(dtype)
     s_ref, z_ref = O.min_max_observer(x, "google", bits, scheme, per_layer)

@@ -28,6 +28,7 @@ VARIANTS = [(True, True), (True, False), (False, False)]
     (64, 256, 1, 128), (37, 512, 1, 64), (8, 64, 1, 8), (5, 1024, 1, 512),   # lane-group kernel
     (48, 96, 1, 48), (7, 126, 1, 6), (64, 128, 0, 16), (30, 50, 0, 10),      # strided kernel
     (128, 64, 0, 128), (3, 40, 1, 40),
+    (33, 4096, 1, 4096), (20, 11008, 1, 11008), (9, 2048, 1, 1024), (70, 960, 1, 96),  # block per group
 ])
 def test_bit_exact_against_the_oracle(bits, symmetric, signed, t, n, k, group_dim, group_size):
     rng = np.random.Generator(np.random.PCG64(n * 7 + k + bits + group_size))
