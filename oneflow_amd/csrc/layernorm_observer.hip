@@ -464,6 +464,8 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
     ln_observer_rows<T, 2, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else if (vec_ok && npacks <= 4 * kLnBlock) {
     ln_observer_rows<T, 4, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
+  } else if (vec_ok && npacks <= 8 * kLnBlock) {
+    ln_observer_rows<T, 8, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else {
     ln_observer_rows_generic<T, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols,
                                                                       eps, sk);

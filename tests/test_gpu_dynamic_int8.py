@@ -21,7 +21,8 @@ def _cfg5_inputs(rows=2048, cols=4096, t="f16"):
 
 
 @pytest.mark.parametrize("t,rows,cols", [("f16", 2048, 4096), ("bf16", 64, 4096), ("f32", 33, 1000),
-                                         ("f16", 7, 8200), ("f16", 5, 24)])
+                                         ("f16", 7, 8200), ("f16", 5, 24), ("f16", 12, 11008),
+                                         ("f32", 6, 16384), ("bf16", 3, 16392)])
 def test_layer_norm_observer(t, rows, cols):
     import oneflow_amd as flow
     x, gamma, beta = _cfg5_inputs(rows, cols, t)
@@ -49,7 +50,7 @@ def test_layer_norm_observer(t, rows, cols):
 
 @pytest.mark.parametrize("t,rows,cols", [("f16", 2048, 4096), ("bf16", 300, 4096), ("f32", 33, 1000),
                                          ("f16", 7, 8200), ("bf16", 5, 24), ("f32", 40, 2048),
-                                         ("bf16", 9, 16384)])
+                                         ("bf16", 9, 16384), ("f16", 4, 11008)])
 @pytest.mark.parametrize("use_bias,use_skip", [(True, True), (False, True), (True, False)])
 def test_skip_layer_norm_observer(t, rows, cols, use_bias, use_skip):
     """The residual input of skip_layer_norm in front of the same LayerNorm + observer: every
