@@ -62,8 +62,13 @@ def _require_gpu(*tensors):
 
 
 def _contig(t):
-    # the runtime hands kernels contiguous inputs (op_interpreter_util.cpp:156)
-    return None if t is None else t.contiguous()
+    # the runtime hands kernels contiguous inputs (op_interpreter_util.cpp:156) in buffers of its
+    # own allocator (512-byte aligned); a view that starts off a 16-byte boundary is copied, since
+    # the kernels use 128-bit accesses
+    if t is None:
+        return None
+    t = t.contiguous()
+    return t.clone() if t.data_ptr() % 16 else t
 
 
 def _workspace(nbytes, device):

@@ -514,3 +514,32 @@ def test_groups_along_n_large_m(m, n, k, g, num_bits):
             for got in outs:
                 H.assert_linear_parity(got, ref, t, f"m={m} n={n} k={k} {t} {symmetric} {qdt}")
             assert H.rel_l2(O.to_f32(outs[0]), O.to_f32(outs[1])) < 1e-3
+
+
+def test_views_off_the_16_byte_grid():
+    """Inputs that are views starting off a 16-byte boundary (the kernels use 128-bit accesses):
+    the Python layer copies them; results equal those of the aligned tensors."""
+    import torch
+    import oneflow_amd as flow
+    rng = np.random.Generator(np.random.PCG64(31))
+    m, n, k, g = 3, 64, 256, 64
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), "f16")
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    w, scale, _ = H.quantize_groupwise(wf, 8, True, 1, g, np.int8, "f16")
+    b = H.as_T(rng.standard_normal(n).astype(np.float32), "f16")
+
+    def shifted(a):
+        t = H.to_torch(a)
+        buf = torch.empty(t.numel() + 1, dtype=t.dtype, device="cuda")
+        v = buf[1:].view(t.shape)
+        v.copy_(t)
+        assert v.data_ptr() % 16 != 0
+        return v
+    ref = _run(x, w, scale, None, b, 8, True, 1, g)
+    got = flow._C.fused_linear_with_groupwise_quantized_weight(
+        shifted(x), shifted(w), shifted(scale), b=shifted(b), num_bits=8, symmetric=True,
+        group_dim=1, group_size=g)
+    assert np.array_equal(H.to_numpy(got), ref)
+    deq = flow._C.groupwise_dequantize(shifted(w), shifted(scale), num_bits=8, symmetric=True,
+                                       group_dim=1, group_size=g)
+    assert np.array_equal(H.to_numpy(deq), O.groupwise_dequantize(w, scale, None, 8, True, 1, g))
