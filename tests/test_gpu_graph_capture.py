@@ -76,11 +76,32 @@ def test_fused_linear_in_a_graph(m, n, k):
     _capture_and_check(inputs, run)
 
 
-def test_dynamic_int8_chain_in_a_graph():
+@pytest.mark.parametrize("m", [1, 40, 100])
+def test_fused_linear_groups_along_n_in_a_graph(m):
+    """group_dim = 0: the streaming kernel (m <= 64) and, beyond, dequantise + copy-fed GEMM in the
+    workspace the Python layer allocates before capture."""
+    import oneflow_amd as flow
+    rng = H.rng_for(27, 0)
+    n, k, g = 512, 512, 64
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    w, scale, zero = H.quantize_groupwise(wf, 4, False, 0, g, np.uint8, "f16")
+    w, scale, zero = _t(w), _t(scale), _t(zero)
+
+    def inputs(seed):
+        return [_t(H.rng_for(28, seed).standard_normal((m, k)).astype(np.float16))]
+
+    def run(x):
+        return flow._C.fused_linear_with_groupwise_quantized_weight(
+            x, w, scale, w_zero=zero, num_bits=4, symmetric=False, group_dim=0, group_size=g)
+    _capture_and_check(inputs, run)
+
+
+@pytest.mark.parametrize("rows", [300, 4])
+def test_dynamic_int8_chain_in_a_graph(rows):
     """LayerNorm+observer -> quantization to int8 -> matmul_quant, captured as one graph."""
     import torch
     import oneflow_amd as flow
-    rows, cols, n = 300, 1024, 704
+    cols, n = 1024, 704   # 4 rows: the streaming int8 kernel; 300: the tiled GEMM
     rng = H.rng_for(23, 0)
     gamma = _t((1 + 0.1 * rng.standard_normal(cols)).astype(np.float16))
     beta = _t((0.1 * rng.standard_normal(cols)).astype(np.float16))
