@@ -460,6 +460,25 @@ def secondary(L, _lib, torch, dev, args):
         "us": round(us, 2), "tops": round(tops, 1),
         "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": MFMA_PEAK_TFLOPS["i8"],
                      "unit": "TOP/s", "frac": round(tops / MFMA_PEAK_TFLOPS["i8"], 4)}}
+    # a batch of 256 rows on a square weight: 32 x 1 tiles of 128 columns, so K is cut into slices
+    # in the workspace the op asks for
+    mm, nn = 256, 4096
+    wsq = torch.randint(-127, 128, (nn, k), dtype=torch.int8, device=dev)
+    wssc = torch.empty(nn, device=dev).uniform_(1e-3, 1e-2)
+    osq = torch.empty((mm, nn), dtype=torch.float16, device=dev)
+    mq_ws_bytes = L.ofq_matmul_quant_workspace_bytes(mm, nn, k)
+    mq_ws = torch.empty(max(mq_ws_bytes, 16), dtype=torch.uint8, device=dev)
+    us = timeit(lambda: chk(L.ofq_matmul_quant_ws(cs(), a8[0].data_ptr(), wsq.data_ptr(), s.data_ptr(),
+                                                  wssc.data_ptr(), None, osq.data_ptr(), _lib.F16, mm,
+                                                  nn, k, mq_ws.data_ptr(), mq_ws_bytes),
+                            "matmul_quant k slices"))
+    tops = 2.0 * mm * nn * k / (us * 1e-6) / 1e12
+    out["matmul_quant_i8_m256_4096x4096"] = {
+        "us": round(us, 2), "tops": round(tops, 1), "workspace_bytes": int(mq_ws_bytes),
+        "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": MFMA_PEAK_TFLOPS["i8"],
+                     "unit": "TOP/s", "frac": round(tops / MFMA_PEAK_TFLOPS["i8"], 4)}}
+    del wsq, osq, mq_ws
+
     # the same op at decode (m = 1 and 16): the streaming int8 kernel; 6 weight sets cycled so that
     # no launch finds its weight in the caches
     reps_w = 6

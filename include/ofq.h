@@ -266,6 +266,18 @@ int ofq_fused_glu_gq(void* stream, const void* x, const void* w, const void* w_s
 int ofq_matmul_quant(void* stream, const void* a, const void* b, const float* a_scale,
                      const float* b_scale, const void* bias, void* out, int out_dtype, int64_t m,
                      int64_t n, int64_t k);
+/*
+ * The same op with an optional workspace (the op's tmp_buffer).  ofq_matmul_quant_workspace_bytes()
+ * is non-zero when 64 < m and the 128-wide output tiles alone would leave most CUs without a
+ * block: K is then cut into up to 8 slices that run as separate blocks, each writing its int32
+ * partial sums to the workspace (splits * m * n * 4 bytes), and a second kernel adds the slices
+ * (integer addition: the result does not depend on the order) and applies the epilogue.  Same
+ * bits as ofq_matmul_quant, which is this call with workspace NULL.
+ */
+size_t ofq_matmul_quant_workspace_bytes(int64_t m, int64_t n, int64_t k);
+int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, const float* a_scale,
+                        const float* b_scale, const void* bias, void* out, int out_dtype,
+                        int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

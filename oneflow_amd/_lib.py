@@ -47,6 +47,8 @@ SIGNATURES = {
     "ofq_fused_glu_gq": (_i, [_vp] * 13 + [_i, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64]),
     "ofq_groupwise_quantize": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64]),
     "ofq_matmul_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64]),
+    "ofq_matmul_quant_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "ofq_matmul_quant_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _vp, _sz]),
 }
 
 

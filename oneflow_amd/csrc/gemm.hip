@@ -262,9 +262,115 @@ using namespace ofq;
 // rows of a up to which matmul_quant streams the weights instead of tiling them
 static constexpr int64_t kMatmulQuantRowsMaxM = 64;
 
+namespace ofq {
+namespace {
+
+// K slices of the int8 GEMM when its 128-wide tiles alone would leave most CUs without a block:
+// as many as still fit one resident round (256x128 tiles: one block per CU; 128x128: two), each
+// at least 4 k-tiles of 128.
+int mq_splits(int64_t m, int64_t n, int64_t k) {
+  // long rows (k >= 8192) already pay for slices from 33 rows of a on: 4096 x 11008 at m = 64
+  // streams in 33 us and runs in 22 us as slices
+  if (m <= (k >= 8192 ? kMatmulQuantRowsMaxM / 2 : kMatmulQuantRowsMaxM) || k % 128 != 0) return 1;
+  const int64_t bm = m > 128 ? 256 : 128;
+  const int64_t slots = m > 128 ? 256 : 512;
+  const int64_t blocks = ((m + bm - 1) / bm) * ((n + 127) / 128);
+  int64_t s = slots / blocks;
+  const int64_t kt = k / 128;
+  if (s > 8) s = 8;
+  if (s > kt / 4) s = kt / 4;
+  if (s < 1) s = 1;
+  while (s > 1 && ((kt + s - 1) / s) * (s - 1) >= kt) --s;  // no empty last slice
+  return (int)s;
+}
+
+// adds the int32 slices (integer addition: any order gives the same sum) and applies the
+// epilogue of EpScale
+template<typename T, int VEC>
+__global__ void __launch_bounds__(256)
+splitk_finalize_i32(const int* __restrict__ part, const float* __restrict__ a_scale,
+                    const float* __restrict__ b_scale,
+                    const typename TT<T>::storage* __restrict__ bias,
+                    typename TT<T>::storage* __restrict__ out, int64_t MN, int N, int splits) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (i >= MN) return;
+  int acc[VEC];
+  if constexpr (VEC == 4) {
+    const i32x4 v = *reinterpret_cast<const i32x4*>(part + i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = v[e];
+    for (int sidx = 1; sidx < splits; ++sidx) {
+      const i32x4 u = *reinterpret_cast<const i32x4*>(part + (int64_t)sidx * MN + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] += u[e];
+    }
+  } else {
+    acc[0] = part[i];
+    for (int sidx = 1; sidx < splits; ++sidx) acc[0] += part[(int64_t)sidx * MN + i];
+  }
+  const int n = (int)(i % N);  // VEC divides N: the VEC elements share a row
+  const float sa = a_scale[0];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    float r = (float)acc[e] * (sa * b_scale[n + e]);
+    if (bias != nullptr) r = r + TT<T>::load(bias + n + e);
+    TT<T>::store(out + i + e, r);
+  }
+}
+
+template<typename T>
+int launch_mq_split(hipStream_t st, const void* a, const BCopyParams& bp, const float* a_scale,
+                    const float* b_scale, const void* bias, void* out, int64_t m, int64_t n,
+                    int64_t k, float* partials, int splits) {
+  typedef typename TT<T>::storage S;
+  EpPartialI32::Params pp;
+  pp.out = partials;
+  int rc;
+  if (m > 128) {
+    rc = launch_core2<MfmaI8, B2Copy<128, 512>, EpPartialI32, 256, 128, 4, 2>(st, a, k, bp, pp, m,
+                                                                             n, k / 128, splits);
+  } else {
+    rc = launch_core2<MfmaI8, B2Copy<128, 512>, EpPartialI32, 128, 128, 4, 2>(st, a, k, bp, pp, m,
+                                                                             n, k / 128, splits);
+  }
+  if (rc != OFQ_OK) return rc;
+  const int64_t mn = m * n;
+  const int* pi = reinterpret_cast<const int*>(partials);
+  if (n % 4 == 0) {
+    splitk_finalize_i32<T, 4><<<(unsigned)((mn / 4 + 255) / 256), 256, 0, st>>>(
+        pi, a_scale, b_scale, static_cast<const S*>(bias), static_cast<S*>(out), mn, (int)n, splits);
+  } else {
+    splitk_finalize_i32<T, 1><<<(unsigned)((mn + 255) / 256), 256, 0, st>>>(
+        pi, a_scale, b_scale, static_cast<const S*>(bias), static_cast<S*>(out), mn, (int)n, splits);
+  }
+  return ofq_check_launch();
+}
+
+}  // namespace
+}  // namespace ofq
+
+extern "C" size_t ofq_matmul_quant_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+  if (m <= 0 || n <= 0 || k <= 0) return 0;
+  const int splits = ofq::mq_splits(m, n, k);
+  return splits > 1 ? (size_t)splits * (size_t)m * (size_t)n * 4 : 0;
+}
+
+extern "C" int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, const float* a_scale,
+                                   const float* b_scale, const void* bias, void* out, int out_dtype,
+                                   int64_t m, int64_t n, int64_t k, void* workspace,
+                                   size_t workspace_bytes);
+
 extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, const float* a_scale,
                                 const float* b_scale, const void* bias, void* out, int out_dtype,
                                 int64_t m, int64_t n, int64_t k) {
+  return ofq_matmul_quant_ws(stream, a, b, a_scale, b_scale, bias, out, out_dtype, m, n, k, nullptr,
+                             0);
+}
+
+extern "C" int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, const float* a_scale,
+                                   const float* b_scale, const void* bias, void* out, int out_dtype,
+                                   int64_t m, int64_t n, int64_t k, void* workspace,
+                                   size_t workspace_bytes) {
   OFQ_RETURN_IF(out_dtype != OFQ_F16 && out_dtype != OFQ_BF16 && out_dtype != OFQ_F32,
                 OFQ_ERR_BAD_DTYPE);
   OFQ_RETURN_IF(m < 0 || n < 0 || k <= 0, OFQ_ERR_BAD_SHAPE);
@@ -278,15 +384,32 @@ extern "C" int ofq_matmul_quant(void* stream, const void* a, const void* b, cons
                 OFQ_ERR_NULL_POINTER);
   OFQ_RETURN_IF(!ofq_aligned16(a) || !ofq_aligned16(b) || !ofq_aligned16(out), OFQ_ERR_MISALIGNED);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  BCopyParams bp;
+  bp.b = static_cast<const uint8_t*>(b);
+  bp.ldb = k;
+  bp.N = (int)n;
+  {
+    const int splits = mq_splits(m, n, k);
+    const size_t need = (size_t)splits * (size_t)m * (size_t)n * 4;
+    if (splits > 1 && workspace != nullptr && workspace_bytes >= need && ofq_aligned16(workspace)) {
+      float* part = static_cast<float*>(workspace);
+      switch (out_dtype) {
+        case OFQ_F16:
+          return launch_mq_split<f16>(st, a, bp, a_scale, b_scale, bias, out, m, n, k, part, splits);
+        case OFQ_BF16:
+          return launch_mq_split<bf16>(st, a, bp, a_scale, b_scale, bias, out, m, n, k, part,
+                                       splits);
+        default:
+          return launch_mq_split<float>(st, a, bp, a_scale, b_scale, bias, out, m, n, k, part,
+                                        splits);
+      }
+    }
+  }
   // few rows of a, or a K the GEMM's tiles do not divide: the weights stream once per 64 rows
   if ((m <= kMatmulQuantRowsMaxM || k % 128 != 0) && matmul_quant_rows_supported(m, n, k)) {
     return launch_matmul_quant_rows(st, a, b, a_scale, b_scale, bias, out, out_dtype, m, n, k);
   }
   OFQ_RETURN_IF(k % 128 != 0, OFQ_ERR_UNSUPPORTED);
-  BCopyParams bp;
-  bp.b = static_cast<const uint8_t*>(b);
-  bp.ldb = k;
-  bp.N = (int)n;
 #define OFQ_MQ(T)                                                                              \
   {                                                                                            \
     typedef EpScale<T> EP;                                                                     \

@@ -108,6 +108,23 @@ struct EpPartial {
   typedef float elem_t;
   static constexpr bool kSplit = true;
 };
+// Split-K of the int8 GEMM: the int32 partial sums go to the workspace bit for bit (the slot type
+// is float only because the epilogue's stores are typed by 4-byte elements; nothing is converted).
+struct EpPartialI32 {
+  struct Params {
+    float* out;
+  };
+  static __device__ __forceinline__ void convert4(const Params&, const int* acc, int,
+                                                  float* out4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out4[e] = __builtin_bit_cast(float, acc[e]);
+  }
+  static __device__ __forceinline__ float convert1(const Params&, int acc, int) {
+    return __builtin_bit_cast(float, acc);
+  }
+  typedef float elem_t;
+  static constexpr bool kSplit = true;
+};
 template<typename T>
 struct EpScale {
   struct Params {

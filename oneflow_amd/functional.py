@@ -518,7 +518,10 @@ def matmul_quant(a, b, a_scale, b_scale, bias=None, out_dtype=torch.float16):
     m, k = a.shape
     n = b.shape[0]
     out = torch.empty((m, n), dtype=out_dtype, device=a.device)
-    st = _lib.lib().ofq_matmul_quant(_stream(a), _ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale),
-                                     _ptr(bias), _ptr(out), _dt(out), m, n, k)
-    _lib.check("ofq_matmul_quant", st)
+    L = _lib.lib()
+    ws_bytes = L.ofq_matmul_quant_workspace_bytes(m, n, k)
+    ws = _workspace(ws_bytes, a.device) if ws_bytes else None
+    st = L.ofq_matmul_quant_ws(_stream(a), _ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale),
+                               _ptr(bias), _ptr(out), _dt(out), m, n, k, _ptr(ws), ws_bytes)
+    _lib.check("ofq_matmul_quant_ws", st)
     return out

@@ -420,9 +420,12 @@ class OfqMatmulQuantKernel final : public user_op::OpKernel, public user_op::Cud
       CHECK_EQ(bias->shape_view().elem_cnt(), n);
       CHECK_EQ(bias->data_type(), out->data_type());
     }
-    CheckOk(ofq_matmul_quant(RawStream(ctx), a->dptr(), b->dptr(), a_scale->dptr<float>(),
-                             b_scale->dptr<float>(), bias ? bias->dptr() : nullptr,
-                             out->mut_dptr(), ToOfq(out->data_type()), m, n, k),
+    user_op::Tensor* tmp = ctx->Tensor4ArgNameAndIndex("tmp_buffer", 0);
+    CheckOk(ofq_matmul_quant_ws(RawStream(ctx), a->dptr(), b->dptr(), a_scale->dptr<float>(),
+                                b_scale->dptr<float>(), bias ? bias->dptr() : nullptr,
+                                out->mut_dptr(), ToOfq(out->data_type()), m, n, k,
+                                tmp ? tmp->mut_dptr() : nullptr,
+                                tmp ? (size_t)tmp->shape_view().elem_cnt() : 0),
             "matmul_quant");
   }
   bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
@@ -433,6 +436,12 @@ class OfqMatmulQuantKernel final : public user_op::OpKernel, public user_op::Cud
       .SetCreateFn<OfqMatmulQuantKernel>()                                  \
       .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)      \
                        && (user_op::HobDataType("out", 0) == dtype))        \
+      .SetInferTmpSizeFn([](user_op::InferContext* ctx) -> size_t {         \
+        const ShapeView as = ctx->InputShape("a", 0);                       \
+        const int64_t k = as.At(as.NumAxes() - 1);                          \
+        return ofq_matmul_quant_workspace_bytes(as.elem_cnt() / k,          \
+                                                ctx->InputShape("b", 0).At(0), k); \
+      })                                                                    \
       .SetPriority(user_op::kKernelPriorityOptimized)
 REGISTER_OFQ_MATMUL_QUANT(DataType::kFloat16);
 REGISTER_OFQ_MATMUL_QUANT(DataType::kBFloat16);

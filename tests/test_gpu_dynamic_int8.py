@@ -219,3 +219,40 @@ def test_matmul_quant_few_rows_streaming(m, n, k, t):
                          {"f32": np.float32, "f16": np.float16, "bf16": np.uint16}[t])
     view = np.uint32 if t == "f32" else np.uint16
     assert np.array_equal(got[np.ix_(rows, cols)].view(view), ref.view(view))
+
+
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(65, 256, 2048), (128, 1000, 4096), (200, 130, 1024), (512, 384, 1024),
+                                   (300, 203, 1536), (40, 256, 8192)])
+def test_matmul_quant_k_slices(m, n, k, t):
+    """64 < m with few output tiles: with the workspace the op asks for, K is cut into slices whose
+    int32 partial sums are added by a second kernel.  Integer sums do not depend on the order, so
+    the result equals the one-kernel path bit for bit, and both equal the oracle."""
+    import torch
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    rng = np.random.Generator(np.random.PCG64(m + n + k))
+    a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, size=(n, k)).astype(np.int8)
+    a_scale = np.array([0.0211], np.float32)
+    b_scale = rng.uniform(1e-3, 1e-2, size=n).astype(np.float32)
+    bias = H.as_T(rng.standard_normal(n).astype(np.float32), t)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[t]
+    tcode = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16}[t]
+    need = L.ofq_matmul_quant_workspace_bytes(m, n, k)
+    assert need > 0 and need % (m * n * 4) == 0 and need // (m * n * 4) >= 2, need
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    at, bt, ast, bst, biast = map(H.to_torch, (a, b, a_scale, b_scale, bias))
+    outs = []
+    for wptr, wbytes in ((ws.data_ptr(), need), (None, 0)):
+        out = torch.empty((m, n), dtype=tdt, device="cuda")
+        rc = L.ofq_matmul_quant_ws(torch.cuda.current_stream().cuda_stream, at.data_ptr(),
+                                   bt.data_ptr(), ast.data_ptr(), bst.data_ptr(), biast.data_ptr(),
+                                   out.data_ptr(), tcode, m, n, k, wptr, wbytes)
+        assert rc == 0
+        outs.append(H.to_numpy(out))
+    view = np.uint32 if t == "f32" else np.uint16
+    assert np.array_equal(outs[0].view(view), outs[1].view(view))
+    ref = O.matmul_quant(a, b, a_scale, b_scale, bias,
+                         {"f32": np.float32, "f16": np.float16, "bf16": np.uint16}[t])
+    assert np.array_equal(outs[0].view(view), ref.view(view))

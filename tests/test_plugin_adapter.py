@@ -39,7 +39,7 @@ def test_registrations(plugin):
                  "grouped_linear_with_groupwise_quantized_weight"):
         assert len(seen[name]) == 3  # half, bfloat16, float
     assert all(t == 1 for _, t in seen["fused_layer_norm_min_max_observer"])
-    assert all(t == 0 for _, t in seen["matmul_quant"])
+    assert all(t == 1 for _, t in seen["matmul_quant"])   # K slices at 64 < m
     assert len(seen["groupwise_dequantize"]) == 3 and len(seen["min_max_observer"]) == 2
     assert len(seen["moving_average_min_max_observer"]) == 2
     # every kernel outranks a stock registration (priority 0); the observers and the fused linear
