@@ -421,8 +421,32 @@ def quantization(in_, scale, zero_point, quantization_formula="google", quantiza
     return out
 
 
+class _FakeQuantizationSTE(torch.autograd.Function):
+    """The reference's gradient of fake_quantization: the output gradient passes to ``in``
+    unchanged, scale and zero_point get none
+    (oneflow/core/autograd/gradient_funcs/fake_quantization.cpp:36-42)."""
+
+    @staticmethod
+    def forward(ctx, in_, scale, zero_point, formula, bit, scheme, zp_mode):
+        return _fake_quantization_forward(in_.detach(), scale, zero_point, formula, bit, scheme,
+                                          zp_mode)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return grad, None, None, None, None, None, None
+
+
 def fake_quantization(in_, scale, zero_point, quantization_formula="google", quantization_bit=8,
                       quantization_scheme="symmetric", *, zp_mode="float"):
+    if torch.is_grad_enabled() and in_.requires_grad:
+        return _FakeQuantizationSTE.apply(in_, scale, zero_point, quantization_formula,
+                                          quantization_bit, quantization_scheme, zp_mode)
+    return _fake_quantization_forward(in_, scale, zero_point, quantization_formula,
+                                      quantization_bit, quantization_scheme, zp_mode)
+
+
+def _fake_quantization_forward(in_, scale, zero_point, quantization_formula, quantization_bit,
+                               quantization_scheme, zp_mode):
     in_, scale, zero_point = _quant_common("fake_quantization", in_, scale, zero_point,
                                            quantization_formula, quantization_bit,
                                            quantization_scheme, None, zp_mode)

@@ -167,3 +167,20 @@ def test_moving_average_observer_large_and_checks():
     with pytest.raises(flow.CheckFailedError):
         flow._C.moving_average_min_max_observer(H.to_torch(x), st.to(torch.int32), mmax, mmin, True, 1,
                                                 "google", 8, "affine", 0.95)
+
+
+def test_fake_quantization_straight_through_gradient():
+    """in_grad = out_grad, no gradient for scale / zero_point
+    (core/autograd/gradient_funcs/fake_quantization.cpp:36-42)."""
+    import torch
+    import oneflow_amd as flow
+    x = torch.randn((64, 256), device="cuda", requires_grad=True)
+    s, z = flow._C.min_max_observer(x.detach(), "google", 8, "symmetric", False)
+    y = flow._C.fake_quantization(x, s, z, "google", 8, "symmetric")
+    assert y.requires_grad
+    g = torch.randn_like(y)
+    y.backward(g)
+    assert torch.equal(x.grad, g)
+    with torch.no_grad():
+        y2 = flow._C.fake_quantization(x, s, z, "google", 8, "symmetric")
+    assert not y2.requires_grad and torch.equal(y2, y.detach())
