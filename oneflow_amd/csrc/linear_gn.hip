@@ -1,5 +1,5 @@
-// fused_linear_with_groupwise_quantized_weight, groups along N (group_dim = 0), fp16 / bf16:
-// launcher of the streaming kernel of gemv_rows_gn.h.  x is taken 64 rows at a time (each pass
+// fused_linear_with_groupwise_quantized_weight, groups along N (group_dim = 0): launchers of the
+// streaming kernels of gemv_rows_gn.h (fp16 / bf16, and fp32 with 16 rows of x per pass).  x is taken 64 rows at a time (each pass
 // streams the weights once), so any m runs; at large m the caller prefers the two-pass GEMM when
 // it has a workspace.
 #include "gemv_rows_gn.h"
@@ -88,10 +88,75 @@ int launch_gn_part(hipStream_t st, const LinearArgs& a, int64_t m0, int m) {
 #undef OFQ_MT
 }
 
+// ---- fp32 activations: 16 rows of x per pass -------------------------------------------------------
+template<int BITS, bool SIGNED, int ZMODE>
+int launch_gn_f32_inst(hipStream_t st, const LinearArgs& a, const float* x, float* out, int m,
+                       int grid, int rows_per_block, size_t lds) {
+  auto kern = gemv_rows_f32_gn<BITS, SIGNED, ZMODE, 16>;
+  static bool attr_set = false;  // idempotent; a benign race at worst repeats the call
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
+        != hipSuccess) {
+      return OFQ_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  kern<<<grid, 16 * 64, lds, st>>>(x, static_cast<const uint8_t*>(a.w),
+                                  static_cast<const float*>(a.scale),
+                                  static_cast<const float*>(a.zero),
+                                  static_cast<const float*>(a.bias), out, m, (int)a.n, (int)a.k,
+                                  (int)a.group_size, rows_per_block);
+  return ofq_check_launch();
+}
+
+int launch_gn_f32(hipStream_t st, const LinearArgs& a) {
+  constexpr int kCUs = 256;
+  int rpb = (int)(((a.n + kCUs - 1) / kCUs + 15) / 16 * 16);
+  if (rpb > 16 * kRowsMaxTiles) rpb = 16 * kRowsMaxTiles;
+  if (rpb < 16) rpb = 16;
+  while (rpb > 16
+         && gemv_rows_f32_gn_lds_bytes(16, (int)a.k, (int)a.group_size, rpb, !a.symmetric)
+                > 160u * 1024u) {
+    rpb -= 16;
+  }
+  const size_t lds = gemv_rows_f32_gn_lds_bytes(16, (int)a.k, (int)a.group_size, rpb, !a.symmetric);
+  if (lds > 160u * 1024u) return OFQ_ERR_UNSUPPORTED;
+  const int grid = (int)((a.n + rpb - 1) / rpb);
+  const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
+  for (int64_t m0 = 0; m0 < a.m; m0 += 16) {
+    const int m = (int)(a.m - m0 < 16 ? a.m - m0 : 16);
+    const float* x = static_cast<const float*>(a.x) + m0 * a.k;
+    float* out = static_cast<float*>(a.out) + m0 * a.n;
+    int rc = OFQ_ERR_UNSUPPORTED;
+#define OFQ_R(B, SG, ZM)                              \
+  if (a.bits == B && a.w_signed == SG && zmode == ZM) \
+    rc = launch_gn_f32_inst<B, SG, ZM>(st, a, x, out, m, grid, rpb, lds);
+    OFQ_R(4, true, kZeroNone)
+    OFQ_R(4, false, kZeroSymU)
+    OFQ_R(4, false, kZeroAsym)
+    OFQ_R(8, true, kZeroNone)
+    OFQ_R(8, false, kZeroSymU)
+    OFQ_R(8, false, kZeroAsym)
+#undef OFQ_R
+    if (rc != OFQ_OK) return rc;
+  }
+  return OFQ_OK;
+}
+
 }  // namespace
 
 bool gemv_gn_supported(const LinearArgs& a) {
-  if (a.group_dim != 0 || (a.t_dtype != OFQ_F16 && a.t_dtype != OFQ_BF16)) return false;
+  if (a.group_dim != 0) return false;
+  if (a.t_dtype == OFQ_F32) {
+    const int ck32 = a.bits == 4 ? 128 : 64;
+    return (a.bits == 4 || a.bits == 8) && a.m >= 1 && a.k % ck32 == 0 && a.group_size % 16 == 0
+           && a.n % a.group_size == 0 && (a.symmetric || !a.w_signed) && a.k <= (1 << 20)
+           && a.n <= 0x7FFFFFFF - 64
+           && gemv_rows_f32_gn_lds_bytes(16, (int)a.k, (int)a.group_size, 16, !a.symmetric)
+                  <= 160u * 1024u;
+  }
+  if (a.t_dtype != OFQ_F16 && a.t_dtype != OFQ_BF16) return false;
   if ((a.bits != 4 && a.bits != 8) || a.m < 1) return false;
   const int ck = a.bits == 4 ? 128 : 64;
   if (a.k % ck != 0 || a.group_size % 16 != 0 || a.n % a.group_size != 0) return false;
@@ -103,6 +168,7 @@ bool gemv_gn_supported(const LinearArgs& a) {
 }
 
 int launch_gemv_gn(hipStream_t st, const LinearArgs& a) {
+  if (a.t_dtype == OFQ_F32) return launch_gn_f32(st, a);
   for (int64_t m0 = 0; m0 < a.m; m0 += 64) {
     const int m = (int)(a.m - m0 < 64 ? a.m - m0 : 64);
     const int rc = launch_gn_part(st, a, m0, m);
