@@ -3,6 +3,7 @@
 // experiments can instantiate tile configurations directly.
 #pragma once
 
+#include <atomic>
 #include "dequant_regs.h"
 #include "ofq_device.h"
 
@@ -548,7 +549,7 @@ int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::
   const size_t lds_bytes = NSTAGE * (size_t)(BM + BN) * kStageRow;
   auto kern = gemm_core2<MF, BP, EP, BM, BN, WM, WN, NSTAGE, DBG>;
   if (lds_bytes > 64 * 1024) {
-    static bool attr_set = false;  // idempotent; a benign race at worst repeats the call
+    static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
     if (!attr_set) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)

@@ -26,6 +26,7 @@
 //     groupwise_dequantize;
 //   - partial sums of the waves are combined through LDS, bias is added in fp32, one rounding
 //     to T.
+#include <atomic>
 #include "gemv_kernels.h"
 #include "gemv_rows.h"
 #include "ofq_device.h"
@@ -121,7 +122,7 @@ template<int NW, bool EXACT, bool SIGNED, int ZMODE>
 int launch_w4p_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block, size_t lds,
                     int cpg_shift) {
   auto kern = gemv_w4p_f16<NW, 1, EXACT, SIGNED, ZMODE>;
-  static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be allowed once
+  static std::atomic<bool> attr_set{false};  // more than 64 KB of dynamic LDS has to be allowed once
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
@@ -188,7 +189,7 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
 int launch_rows_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block,
                      size_t lds, int gs_shift) {
   auto kern = gemv_rows<T, BITS, SIGNED, ZMODE, NW, STAGED>;
-  static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be allowed once
+  static std::atomic<bool> attr_set{false};  // more than 64 KB of dynamic LDS has to be allowed once
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
@@ -334,7 +335,7 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT>
 int launch_rows_mt_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m,
                         int grid, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_mt<T, BITS, SIGNED, ZMODE, NW, MT>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
@@ -402,7 +403,7 @@ template<int BITS, bool SIGNED, int ZMODE>
 int launch_rows_f32_inst(hipStream_t st, const LinearArgs& a, const float* x, float* out, int m,
                          int grid, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_f32<BITS, SIGNED, ZMODE, 16>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
@@ -464,7 +465,7 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
 int launch_rows_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
                              int group_size, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_grouped<T, BITS, SIGNED, ZMODE, NW, STAGED>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
@@ -499,7 +500,7 @@ template<int NW, bool EXACT, bool SIGNED, int ZMODE>
 int launch_w4p_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
                             int group_size, int rows_per_block, size_t lds) {
   auto kern = gemv_w4p_f16_grouped<NW, EXACT, SIGNED, ZMODE>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
@@ -589,7 +590,7 @@ template<int NW, bool EXACT, bool SIGNED, int ZMODE>
 int launch_w4p_glu_inst(hipStream_t st, const LinearArgs& a, const GluArgs& glu, int grid,
                         int rows_per_block, size_t lds) {
   auto kern = gemv_w4p_f16_glu<NW, EXACT, SIGNED, ZMODE>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)

@@ -2,6 +2,7 @@
 // streaming kernels of gemv_rows_gn.h (fp16 / bf16, and fp32 with 16 rows of x per pass).  x is taken 64 rows at a time (each pass
 // streams the weights once), so any m runs; at large m the caller prefers the two-pass GEMM when
 // it has a workspace.
+#include <atomic>
 #include "gemv_rows_gn.h"
 #include "ofq_device.h"
 #include "ofq_internal.h"
@@ -13,7 +14,7 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT>
 int launch_gn_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m, int grid,
                    int rows_per_block, size_t lds) {
   auto kern = gemv_rows_gn<T, BITS, SIGNED, ZMODE, NW, MT>;
-  static bool attr_set = false;  // idempotent; a benign race at worst repeats the call
+  static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
@@ -93,7 +94,7 @@ template<int BITS, bool SIGNED, int ZMODE>
 int launch_gn_f32_inst(hipStream_t st, const LinearArgs& a, const float* x, float* out, int m,
                        int grid, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_f32_gn<BITS, SIGNED, ZMODE, 16>;
-  static bool attr_set = false;  // idempotent; a benign race at worst repeats the call
+  static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)

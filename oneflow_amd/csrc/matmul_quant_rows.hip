@@ -10,6 +10,7 @@
 // addition: the order cannot matter) and leave through the epilogue of the GEMM path,
 //   out = T(float(acc) * (a_scale * b_scale[n]) + bias[n]),
 // so both paths give the same bits.
+#include <atomic>
 #include "ofq_device.h"
 #include "ofq_internal.h"
 
@@ -124,7 +125,7 @@ int launch_inst(hipStream_t st, const uint8_t* a, const uint8_t* b, const float*
   const size_t lds = (size_t)NW * MT * 256 * 4;
   auto kern = matmul_quant_rows<T, NW, MT>;
   if (lds > 64 * 1024) {
-    static bool attr_set = false;  // idempotent; a benign race at worst repeats the call
+    static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
     if (!attr_set) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
