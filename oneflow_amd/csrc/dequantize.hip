@@ -110,54 +110,70 @@ dequant_vec8(const uint8_t* __restrict__ q, const typename TT<T>::storage* __res
   }
 }
 
-// ---- fp16, 8-bit codes, group axis innermost, 16 | group_size: native packed fp16 math -----
-// A lane owns 16 bytes of codes (one 128-bit load) and writes two 128-bit stores.  Bytes are
-// turned into fp16 by the 0x6400 trick: the half with bits 0x6400|b is exactly 1024 + b, so one
-// v_perm_b32 builds two halves and one packed subtract recovers the code exactly.
+// ---- fp16, 8-bit codes, group axis innermost, 8 | group_size: native packed fp16 math ------
+// A lane owns two packs of 8 codes, 64 packs apart: each of its two 64-bit loads is one of 64
+// consecutive ones (512 contiguous bytes per wave instruction) and each of its two 128-bit stores
+// one of 64 consecutive ones (1 KB per instruction) -- a lane that owned 16 consecutive codes
+// would write its 32 bytes as two interleaved half-used store instructions (measured 6 % slower).
+// Bytes are turned into fp16 by the 0x6400 trick: the half with bits 0x6400|b is exactly
+// 1024 + b, so one v_perm_b32 builds two halves and one packed subtract recovers the code.
 template<bool SIGNED, bool SYM>
+__device__ __forceinline__ u32x4 dequant8_f16_b8(u32x2 c, f16 s, f16 zin) {
+  f16 z = zin;
+  if (SYM) z = SIGNED ? (f16)0.0f : (f16)(-127.0f) * s;
+  const f16x2 s2 = {s, s};
+  const f16x2 z2 = {z, z};
+  const f16 off = SIGNED ? (f16)(-1152.0f) : (f16)(-1024.0f);
+  const f16x2 off2 = {off, off};
+  uint32_t r[4];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    uint32_t word = c[w];
+    if (SIGNED) word ^= 0x80808080u;  // two's complement -> offset binary
+    const uint32_t lo = __builtin_amdgcn_perm(word, 0x64646464u, 0x00050004u);
+    const uint32_t hi = __builtin_amdgcn_perm(word, 0x64646464u, 0x00070006u);
+    f16x2 a = __builtin_bit_cast(f16x2, lo) + off2;
+    f16x2 b = __builtin_bit_cast(f16x2, hi) + off2;
+    a = a * s2;
+    b = b * s2;
+    if (!(SYM && SIGNED)) {
+      a = a + z2;
+      b = b + z2;
+    }
+    r[2 * w] = __builtin_bit_cast(uint32_t, a);
+    r[2 * w + 1] = __builtin_bit_cast(uint32_t, b);
+  }
+  return u32x4{r[0], r[1], r[2], r[3]};
+}
+
+template<bool SIGNED, bool SYM, int PPL>
 __global__ void __launch_bounds__(256)
-dequant_f16_b8_rows(const u32x4* __restrict__ q, const f16* __restrict__ scale,
+dequant_f16_b8_rows(const u32x2* __restrict__ q, const f16* __restrict__ scale,
                     const f16* __restrict__ zero, u32x4* __restrict__ out, int64_t n_packs,
                     int64_t packs_per_group) {
-  const int64_t step = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < n_packs; p += step) {
-    const int64_t g = p / packs_per_group;
-    const u32x4 c = __builtin_nontemporal_load(q + p);
-    const f16 s = scale[g];
-    f16 z;
-    if (!SYM) {
-      z = zero[g];
-    } else if (SIGNED) {
-      z = (f16)0.0f;
-    } else {
-      z = (f16)(-127.0f) * s;
-    }
-    const f16x2 s2 = {s, s};
-    const f16x2 z2 = {z, z};
-    const f16 off = SIGNED ? (f16)(-1152.0f) : (f16)(-1024.0f);
-    const f16x2 off2 = {off, off};
-    uint32_t r[8];
+  // wave chunk = 64 * PPL consecutive packs; lane l takes packs l, 64 + l, ... of the chunk
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+  for (int64_t base = wave * (64 * PPL); base < n_packs; base += nwaves * (64 * PPL)) {
+    u32x2 c[PPL];
+    f16 s[PPL], z[PPL];
+    bool v[PPL];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      uint32_t word = c[w];
-      if (SIGNED) word ^= 0x80808080u;  // two's complement -> offset binary
-      const uint32_t lo = __builtin_amdgcn_perm(word, 0x64646464u, 0x00050004u);
-      const uint32_t hi = __builtin_amdgcn_perm(word, 0x64646464u, 0x00070006u);
-      f16x2 a = __builtin_bit_cast(f16x2, lo) + off2;
-      f16x2 b = __builtin_bit_cast(f16x2, hi) + off2;
-      a = a * s2;
-      b = b * s2;
-      if (!(SYM && SIGNED)) {
-        a = a + z2;
-        b = b + z2;
-      }
-      r[2 * w] = __builtin_bit_cast(uint32_t, a);
-      r[2 * w + 1] = __builtin_bit_cast(uint32_t, b);
+    for (int i = 0; i < PPL; ++i) {
+      const int64_t p = base + i * 64 + lane;
+      v[i] = p < n_packs;
+      c[i] = u32x2{0u, 0u};
+      if (v[i]) c[i] = __builtin_nontemporal_load(q + p);
+      const int64_t g = (v[i] ? p : 0) / packs_per_group;
+      s[i] = scale[g];
+      z[i] = SYM ? (f16)0.0f : zero[g];
     }
-    const u32x4 o0 = {r[0], r[1], r[2], r[3]};
-    const u32x4 o1 = {r[4], r[5], r[6], r[7]};
-    __builtin_nontemporal_store(o0, out + 2 * p);
-    __builtin_nontemporal_store(o1, out + 2 * p + 1);
+#pragma unroll
+    for (int i = 0; i < PPL; ++i) {
+      const int64_t p = base + i * 64 + lane;
+      if (v[i]) __builtin_nontemporal_store(dequant8_f16_b8<SIGNED, SYM>(c[i], s[i], z[i]), out + p);
+    }
   }
 }
 
@@ -179,11 +195,12 @@ int launch(hipStream_t st, const void* in, const void* scale, const void* zero, 
   const S* ze = static_cast<const S*>(zero);
   S* o = static_cast<S*>(out);
   if constexpr (BITS == 8 && sizeof(S) == 2 && TT<T>::dtype == OFQ_F16) {
-    if (inner == 1 && group_size % 16 == 0) {
-      const int64_t n_packs = elem_cnt / 16;
-      dequant_f16_b8_rows<SIGNED, SYM><<<grid_for(n_packs, 256), 256, 0, st>>>(
-          reinterpret_cast<const u32x4*>(q), sc, ze, reinterpret_cast<u32x4*>(o), n_packs,
-          group_size / 16);
+    if (inner == 1 && group_size % 8 == 0) {
+      const int64_t n_packs = elem_cnt / 8;
+      // two packs per lane; more packs per lane or more blocks per CU measure the same
+      dequant_f16_b8_rows<SIGNED, SYM, 2><<<grid_for((n_packs + 1) / 2, 256), 256, 0, st>>>(
+          reinterpret_cast<const u32x2*>(q), sc, ze, reinterpret_cast<u32x4*>(o), n_packs,
+          group_size / 8);
       return ofq_check_launch();
     }
   }
