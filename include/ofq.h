@@ -95,7 +95,8 @@ int ofq_groupwise_dequantize(void* stream, const void* in, const void* scale, co
  *   copy-fed MFMA GEMM runs on the result (the functor's own m > 8 decomposition); with NULL or
  *   a smaller buffer the weight tiles are dequantised inside the GEMM instead (same results up to
  *   fp32 summation order, slower at large m).  With group_dim 0 it is n*k*sizeof(T) for m > 64
- *   (same decomposition); without it the streaming kernel takes x 64 rows at a time.
+ *   (same decomposition; plus fp32 partial sums of K slices when there are few output tiles);
+ *   without it the streaming kernel takes x 64 rows at a time.
  */
 size_t ofq_fused_linear_gq_workspace_bytes(int w_dtype, int t_dtype, int num_bits, int symmetric,
                                            int group_dim, int64_t group_size, int64_t m,

@@ -239,10 +239,58 @@ int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t 
 // need 64 scales); above the streaming kernel's range the weight is dequantised once into the
 // workspace -- the reference functor's own decomposition for m > 8,
 // oneflow/core/functional/impl/quantization.cpp:341-350 -- and the copy-fed GEMM runs on it.
+namespace {
+
+// K slices of the copy-fed GEMM when its 256 x 128 tiles alone would leave most CUs without a
+// block (m = 256 at n = 4096: 32 tiles): as many as fit one resident round, each >= 4 k-tiles
+int gn_splits(const LinearArgs& a) {
+  const int64_t blocks = ((a.m + 255) / 256) * ((a.n + 127) / 128);
+  int64_t s = 256 / blocks;
+  const int64_t kt = a.k / 64;
+  if (s > 8) s = 8;
+  if (s > kt / 4) s = kt / 4;
+  if (s < 1) s = 1;
+  while (s > 1 && ((kt + s - 1) / s) * (s - 1) >= kt) --s;  // no empty last slice
+  return (int)s;
+}
+
+template<typename T, class MF>
+int launch_plain_split(hipStream_t st, const LinearArgs& a, const void* wt, float* partials,
+                       int splits) {
+  typedef typename TT<T>::storage S;
+  BCopyParams bp;
+  bp.b = static_cast<const uint8_t*>(wt);
+  bp.ldb = a.k * 2;
+  bp.N = (int)a.n;
+  EpPartial::Params pp;
+  pp.out = partials;
+  const int rc = launch_core2<MF, B2Copy<128, 512>, EpPartial, 256, 128, 4, 2>(
+      st, a.x, a.k * 2, bp, pp, a.m, a.n, a.k / 64, splits);
+  if (rc != OFQ_OK) return rc;
+  const int64_t mn = a.m * a.n;
+  const S* bias = static_cast<const S*>(a.bias);
+  S* out = static_cast<S*>(a.out);
+  if (a.n % 4 == 0) {
+    splitk_finalize<T, 4><<<(unsigned)((mn / 4 + 255) / 256), 256, 0, st>>>(partials, bias, out, mn,
+                                                                          (int)a.n, splits);
+  } else {
+    splitk_finalize<T, 1><<<(unsigned)((mn + 255) / 256), 256, 0, st>>>(partials, bias, out, mn,
+                                                                      (int)a.n, splits);
+  }
+  return ofq_check_launch();
+}
+
+inline size_t round_up_256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace
+
+// [dequantised weight n*k*sizeof(T), padded to 256 B][fp32 partial sums of the K slices, if any]
 size_t gemm_gn_workspace_bytes(const LinearArgs& a) {
   if (a.group_dim != 0 || (a.t_dtype != OFQ_F16 && a.t_dtype != OFQ_BF16)) return 0;
   if (a.m <= 64 || a.k % 64 != 0 || a.n % a.group_size != 0) return 0;
-  return (size_t)a.n * (size_t)a.k * 2;
+  const int splits = gn_splits(a);
+  return round_up_256((size_t)a.n * (size_t)a.k * 2)
+         + (splits > 1 ? (size_t)splits * (size_t)a.m * (size_t)a.n * 4 : 0);
 }
 
 int launch_gemm_gn(hipStream_t st, const LinearArgs& a, void* workspace) {
@@ -251,6 +299,15 @@ int launch_gemm_gn(hipStream_t st, const LinearArgs& a, void* workspace) {
                                           a.symmetric ? 1 : 0, a.n / a.group_size, a.group_size,
                                           a.k);
   if (rc != OFQ_OK) return rc;
+  const int splits = gn_splits(a);
+  if (splits > 1) {
+    float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace)
+                                               + round_up_256((size_t)a.n * (size_t)a.k * 2));
+    if (a.t_dtype == OFQ_F16) {
+      return launch_plain_split<f16, MfmaF16>(st, a, workspace, partials, splits);
+    }
+    return launch_plain_split<bf16, MfmaBF16>(st, a, workspace, partials, splits);
+  }
   if (a.t_dtype == OFQ_F16) return launch_plain<f16, MfmaF16>(st, a, workspace);
   return launch_plain<bf16, MfmaBF16>(st, a, workspace);
 }

@@ -83,7 +83,10 @@ def test_fused_linear_argument_errors(lib):
     assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 1, 128, 1, 4096, 4096) == 0
     # groups along N: no workspace up to 64 rows of x, the dequantised weight beyond
     assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 0, 128, 64, 4096, 4096) == 0
-    assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 0, 128, 65, 4096, 4096) == 4096 * 4096 * 2
+    # (32 tiles of 256 x 128 for m = 65: 8 K slices of fp32 partial sums behind the weight)
+    assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 0, 128, 65, 4096, 4096) \
+        == 4096 * 4096 * 2 + 8 * 65 * 4096 * 4
+    assert lib.ofq_fused_linear_gq_workspace_bytes(I8, F16, 4, 1, 0, 128, 2048, 11008, 4096) == 11008 * 4096 * 2
 
 
 def test_observer_and_quantization_argument_errors(lib):

@@ -481,7 +481,8 @@ def test_groups_along_n_streaming(t, num_bits, m, n, k, g):
         assert r < (3e-3 if t == "bf16" else 1e-4), r
 
 
-@pytest.mark.parametrize("m,n,k,g", [(65, 256, 512, 64), (130, 1024, 256, 128), (200, 352, 1024, 16)])
+@pytest.mark.parametrize("m,n,k,g", [(65, 256, 512, 64), (130, 1024, 256, 128), (200, 352, 1024, 16),
+                                     (300, 4096, 512, 128)])
 @pytest.mark.parametrize("num_bits", [4, 8])
 def test_groups_along_n_large_m(m, n, k, g, num_bits):
     """group_dim = 0 beyond 64 rows of x: with the workspace the op asks for (n*k*sizeof(T)) the
@@ -500,7 +501,7 @@ def test_groups_along_n_large_m(m, n, k, g, num_bits):
             wcode = _lib.I8 if qdt == np.int8 else _lib.U8
             need = L.ofq_fused_linear_gq_workspace_bytes(wcode, tcode, num_bits, int(symmetric), 0,
                                                          g, m, n, k)
-            assert need == n * k * 2, need
+            assert need >= n * k * 2, need   # + fp32 partial sums when K is cut into slices
             ws = torch.empty(need, dtype=torch.uint8, device="cuda")
             xt, wt, st, bt = map(H.to_torch, (x, w, scale, b))
             zt = H.to_torch(zero)
