@@ -12,7 +12,11 @@
  *     for the default stream), so the calls are safe under stream capture;
  *   - the return value is an ofq_status; invalid arguments are reported, never aborted on, and
  *     nothing is launched when the status is not OFQ_OK;
- *   - there is no global state: calls on different streams may run concurrently.
+ *   - calls on different streams, and on different devices, may run concurrently.  The only
+ *     state the library keeps is, per kernel, one bit per device saying that the kernel's
+ *     dynamic-LDS limit has been raised there (set at the first launch on the device that is
+ *     current in the calling thread; the caller makes the device of `stream` current, as the
+ *     OneFlow worker thread that owns a stream does, oneflow/core/ep/cuda/cuda_stream.cpp:209-213);
  * Pointers must be aligned to 16 bytes (OneFlow's allocator aligns to 512,
  * oneflow/core/common/util.h:158-160).
  */
@@ -89,6 +93,14 @@ int ofq_groupwise_dequantize(void* stream, const void* in, const void* scale, co
  *   [n, k/group_size] for group_dim 1, [n/group_size, k] for group_dim 0 (t_dtype),
  *   w_zero NULL iff symmetric, b[n] (t_dtype) or NULL, out[m,n] (t_dtype).
  * out = T( sum_k float(x * w~) + float(b) ), w~ = T(T(q)*scale) + zero as in groupwise_dequantize.
+ *   One family of kernels departs from the rounding of w~: fp16, 4-bit symmetric codes in an
+ *   int8 container (no zero term), groups along K with 128 | group_size, m <= 16 -- the Llama
+ *   decode case.  There the group scale multiplies the exact fp32 sum of x*q over the group, so
+ *   q*scale is never rounded to fp16; the result is closer to exact arithmetic and differs from
+ *   the composition above by ~3e-4 rel-L2 (contract: 1e-3).  Every other combination (uint8
+ *   container, a zero term, 8 bit, bf16, fp32, m > 16, groups along N) forms w~ with the two
+ *   roundings of groupwise_dequantize.  The same weights in the two containers can therefore
+ *   differ in the last bits of the output.
  * Any m is accepted (the reference kernel has no m limit either, :473,590).
  * workspace: optional.  ofq_fused_linear_gq_workspace_bytes() is non-zero only for large m on the
  *   GEMM path (n*k*sizeof(T)): with it the weight is dequantised once into the workspace and a

@@ -549,15 +549,8 @@ int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::
   const size_t lds_bytes = NSTAGE * (size_t)(BM + BN) * kStageRow;
   auto kern = gemm_core2<MF, BP, EP, BM, BN, WM, WN, NSTAGE, DBG>;
   if (lds_bytes > 64 * 1024) {
-    static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
-    if (!attr_set) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes)
-          != hipSuccess) {
-        return OFQ_ERR_LAUNCH;
-      }
-      attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+    if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)lds_bytes, lds_allowed)) return OFQ_ERR_LAUNCH;
   }
   if (splits < 1 || (splits > 1 && !EP::kSplit)) return OFQ_ERR_UNSUPPORTED;
   const int kt_split = (int)((KT + splits - 1) / splits);

@@ -131,6 +131,7 @@ ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
         float t = TT<T>::round((v[i][e] - mean) * inv);
         if (gamma) t = TT<T>::round(t * g[e]);
         if (beta) t = TT<T>::round(t + b[e]);
+        else if (gamma) t = t + 0.0f;  // the reference adds its default beta 0: -0 becomes +0
         o[e] = t;
         amax = fmaxf(amax, fabsf(t));
       }
@@ -309,6 +310,7 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
           for (int e = 0; e < 8; ++e) t[e] = (f16)((f[e] - mean) * inv);
           if (gamma) t = t * __builtin_bit_cast(f16x8, gr[i].q[0]);
           if (beta) t = t + __builtin_bit_cast(f16x8, br[i].q[0]);
+          else if (gamma) t = t + (f16)0.0f;  // the reference adds its default beta 0: -0 -> +0
           amax8 = __builtin_elementwise_max(amax8, __builtin_elementwise_abs(t));
           *reinterpret_cast<u32x4*>(yr + (int64_t)p * 8) = __builtin_bit_cast(u32x4, t);
         } else {
@@ -321,6 +323,7 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
             float t = TT<T>::round((f[e] - mean) * inv);
             if (gamma) t = TT<T>::round(t * g[e]);
             if (beta) t = TT<T>::round(t + b[e]);
+            else if (gamma) t = t + 0.0f;  // default beta 0 of the reference: -0 -> +0
             o[e] = t;
             amax = fmaxf(amax, fabsf(t));
           }
@@ -374,6 +377,7 @@ ln_observer_rows_generic(const typename TT<T>::storage* __restrict__ x,
     float t = TT<T>::round((input(c) - mean) * inv);
     if (gamma) t = TT<T>::round(t * TT<T>::load(gamma + c));
     if (beta) t = TT<T>::round(t + TT<T>::load(beta + c));
+    else if (gamma) t = t + 0.0f;  // default beta 0 of the reference: -0 -> +0
     TT<T>::store(yr + c, t);
     amax = fmaxf(amax, fabsf(t));
   }

@@ -22,8 +22,10 @@
 //     turn two's complement nibbles into offset binary.  The codes come out pairwise
 //     (e1,e5),(e0,e4),(e3,e7),(e2,e6) and x is permuted to match with four v_perm_b32;
 //   - w~ is then formed exactly as the reference does (packed fp16 multiply by the group scale,
-//     packed add of the zero term), which keeps the kernel bit-compatible with
-//     groupwise_dequantize;
+//     packed add of the zero term), bit-compatible with groupwise_dequantize -- in every kernel
+//     but the fp16 fast path for symmetric 4-bit codes in an int8 container (gemv_w4s_f16 and
+//     gemv_w4p_f16 with EXACT = false), which scales the exact fp32 group sum instead and never
+//     rounds q*scale to fp16 (~3e-4 rel-L2 from the composition);
 //   - partial sums of the waves are combined through LDS, bias is added in fp32, one rounding
 //     to T.
 #include <atomic>
@@ -122,15 +124,8 @@ template<int NW, bool EXACT, bool SIGNED, int ZMODE>
 int launch_w4p_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block, size_t lds,
                     int cpg_shift) {
   auto kern = gemv_w4p_f16<NW, 1, EXACT, SIGNED, ZMODE>;
-  static std::atomic<bool> attr_set{false};  // more than 64 KB of dynamic LDS has to be allowed once
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
                                   static_cast<const f16*>(a.scale),
                                   static_cast<const f16*>(a.zero),
@@ -189,15 +184,8 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
 int launch_rows_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block,
                      size_t lds, int gs_shift) {
   auto kern = gemv_rows<T, BITS, SIGNED, ZMODE, NW, STAGED>;
-  static std::atomic<bool> attr_set{false};  // more than 64 KB of dynamic LDS has to be allowed once
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(
       static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.w),
       static_cast<const uint16_t*>(a.scale), static_cast<const uint16_t*>(a.zero),
@@ -335,15 +323,8 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT>
 int launch_rows_mt_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m,
                         int grid, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_mt<T, BITS, SIGNED, ZMODE, NW, MT>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(
       static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(a.w),
       static_cast<const uint16_t*>(a.scale), static_cast<const uint16_t*>(a.zero),
@@ -403,15 +384,8 @@ template<int BITS, bool SIGNED, int ZMODE>
 int launch_rows_f32_inst(hipStream_t st, const LinearArgs& a, const float* x, float* out, int m,
                          int grid, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_f32<BITS, SIGNED, ZMODE, 16>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, 16 * 64, lds, st>>>(x, static_cast<const uint8_t*>(a.w),
                                   static_cast<const float*>(a.scale),
                                   static_cast<const float*>(a.zero),
@@ -465,15 +439,8 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, bool STAGED>
 int launch_rows_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
                              int group_size, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_grouped<T, BITS, SIGNED, ZMODE, NW, STAGED>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(g, m, k, group_size, ilog2_exact(group_size), rows_per_block);
   return ofq_check_launch();
 }
@@ -500,15 +467,8 @@ template<int NW, bool EXACT, bool SIGNED, int ZMODE>
 int launch_w4p_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
                             int group_size, int rows_per_block, size_t lds) {
   auto kern = gemv_w4p_f16_grouped<NW, EXACT, SIGNED, ZMODE>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(g, m, k, group_size, ilog2_exact(group_size / 128),
                                   rows_per_block);
   return ofq_check_launch();
@@ -590,15 +550,8 @@ template<int NW, bool EXACT, bool SIGNED, int ZMODE>
 int launch_w4p_glu_inst(hipStream_t st, const LinearArgs& a, const GluArgs& glu, int grid,
                         int rows_per_block, size_t lds) {
   auto kern = gemv_w4p_f16_glu<NW, EXACT, SIGNED, ZMODE>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
                                   static_cast<const f16*>(a.scale),
                                   static_cast<const f16*>(a.zero),

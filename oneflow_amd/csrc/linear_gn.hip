@@ -14,15 +14,8 @@ template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT>
 int launch_gn_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m, int grid,
                    int rows_per_block, size_t lds) {
   auto kern = gemv_rows_gn<T, BITS, SIGNED, ZMODE, NW, MT>;
-  static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(
       static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(a.w),
       static_cast<const uint16_t*>(a.scale), static_cast<const uint16_t*>(a.zero),
@@ -94,15 +87,8 @@ template<int BITS, bool SIGNED, int ZMODE>
 int launch_gn_f32_inst(hipStream_t st, const LinearArgs& a, const float* x, float* out, int m,
                        int grid, int rows_per_block, size_t lds) {
   auto kern = gemv_rows_f32_gn<BITS, SIGNED, ZMODE, 16>;
-  static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)
-        != hipSuccess) {
-      return OFQ_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+  if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, 16 * 64, lds, st>>>(x, static_cast<const uint8_t*>(a.w),
                                   static_cast<const float*>(a.scale),
                                   static_cast<const float*>(a.zero),

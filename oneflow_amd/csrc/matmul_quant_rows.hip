@@ -125,15 +125,8 @@ int launch_inst(hipStream_t st, const uint8_t* a, const uint8_t* b, const float*
   const size_t lds = (size_t)NW * MT * 256 * 4;
   auto kern = matmul_quant_rows<T, NW, MT>;
   if (lds > 64 * 1024) {
-    static std::atomic<bool> attr_set{false};  // idempotent: two threads at worst both make the call
-    if (!attr_set) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
-          != hipSuccess) {
-        return OFQ_ERR_LAUNCH;
-      }
-      attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
+    if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)lds, lds_allowed)) return OFQ_ERR_LAUNCH;
   }
   kern<<<grid, NW * 64, lds, st>>>(a, b, a_scale, b_scale, static_cast<const S*>(bias),
                                    static_cast<S*>(out), m, (int)n, (int)k, rpb);

@@ -129,3 +129,19 @@ static inline int ofq_check_launch() {
   return hipGetLastError() == hipSuccess ? OFQ_OK : OFQ_ERR_LAUNCH;
 }
 static inline bool ofq_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// A kernel that uses more than 64 KB of dynamic LDS has to be allowed to once per device.
+// `done` holds one bit per device ordinal (a function-local static of the launcher, one per
+// kernel instantiation); the call is idempotent, so two threads racing here at worst both make it.
+#include <atomic>
+static inline bool ofq_allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+    return false;
+  }
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
+}

@@ -23,6 +23,8 @@
 // kernels registered for the same (op, device, dtype)
 // (oneflow/core/framework/user_op_registry_manager.cpp:95-114).
 #include "oneflow/core/framework/framework.h"
+#include "oneflow/core/ep/cuda/cuda_stream.h"
+#include "oneflow/core/kernel/cuda_graph_support.h"
 
 #include "ofq.h"
 
@@ -30,16 +32,12 @@ namespace oneflow {
 
 namespace {
 
-// How the raw stream is obtained is the one place that differs between a real OneFlow build and
-// the standalone build: OneFlow hands out ep::CudaStream::cuda_stream()
-// (oneflow/core/ep/cuda/cuda_stream.h:91); on a ROCm build of the EP layer that handle IS the
-// hipStream_t.
+// OneFlow hands out the raw device stream through ep::CudaStream::cuda_stream()
+// (oneflow/core/ep/cuda/cuda_stream.h:91, the call of groupwise_quantization_kernels.cu:531); on
+// a ROCm build of the EP layer that handle IS the hipStream_t.  The standalone build carries the
+// same two headers with the same spelling, so this source is one text for both builds.
 inline void* RawStream(user_op::KernelComputeContext* ctx) {
-#ifdef OFQ_PLUGIN_STANDALONE
-  return ctx->stream() ? ctx->stream()->raw_stream() : nullptr;
-#else
   return ctx->stream()->As<ep::CudaStream>()->cuda_stream();
-#endif
 }
 
 inline int ToOfq(DataType dt) {
@@ -580,15 +578,6 @@ REGISTER_OFQ_GROUPED_LINEAR(DataType::kFloat);
 using namespace oneflow;
 
 namespace {
-class RawStreamHolder final : public ep::Stream {
- public:
-  explicit RawStreamHolder(void* s) : s_(s) {}
-  void* raw_stream() const override { return s_; }
-
- private:
-  void* s_;
-};
-
 const user_op::KernelRegistration* Lookup(const std::string& op, const user_op::KernelRegContext& c) {
   const user_op::KernelRegistration* best = nullptr;
   for (const auto& r : user_op::KernelRegistry()) {
@@ -670,7 +659,7 @@ extern "C" int ofq_plugin_run_fused_linear(void* stream, void* x, void* w, void*
   c.arg_dtypes["out"] = (DataType)t_dtype;
   const auto* r = Lookup("fused_linear_with_groupwise_quantized_weight", c);
   if (r == nullptr) return -1;
-  RawStreamHolder st(stream);
+  ep::CudaStream st(stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   const DataType T = (DataType)t_dtype;
@@ -706,7 +695,7 @@ extern "C" int ofq_plugin_run_layer_norm_observer(void* stream, void* x, void* g
   c.arg_dtypes["y"] = (DataType)t_dtype;
   const auto* r = Lookup("fused_layer_norm_min_max_observer", c);
   if (r == nullptr) return -1;
-  RawStreamHolder st(stream);
+  ep::CudaStream st(stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   const DataType T = (DataType)t_dtype;
@@ -735,7 +724,7 @@ extern "C" int ofq_plugin_run_matmul_quant(void* stream, void* a, void* b, void*
   c.arg_dtypes["out"] = (DataType)out_dtype;
   const auto* r = Lookup("matmul_quant", c);
   if (r == nullptr) return -1;
-  RawStreamHolder st(stream);
+  ep::CudaStream st(stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   ctx.AddTensor("a", {m, k}, DataType::kInt8, a);
@@ -760,7 +749,7 @@ extern "C" int ofq_plugin_run_grouped_linear(void* stream, int count, void* x, v
   c.arg_dtypes["ys"] = (DataType)t_dtype;
   const auto* r = Lookup("grouped_linear_with_groupwise_quantized_weight", c);
   if (r == nullptr) return -1;
-  RawStreamHolder st(stream);
+  ep::CudaStream st(stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   const DataType T = (DataType)t_dtype;

@@ -60,9 +60,11 @@ namespace ep {
 class Stream {
  public:
   virtual ~Stream() = default;
-  // the adapter only needs the raw HIP stream; a real build reaches it through its own
-  // ep::Stream subclass
-  virtual void* raw_stream() const { return nullptr; }
+  // oneflow/core/ep/include/stream.h:53-56: the device-specific stream is reached by a cast
+  template<typename T>
+  T* As() {
+    return static_cast<T*>(this);
+  }
 };
 }  // namespace ep
 
@@ -158,7 +160,6 @@ class OpKernel {
   virtual void Compute(KernelComputeContext*) const {}
   virtual bool AlwaysComputeWhenAllOutputsEmpty() const = 0;
 };
-class CudaGraphSupport {};
 
 // predicates: only what is needed to record and evaluate (device, dtype-of-arg) matches
 struct KernelRegContext {

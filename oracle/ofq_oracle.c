@@ -11,9 +11,11 @@
  *
  * Pinning status (what independent evidence fixes each function; see tests/test_oracle_*.py):
  *   min_max_observer / quantization / fake_quantization (f32):
- *       pinned by the known-answer table produced by the reference's own CPU kernels
- *       (tests/golden/ref_cpu_known_answers.json), by round-half-even tie vectors, and by
- *       invariants (|x/s - code| <= 0.5, row absmax -> +-(2^(b-1)-1), codes in range).
+ *       pinned by a 12-row known-answer table (tests/golden/ref_cpu_known_answers.json) that a
+ *       test rebuilds in exact rational arithmetic with one fp32 rounding per operation of
+ *       min_max_observer_kernel.cpp:22-46 / quantization_kernel.cpp:22-48, symmetric and affine,
+ *       by round-half-even tie vectors, and by invariants (|x/s - code| <= 0.5, row absmax ->
+ *       +-(2^(b-1)-1), codes in range).
  *   groupwise_dequantize:
  *       pinned by brute force over every code value against exact rational arithmetic rounded
  *       once per operation (fractions + numpy.float16 / bit-level bf16), by s=1,z=0 identity and
@@ -23,8 +25,12 @@
  *       an independent numpy float64 composition within fp32-accumulation error.
  *   layer_norm_min_max_observer, matmul_quant:
  *       the reference holds no such op (only the env-var name ONEFLOW_MLIR_GROUP_MATMUL_QUANT);
- *       semantics are defined by composition of reference rules and pinned by closed forms and an
- *       exact int64 GEMM.  PARITY WITH THE REFERENCE UNPINNED for these two.
+ *       semantics are defined by composition of reference rules.  The LayerNorm half is pinned
+ *       on its rule (layer_norm_gpu_kernel.cu:61-68) bit for bit in fp16 and bf16: rows with
+ *       exactly known mean and variance, expected bits built with numpy / torch casts as
+ *       T(T(T(n) * gamma) + beta), and three plausible wrong rounding orders shown to differ;
+ *       matmul_quant by an exact int64 GEMM.  As fused ops they have no counterpart to compare
+ *       with: PARITY OF THE COMPOSITION WITH THE REFERENCE UNPINNED for these two.
  *   groupwise_quantize, moving_average_min_max_observer:
  *       pinned against an independent numpy restatement of the reference test's quantiser and
  *       closed forms / hand-written fp32 step sequences.
@@ -542,8 +548,12 @@ static int layer_norm_observer_impl(const void* x, const void* bias, const void*
       const float xin = skip_input(x, bias, skip, alpha_t, r, c, cols, t, with_skip);
       const float xn = t_round((xin - mean_f) * inv_f, t);
       float v = xn;
-      if (gamma) v = t_round(v * t_load(gamma, c, t), t);
-      if (beta) v = t_round(v + t_load(beta, c, t), t);
+      /* layer_norm_gpu_kernel.cu:46-59,63-64: with either of gamma / beta present both
+       * operations run, the absent operand being 1 or 0 (so -0 + 0 gives +0) */
+      if (gamma || beta) {
+        v = t_round(v * (gamma ? t_load(gamma, c, t) : 1.0f), t);
+        v = t_round(v + (beta ? t_load(beta, c, t) : 0.0f), t);
+      }
       t_store(y, r * cols + c, v, t);
       const float a = fabsf(t_round(v, t));
       if (a > absmax) absmax = a;

@@ -100,6 +100,32 @@ def test_layer_norm_closed_form():
     assert np.isclose(H.to_numpy(s)[0], expect / 127.0, rtol=3e-7)
 
 
+@pytest.mark.parametrize("t", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("cols", [256, 4096, 8192, 20000])
+def test_layer_norm_exact_statistics_rows_bit_exact(t, cols):
+    """Rows of +-4 (any order) have mean 0, variance 16 and, with eps = 0, inv = 1/4 exactly in
+    every summation order, so only the roundings of the affine are left: the bits must equal the
+    oracle's, for gamma and beta together, gamma alone (the reference then adds its default beta
+    0, which turns a -0 product into +0) and beta alone.  The column counts reach the one-wave,
+    one-block and any-length kernels."""
+    import oneflow_amd as flow
+    rng = np.random.default_rng(cols)
+    base = np.concatenate([np.full(cols // 2, 4.0, np.float32), np.full(cols // 2, -4.0, np.float32)])
+    x = H.as_T(np.stack([rng.permutation(base) for _ in range(5)]), t)
+    gamma_f = (1 + 0.37 * rng.standard_normal(cols)).astype(np.float32)
+    gamma_f[::7] = 0.0
+    gamma = H.as_T(gamma_f, t)
+    beta = H.as_T((0.21 * rng.standard_normal(cols)).astype(np.float32), t)
+    for g, b in ((gamma, beta), (gamma, None), (None, beta), (None, None)):
+        y_ref, s_ref, _ = O.layer_norm_min_max_observer(x, g, b, 0.0, 8)
+        y, s, z = flow._C.fused_layer_norm_min_max_observer(
+            H.to_torch(x), None if g is None else H.to_torch(g), None if b is None else H.to_torch(b), 0.0, 8)
+        y = H.to_numpy(y)
+        view = np.uint32 if t == "f32" else np.uint16
+        assert np.array_equal(y.view(view), y_ref.view(view)), (t, cols, g is None, b is None)
+        assert H.to_numpy(s)[0] == s_ref[0]
+
+
 def test_dynamic_quantize_and_matmul_quant():
     import oneflow_amd as flow
     import torch

@@ -71,6 +71,27 @@ def test_decode_w4a16_llama_shapes(m, n, k, container):
     assert r < (5e-4 if container == np.int8 else 1e-4)
 
 
+@pytest.mark.parametrize("m", [1, 8])
+def test_same_weights_in_both_containers_differ_by_rounding_of_w_only(m):
+    """The same symmetric 4-bit weights stored as int8 codes q and as uint8 codes q + 7: the int8
+    fast path scales the exact group sum (q*scale never rounded to fp16), the uint8 path forms
+    w~ = T(T(u*s) + T(-7s)) as groupwise_dequantize does.  Both are within the contract of the
+    composition; between them the difference is the rounding of w~ alone, bounded here."""
+    n, k = 4096, 4096
+    x, w_i8, scale, b = _decode_inputs(m, n, k, np.int8)
+    codes = H.unpack_int4(w_i8.view(np.uint8)).astype(np.int16)
+    codes = np.where(codes > 7, codes - 16, codes)  # sign-extend the nibbles
+    w_u8 = H.pack_int4((codes + 7).astype(np.uint8))
+    got_i8 = _run(x, w_i8, scale, None, b, 4, True, 1, 128)
+    got_u8 = _run(x, w_u8, scale, None, b, 4, True, 1, 128)
+    ref_i8 = O.fused_linear(x, w_i8, scale, None, b, 4, True, 1, 128)
+    ref_u8 = O.fused_linear(x, w_u8, scale, None, b, 4, True, 1, 128)
+    H.assert_linear_parity(got_i8, ref_i8, "f16", "int8 container")
+    H.assert_linear_parity(got_u8, ref_u8, "f16", "uint8 container")
+    d = H.rel_l2(got_i8.astype(np.float32), got_u8.astype(np.float32))
+    assert 0 < d < 1e-3, d
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 5000, 256), (3, 4099, 384), (16, 6000, 128), (2, 40000, 256),
                                    (5, 33000, 128), (8, 4112, 1024), (16, 688, 256), (12, 100, 128),
                                    (9, 2048, 128)])
