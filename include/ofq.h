@@ -40,7 +40,9 @@ typedef enum {
   OFQ_ERR_UNSUPPORTED = 5,     /* valid for the op, but no kernel covers the combination */
   OFQ_ERR_WORKSPACE = 6,       /* workspace missing or smaller than *_workspace_bytes() */
   OFQ_ERR_MISALIGNED = 7,      /* a pointer is not 16-byte aligned */
-  OFQ_ERR_LAUNCH = 8           /* hipGetLastError() after the launch was not hipSuccess */
+  OFQ_ERR_LAUNCH = 8,          /* hipGetLastError() after the launch was not hipSuccess */
+  OFQ_ERR_TOO_LARGE = 9        /* input beyond the fixed capacity of an entry point that
+                                  allocates nothing and takes no workspace */
 } ofq_status;
 
 /* element types; values follow no OneFlow enum on purpose (the adapter maps DataType) */
@@ -187,6 +189,24 @@ int ofq_fused_layer_norm_min_max_observer(void* stream, const void* x, const voi
                                           float* zero_point, int t_dtype, int64_t rows,
                                           int64_t cols, double epsilon, int quantization_bit,
                                           void* workspace, size_t workspace_bytes);
+
+/*
+ * fused_layer_norm_min_max_observer for callers that cannot allocate device memory.
+ * No counterpart in the reference (there the framework allocates every tmp_buffer before Compute):
+ * it is for code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc.  Same arguments and results (bit for bit) as the entry point above without the
+ * workspace; the per-row partial maxima go to a fixed array in the library's device image
+ * (OFQ_LN_STATIC_MAX_ROWS floats = 256 KB, present on every device the library runs on), whose
+ * address is looked up once per device at the first call made with that device current (make
+ * that first call outside stream capture).  Calls no hipMalloc / hipFree or allocating routine.
+ * rows > 65536 returns OFQ_ERR_TOO_LARGE and launches nothing.  All calls on one device share
+ * the array: calls that overlap on one device (different streams) race; calls on one stream do not.
+ */
+int ofq_fused_layer_norm_min_max_observer_static(void* stream, const void* x, const void* gamma,
+                                                 const void* beta, void* y, float* scale,
+                                                 float* zero_point, int t_dtype, int64_t rows,
+                                                 int64_t cols, double epsilon,
+                                                 int quantization_bit);
 
 /*
  * fused_skip_layer_norm_min_max_observer: the op above on the input of skip_layer_norm,

@@ -39,6 +39,8 @@ SIGNATURES = {
     "ofq_fused_layer_norm_min_max_observer_workspace_bytes": (_sz, [_i, _i64, _i64]),
     "ofq_fused_layer_norm_min_max_observer": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64,
                                                    _i64, ctypes.c_double, _i, _vp, _sz]),
+    "ofq_fused_layer_norm_min_max_observer_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i,
+                                                          _i64, _i64, ctypes.c_double, _i]),
     "ofq_fused_skip_layer_norm_min_max_observer": (_i, [_vp, _vp, _vp, _vp, ctypes.c_double, _vp,
                                                         _vp, _vp, _vp, _vp, _i, _i64, _i64,
                                                         ctypes.c_double, _i, _vp, _sz]),

@@ -16,7 +16,16 @@
 // waves of a CU drift apart, which overlaps one wave's loads with another's stores.  Longer rows
 // use one block per row.  The absmax of the stored values goes to the workspace (one float per
 // wave or per row) and a second one-wave launch folds them and divides.
+#include <atomic>
 #include "ofq_device.h"
+
+// Scratch of the entry point that allocates nothing (ofq_fused_layer_norm_min_max_observer_static):
+// one partial absmax per row or wave, the role the caller's workspace plays in the other entry
+// points.  Every device the library runs on holds its own copy until the process ends.  In host
+// code the name below is only a handle for hipGetSymbolAddress; the device address it yields is
+// what kernels and copies are given.
+#define OFQ_LN_STATIC_MAX_ROWS 65536
+static __device__ __align__(256) float scratch[OFQ_LN_STATIC_MAX_ROWS];
 
 namespace ofq {
 namespace {
@@ -511,8 +520,45 @@ int run(void* stream, const void* x, const void* bias, const void* skip, double 
 #undef OFQ_LN_RUN
 }
 
+// device address of `scratch` on the current device, looked up once per device
+constexpr int kMaxDevices = 64;
+std::atomic<float*> scratch_on_device[kMaxDevices];
+
+int static_scratch(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return OFQ_ERR_LAUNCH;
+  float* p = scratch_on_device[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void* addr = nullptr;
+    if (hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)) != hipSuccess || addr == nullptr) {
+      return OFQ_ERR_LAUNCH;
+    }
+    p = static_cast<float*>(addr);
+    scratch_on_device[dev].store(p, std::memory_order_release);  // same value from any thread
+  }
+  *out = p;
+  return OFQ_OK;
+}
+
 }  // namespace
 }  // namespace ofq
+
+extern "C" int ofq_fused_layer_norm_min_max_observer_static(void* stream, const void* x,
+                                                            const void* gamma, const void* beta,
+                                                            void* y, float* scale,
+                                                            float* zero_point, int t_dtype,
+                                                            int64_t rows, int64_t cols,
+                                                            double epsilon, int quantization_bit) {
+  if (rows > OFQ_LN_STATIC_MAX_ROWS) return OFQ_ERR_TOO_LARGE;
+  float* ws = nullptr;
+  const int st = ofq::static_scratch(&ws);
+  if (st != OFQ_OK) return st;
+  // every partial the finalize kernel reads is written by the row kernel of the same call, so
+  // nothing has to be cleared between calls
+  return ofq::run(stream, x, nullptr, nullptr, 0.0, false, gamma, beta, y, scale, zero_point,
+                  t_dtype, rows, cols, epsilon, quantization_bit, ws,
+                  (size_t)OFQ_LN_STATIC_MAX_ROWS * sizeof(float));
+}
 
 extern "C" size_t ofq_fused_layer_norm_min_max_observer_workspace_bytes(int, int64_t rows,
                                                                         int64_t) {

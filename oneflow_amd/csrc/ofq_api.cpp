@@ -12,6 +12,7 @@ extern "C" const char* ofq_status_string(int status) {
     case OFQ_ERR_WORKSPACE: return "workspace missing or too small";
     case OFQ_ERR_MISALIGNED: return "pointer not 16-byte aligned";
     case OFQ_ERR_LAUNCH: return "kernel launch failed";
+    case OFQ_ERR_TOO_LARGE: return "input exceeds the fixed scratch capacity of this entry point";
     default: return "unknown status";
   }
 }
