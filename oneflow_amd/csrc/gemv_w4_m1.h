@@ -1,0 +1,211 @@
+// Decode kernel for ONE row of x (m = 1) of fused_linear_with_groupwise_quantized_weight:
+// fp16, 4-bit symmetric codes in an int8 container, groups along K with 128 | group_size (a power
+// of two times 128), K a multiple of 256.
+//
+// A decode linear on this chip is a one-shot kernel that ends one HBM round trip after it
+// started, so what counts is what stands in front of the first request and behind the last byte.
+// Measured on 4096 x 4096 (launch to launch, weights cold): the weights alone, requested 1 KB
+// per instruction, take 2.7 us; requested as an MFMA operand layout wants them (adjacent lanes in
+// different rows) 3.1 us; and the MFMA kernel 4.1 us, of which the cross-wave fold behind a
+// barrier is 0.56 us, the per-lane scale gathers 0.2 us and the arithmetic itself next to
+// nothing.  For one row of x the matrix core has nothing to offer either: 15 of its 16 rows are
+// idle, and a packed dot product (v_dot2_f32_f16) reaches the same 32 useful MACs per clock.
+//
+// So here a WAVE owns whole weight rows:
+//   - a lane reads 16 contiguous bytes, a wave-level request is 1 KB of one row: the cheapest
+//     pattern for the address pipe and for DRAM;
+//   - the k-reduction is 16 dot2 per 16 bytes of codes in the lane plus one cross-lane sum per row
+//     (DPP), so there is no LDS fold, no second barrier, and a wave stores its row's output the
+//     moment its own data has arrived;
+//   - the scales of a row are 2 bytes per lane out of one or two cache lines, requested behind
+//     the weights;
+//   - x is permuted into the order the nibble masks deliver the codes ONCE per block, into LDS,
+//     laid out lane-major, and every wave copies it to registers while the weights are in
+//     flight.
+// Arithmetic as in gemv_kernels.h: 0x6400|nibble is the half 1032+q (low nibbles) or 1152+16q
+// (high nibbles, met by x/16); the constant part per lane, 1032*sum_lo(x) + 72*sum_hi(x), is
+// computed at staging and seeds the accumulator negated; products are exact in fp32, the group
+// scale multiplies the lane's fp32 sum (w~ = q*s is not rounded to fp16).
+#pragma once
+
+#include "gemv_kernels.h"
+
+namespace ofq {
+namespace {
+
+struct M1Shape {
+  int N, K;
+  int rows_per_block;
+  int gshift;  // log2(group_size)
+  int G;       // groups per row
+};
+
+// LDS: [x operands H x 4 pieces x 64 lanes x 16 B] [corr H x 64 f32]
+inline size_t gemv_m1_lds_bytes(int H) { return (size_t)H * 4096 + (size_t)H * 256; }
+
+template<int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// sum over the 64 lanes, the same value in every lane's view of lanes 0, 16, 32, 48
+__device__ __forceinline__ float wave_sum_m1(float v) {
+  v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f32<0x141>(v);  // row_half_mirror
+  v += dpp_f32<0x140>(v);  // row_mirror: every lane of a row of 16 holds the row's sum
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  return (a + b) + (c + d);
+}
+
+// 16 bytes of codes (32 k) against the lane's x operands: xa[0]/xa[1] = low/high nibbles of words
+// 0,1, xa[2]/xa[3] = of words 2,3 (the layout permute_unit writes)
+__device__ __forceinline__ float m1_dot32(const u32x4 wq, const u32x4 (&xa)[4], float acc) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint32_t w0 = wq[2 * h];
+    const uint32_t w1 = wq[2 * h + 1];
+    const uint32_t w0s = w0 >> 8, w1s = w1 >> 8;
+    uint32_t blo[4], bhi[4];
+    blo[0] = (w0 & 0x000F000Fu) ^ 0x64086408u;
+    blo[1] = (w0s & 0x000F000Fu) ^ 0x64086408u;
+    blo[2] = (w1 & 0x000F000Fu) ^ 0x64086408u;
+    blo[3] = (w1s & 0x000F000Fu) ^ 0x64086408u;
+    bhi[0] = (w0 & 0x00F000F0u) ^ 0x64806480u;
+    bhi[1] = (w0s & 0x00F000F0u) ^ 0x64806480u;
+    bhi[2] = (w1 & 0x00F000F0u) ^ 0x64806480u;
+    bhi[3] = (w1s & 0x00F000F0u) ^ 0x64806480u;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc = __builtin_amdgcn_fdot2(as_h2(blo[e]), as_h2(xa[2 * h][e]), acc, false);
+      acc = __builtin_amdgcn_fdot2(as_h2(bhi[e]), as_h2(xa[2 * h + 1][e]), acc, false);
+    }
+  }
+  return acc;
+}
+
+// NW waves per block; RPW rows per wave (rows wave, wave + NW, ..); H = KB of codes per row,
+// rounded up (a lane owns bytes [h*1024 + lane*16, +16) of a row for h < H).
+template<int NW, int RPW, int H, int XU = 1>
+__global__ void __launch_bounds__(NW * 64)
+gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+           const f16* __restrict__ scale, const f16* __restrict__ bias, f16* __restrict__ out,
+           M1Shape sh) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int K = sh.K;
+  const int row_bytes = K >> 1;
+  asm volatile("" ::"s"(out));  // fetch the output pointer with the other arguments
+  const int row0 = blockIdx.x * sh.rows_per_block;
+  int rows_blk = sh.N - row0;
+  if (rows_blk > sh.rows_per_block) rows_blk = sh.rows_per_block;
+
+  // ---- requests: x (feeds LDS, so it goes first), bias, weights, scales -----------------------
+  constexpr int NTH = NW * 64;
+  const int nunits = K >> 4;  // 32-byte units of x; XU per thread (K <= 16 * XU * NW * 64)
+  const bool stage_wave = wave * 64 < nunits;  // wave-uniform
+  u32x4 xu[XU][2];
+  if (stage_wave) {
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+      int u = tid + i * NTH;
+      u = u < nunits ? u : nunits - 1;
+      const u32x4* src = reinterpret_cast<const u32x4*>(x) + (size_t)u * 2;
+      xu[i][0] = src[0];
+      xu[i][1] = src[1];
+    }
+  }
+  uint16_t bias_raw[RPW];
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) bias_raw[i] = 0;
+  if (bias != nullptr) {
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+      const int row_l = wave + i * NW;
+      bias_raw[i] = reinterpret_cast<const uint16_t*>(bias)[row0 + (row_l < rows_blk ? row_l : 0)];
+    }
+  }
+  const uint8_t* wblk = w + (int64_t)row0 * row_bytes;
+  u32x4 wq[RPW][H];
+  bool valid[H];
+#pragma unroll
+  for (int h = 0; h < H; ++h) valid[h] = h * 1024 + lane * 16 < row_bytes;
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) {
+    const int row_l = wave + i * NW;
+    const uint8_t* rowp = wblk + (size_t)(row_l < rows_blk ? row_l : 0) * row_bytes;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const uint32_t off = valid[h] ? (uint32_t)(h * 1024 + lane * 16) : 0u;
+      wq[i][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rowp + off));
+    }
+  }
+  const f16* sblk = scale + (int64_t)row0 * sh.G;
+  f16 sc[RPW][H];
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) {
+    const int row_l = wave + i * NW;
+    const f16* srow = sblk + (size_t)(row_l < rows_blk ? row_l : 0) * sh.G;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const int g = valid[h] ? (h * 2048 + lane * 32) >> sh.gshift : 0;
+      sc[i][h] = srow[g];
+    }
+  }
+
+  // ---- x -> LDS: piece t of lane l of KB h at ((h*4 + t)*64 + l)*16 ---------------------------
+  float* corr_l = reinterpret_cast<float*>(smem + (size_t)H * 4096);
+#pragma unroll
+  for (int i = 0; i < XU; ++i) {
+    if (wave * 64 + i * NTH >= nunits) break;  // wave-uniform
+    const int u = tid + i * NTH;
+    const bool ok = u < nunits;
+    u32x4 lo, hi;
+    permute_unit(xu[i][0], xu[i][1], lo, hi);
+    const int h = u >> 7, l = (u >> 1) & 63, p = u & 1;
+    if (ok) {
+      *reinterpret_cast<u32x4*>(smem + (size_t)(((h * 4 + 2 * p) * 64 + l) * 16)) = lo;
+      *reinterpret_cast<u32x4*>(smem + (size_t)(((h * 4 + 2 * p + 1) * 64 + l) * 16)) = hi;
+    }
+    float cpart = ok ? unit_corr(lo, hi) : 0.f;
+    cpart += __shfl_xor(cpart, 1, 64);
+    if (ok && p == 0) corr_l[h * 64 + l] = -cpart;
+  }
+  __syncthreads();
+
+  // ---- per KB of the row: operands from LDS, then the rows of the wave -------------------------
+  float tot[RPW];
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) tot[i] = 0.f;
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    u32x4 xa[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      xa[t] = *reinterpret_cast<const u32x4*>(smem + (size_t)(((h * 4 + t) * 64 + lane) * 16));
+    }
+    const float cr = corr_l[h * 64 + lane];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+      const float acc = m1_dot32(wq[i][h], xa, cr);
+      const float term = acc * (float)sc[i][h];
+      tot[i] += valid[h] ? term : 0.f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) {
+    const int row_l = wave + i * NW;
+    const float sum = wave_sum_m1(tot[i]);
+    if (lane == 0 && row_l < rows_blk) {
+      out[row0 + row_l] = (f16)(sum + (float)bias_at_end(bias_raw[i]));
+    }
+  }
+}
+
+}  // namespace
+}  // namespace ofq

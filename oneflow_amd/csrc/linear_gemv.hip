@@ -679,6 +679,10 @@ bool gemv_wq_supported(const LinearArgs& a) {
 }
 
 int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
+  if (gemv_m1_supported(a)) {
+    const int rc = launch_gemv_m1(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   if (w4s_supported(a)) {
     const int rc = launch_w4s(st, a);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;

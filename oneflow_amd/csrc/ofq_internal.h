@@ -31,6 +31,11 @@ bool gemm_wq_supported(const LinearArgs& a);
 size_t gemm_wq_workspace_bytes(const LinearArgs& a);
 int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t workspace_bytes);
 
+// m = 1, fp16, 4-bit symmetric codes in an int8 container, groups along K: a wave owns whole
+// weight rows (contiguous requests, packed dot products, no cross-wave fold).
+bool gemv_m1_supported(const LinearArgs& a);
+int launch_gemv_m1(hipStream_t st, const LinearArgs& a);
+
 // Skinny-M (m <= 16) MFMA GEMV that streams the weights once.
 bool gemv_wq_supported(const LinearArgs& a);
 int launch_gemv_wq(hipStream_t st, const LinearArgs& a);

@@ -71,6 +71,28 @@ def test_decode_w4a16_llama_shapes(m, n, k, container):
     assert r < (5e-4 if container == np.int8 else 1e-4)
 
 
+@pytest.mark.parametrize("n,k,g,with_bias", [
+    (4096, 256, 128, True), (37, 512, 128, False), (4099, 2048, 256, True), (1000, 3072, 128, True),
+    (513, 4096, 512, True), (300, 5120, 128, False), (2048, 8192, 1024, True), (129, 9216, 128, True),
+    (64, 11008, 128, True), (77, 13824, 128, True), (50, 14336, 256, False), (33, 16384, 128, True),
+    (128256, 256, 128, True),
+])
+def test_decode_m1_row_per_wave_shapes(n, k, g, with_bias):
+    """m = 1, fp16, symmetric int4 in an int8 container: the kernel in which a wave owns whole
+    rows.  Every row length class (1 .. 8 KB of codes per row, with a partial last KB), group
+    sizes above 128, row counts off the block size, no bias."""
+    rng = np.random.default_rng(n * 31 + k)
+    x = H.as_T(rng.standard_normal((1, k)).astype(np.float32), "f16")
+    codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    w = H.pack_int4(codes)
+    scale = H.as_T(rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float32), "f16")
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), "f16") if with_bias else None
+    ref = O.fused_linear(x, w, scale, None, b, 4, True, 1, g)
+    got = _run(x, w, scale, None, b, 4, True, 1, g)
+    r, e = H.assert_linear_parity(got, ref, "f16", f"n={n} k={k} g={g}")
+    assert r < 5e-4
+
+
 @pytest.mark.parametrize("m", [1, 8])
 def test_same_weights_in_both_containers_differ_by_rounding_of_w_only(m):
     """The same symmetric 4-bit weights stored as int8 codes q and as uint8 codes q + 7: the int8
