@@ -87,26 +87,38 @@ __device__ __forceinline__ float m1_dot32(const u32x4 wq, const u32x4 (&xa)[4], 
   return acc;
 }
 
+// The gate of a fused GLU: the same rows of a second weight of equal shape, owned by the same
+// wave, which then forms y = T(hidden * T(act(gate))) itself
+// (oneflow/user/kernels/fused_glu_kernel.cu:303-347); both linears are stored as well.
+struct M1Glu {
+  const uint8_t* w2;
+  const f16* scale2;
+  const f16* bias2;
+  f16* out2;
+  f16* y;
+  int act;
+};
+
 // NW waves per block; RPW rows per wave (rows wave, wave + NW, ..); H = KB of codes per row,
-// rounded up (a lane owns bytes [h*1024 + lane*16, +16) of a row for h < H).
-template<int NW, int RPW, int H, int XU = 1>
-__global__ void __launch_bounds__(NW * 64)
-gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,
-           const f16* __restrict__ scale, const f16* __restrict__ bias, f16* __restrict__ out,
-           M1Shape sh) {
+// rounded up (a lane owns bytes [h*1024 + lane*16, +16) of a row for h < H); XU units of x per
+// thread at staging; NM = 1, or 2 for the GLU (hidden and gate).
+template<int NW, int RPW, int H, int XU, int NM>
+__device__ __forceinline__ void
+m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
+        const f16* __restrict__ scale, const f16* __restrict__ bias, f16* __restrict__ out, int N,
+        const M1Shape& sh, const M1Glu& glu) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NTH = NW * 64;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = sh.K;
   const int row_bytes = K >> 1;
-  asm volatile("" ::"s"(out));  // fetch the output pointer with the other arguments
-  const int row0 = blockIdx.x * sh.rows_per_block;
-  int rows_blk = sh.N - row0;
+  const int row0 = block * sh.rows_per_block;
+  int rows_blk = N - row0;
   if (rows_blk > sh.rows_per_block) rows_blk = sh.rows_per_block;
 
   // ---- requests: x (feeds LDS, so it goes first), bias, weights, scales -----------------------
-  constexpr int NTH = NW * 64;
   const int nunits = K >> 4;  // 32-byte units of x; XU per thread (K <= 16 * XU * NW * 64)
   const bool stage_wave = wave * 64 < nunits;  // wave-uniform
   u32x4 xu[XU][2];
@@ -120,41 +132,50 @@ gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,
       xu[i][1] = src[1];
     }
   }
-  uint16_t bias_raw[RPW];
+  uint16_t bias_raw[NM][RPW];
 #pragma unroll
-  for (int i = 0; i < RPW; ++i) bias_raw[i] = 0;
-  if (bias != nullptr) {
+  for (int q = 0; q < NM; ++q) {
+    const f16* bq = q == 0 ? bias : glu.bias2;
 #pragma unroll
     for (int i = 0; i < RPW; ++i) {
+      bias_raw[q][i] = 0;
       const int row_l = wave + i * NW;
-      bias_raw[i] = reinterpret_cast<const uint16_t*>(bias)[row0 + (row_l < rows_blk ? row_l : 0)];
+      if (bq != nullptr) {
+        bias_raw[q][i] = reinterpret_cast<const uint16_t*>(bq)[row0 + (row_l < rows_blk ? row_l : 0)];
+      }
     }
   }
-  const uint8_t* wblk = w + (int64_t)row0 * row_bytes;
-  u32x4 wq[RPW][H];
+  u32x4 wq[NM][RPW][H];
   bool valid[H];
 #pragma unroll
   for (int h = 0; h < H; ++h) valid[h] = h * 1024 + lane * 16 < row_bytes;
 #pragma unroll
-  for (int i = 0; i < RPW; ++i) {
-    const int row_l = wave + i * NW;
-    const uint8_t* rowp = wblk + (size_t)(row_l < rows_blk ? row_l : 0) * row_bytes;
+  for (int q = 0; q < NM; ++q) {
+    const uint8_t* wblk = (q == 0 ? w : glu.w2) + (int64_t)row0 * row_bytes;
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
-      const uint32_t off = valid[h] ? (uint32_t)(h * 1024 + lane * 16) : 0u;
-      wq[i][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rowp + off));
+    for (int i = 0; i < RPW; ++i) {
+      const int row_l = wave + i * NW;
+      const uint8_t* rowp = wblk + (size_t)(row_l < rows_blk ? row_l : 0) * row_bytes;
+#pragma unroll
+      for (int h = 0; h < H; ++h) {
+        const uint32_t off = valid[h] ? (uint32_t)(h * 1024 + lane * 16) : 0u;
+        wq[q][i][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rowp + off));
+      }
     }
   }
-  const f16* sblk = scale + (int64_t)row0 * sh.G;
-  f16 sc[RPW][H];
+  f16 sc[NM][RPW][H];
 #pragma unroll
-  for (int i = 0; i < RPW; ++i) {
-    const int row_l = wave + i * NW;
-    const f16* srow = sblk + (size_t)(row_l < rows_blk ? row_l : 0) * sh.G;
+  for (int q = 0; q < NM; ++q) {
+    const f16* sblk = (q == 0 ? scale : glu.scale2) + (int64_t)row0 * sh.G;
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
-      const int g = valid[h] ? (h * 2048 + lane * 32) >> sh.gshift : 0;
-      sc[i][h] = srow[g];
+    for (int i = 0; i < RPW; ++i) {
+      const int row_l = wave + i * NW;
+      const f16* srow = sblk + (size_t)(row_l < rows_blk ? row_l : 0) * sh.G;
+#pragma unroll
+      for (int h = 0; h < H; ++h) {
+        const int g = valid[h] ? (h * 2048 + lane * 32) >> sh.gshift : 0;
+        sc[q][i][h] = srow[g];
+      }
     }
   }
 
@@ -179,9 +200,12 @@ gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   __syncthreads();
 
   // ---- per KB of the row: operands from LDS, then the rows of the wave -------------------------
-  float tot[RPW];
+  float tot[NM][RPW];
 #pragma unroll
-  for (int i = 0; i < RPW; ++i) tot[i] = 0.f;
+  for (int q = 0; q < NM; ++q) {
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) tot[q][i] = 0.f;
+  }
 #pragma unroll
   for (int h = 0; h < H; ++h) {
     u32x4 xa[4];
@@ -191,20 +215,62 @@ gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,
     }
     const float cr = corr_l[h * 64 + lane];
 #pragma unroll
-    for (int i = 0; i < RPW; ++i) {
-      const float acc = m1_dot32(wq[i][h], xa, cr);
-      const float term = acc * (float)sc[i][h];
-      tot[i] += valid[h] ? term : 0.f;
+    for (int q = 0; q < NM; ++q) {
+#pragma unroll
+      for (int i = 0; i < RPW; ++i) {
+        const float acc = m1_dot32(wq[q][i][h], xa, cr);
+        const float term = acc * (float)sc[q][i][h];
+        tot[q][i] += valid[h] ? term : 0.f;
+      }
     }
   }
 #pragma unroll
   for (int i = 0; i < RPW; ++i) {
     const int row_l = wave + i * NW;
-    const float sum = wave_sum_m1(tot[i]);
-    if (lane == 0 && row_l < rows_blk) {
-      out[row0 + row_l] = (f16)(sum + (float)bias_at_end(bias_raw[i]));
+    const float sum = wave_sum_m1(tot[0][i]);
+    if (NM == 1) {
+      if (lane == 0 && row_l < rows_blk) {
+        out[row0 + row_l] = (f16)(sum + (float)bias_at_end(bias_raw[0][i]));
+      }
+    } else {
+      const float sum2 = wave_sum_m1(tot[NM - 1][i]);
+      if (lane == 0 && row_l < rows_blk) {
+        const f16 hidden = (f16)(sum + (float)bias_at_end(bias_raw[0][i]));
+        const f16 gate = (f16)(sum2 + (float)bias_at_end(bias_raw[NM - 1][i]));
+        out[row0 + row_l] = hidden;
+        glu.out2[row0 + row_l] = gate;
+        glu.y[row0 + row_l] = hidden * (f16)glu_activation((float)gate, glu.act);
+      }
     }
   }
+}
+
+template<int NW, int RPW, int H, int XU = 1>
+__global__ void __launch_bounds__(NW * 64)
+gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+           const f16* __restrict__ scale, const f16* __restrict__ bias, f16* __restrict__ out,
+           M1Shape sh) {
+  asm volatile("" ::"s"(out));  // fetch the output pointer with the other arguments
+  m1_body<NW, RPW, H, XU, 1>(blockIdx.x, x, w, scale, bias, out, sh.N, sh, M1Glu());
+}
+
+// hidden = x w~^T + b, gate = x v~^T + c, y = hidden * act(gate): one launch, one wave per row pair
+template<int NW, int H, int XU = 1>
+__global__ void __launch_bounds__(NW * 64)
+gemv_w4_m1_glu(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+               const f16* __restrict__ scale, const f16* __restrict__ bias,
+               f16* __restrict__ out, M1Glu glu, M1Shape sh) {
+  m1_body<NW, 1, H, XU, 2>(blockIdx.x, x, w, scale, bias, out, sh.N, sh, glu);
+}
+
+// several problems of equal k in one launch: the grid is the concatenation of the problems'
+// blocks, a block finds its problem in the table
+template<int NW, int H, int XU = 1>
+__global__ void __launch_bounds__(NW * 64) gemv_w4_m1_grouped(GemvGroup g, M1Shape sh) {
+  const GemvProblem pr = select_problem(g, (int)blockIdx.x);
+  m1_body<NW, 1, H, XU, 1>((int)blockIdx.x - pr.first_block, static_cast<const f16*>(pr.x), pr.w,
+                           static_cast<const f16*>(pr.scale), static_cast<const f16*>(pr.bias),
+                           static_cast<f16*>(pr.out), pr.N, sh, M1Glu());
 }
 
 }  // namespace

@@ -564,6 +564,10 @@ int launch_w4p_glu_inst(hipStream_t st, const LinearArgs& a, const GluArgs& glu,
 }  // namespace
 
 int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act) {
+  {
+    const int rc = launch_gemv_m1_glu(st, a, g, y, act);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   if (!w4p_supported(a) || !w4p_supported(g)) return OFQ_ERR_UNSUPPORTED;
   if (g.n != a.n || g.k != a.k || g.m != a.m || g.x != a.x) return OFQ_ERR_UNSUPPORTED;
   constexpr int kCUs = 256;
@@ -606,6 +610,10 @@ int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, vo
 
 int launch_gemv_grouped(hipStream_t st, const LinearArgs* pr, int count) {
   if (count < 1 || count > kGemvMaxProblems) return OFQ_ERR_UNSUPPORTED;
+  {
+    const int rc = launch_gemv_m1_grouped(st, pr, count);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   const LinearArgs& a = pr[0];
   bool all_w4p = true;
   for (int i = 0; i < count; ++i) {

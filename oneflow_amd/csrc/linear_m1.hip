@@ -30,6 +30,67 @@ int launch_m1_inst(hipStream_t st, const LinearArgs& a) {
   return ofq_check_launch();
 }
 
+template<int NW, int H, int XU>
+int launch_m1_glu_inst(hipStream_t st, const LinearArgs& a, const M1Glu& glu) {
+  M1Shape sh;
+  sh.N = (int)a.n;
+  sh.K = (int)a.k;
+  sh.rows_per_block = NW;
+  sh.gshift = log2_exact(a.group_size);
+  sh.G = (int)(a.k / a.group_size);
+  const int grid = (int)((a.n + NW - 1) / NW);
+  gemv_w4_m1_glu<NW, H, XU><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
+      static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
+      static_cast<const f16*>(a.scale), static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
+      glu, sh);
+  return ofq_check_launch();
+}
+
+template<int NW, int H, int XU>
+int launch_m1_grouped_inst(hipStream_t st, const LinearArgs* pr, int count) {
+  GemvGroup g{};
+  g.count = count;
+  int first = 0;
+  for (int i = 0; i < count; ++i) {
+    g.p[i].x = pr[i].x;
+    g.p[i].w = static_cast<const uint8_t*>(pr[i].w);
+    g.p[i].scale = pr[i].scale;
+    g.p[i].zero = nullptr;
+    g.p[i].bias = pr[i].bias;
+    g.p[i].out = pr[i].out;
+    g.p[i].N = (int)pr[i].n;
+    g.p[i].first_block = first;
+    first += (int)((pr[i].n + NW - 1) / NW);
+  }
+  M1Shape sh;
+  sh.N = 0;  // per problem
+  sh.K = (int)pr[0].k;
+  sh.rows_per_block = NW;
+  sh.gshift = log2_exact(pr[0].group_size);
+  sh.G = (int)(pr[0].k / pr[0].group_size);
+  gemv_w4_m1_grouped<NW, H, XU><<<first, NW * 64, gemv_m1_lds_bytes(H), st>>>(g, sh);
+  return ofq_check_launch();
+}
+
+// picks the instance for k: NW = 16 up to 2 KB of codes per row, 8 beyond
+#define OFQ_M1_DISPATCH(k, CALL)                      \
+  do {                                                \
+    const int h_ = (int)(((k) / 2 + 1023) / 1024);    \
+    if ((k) <= 4096) {                                \
+      if (h_ == 1) return CALL(16, 1, 1);             \
+      return CALL(16, 2, 1);                          \
+    }                                                 \
+    switch (h_) {                                     \
+      case 3: return CALL(8, 3, 1);                   \
+      case 4: return CALL(8, 4, 1);                   \
+      case 5: return CALL(8, 5, 2);                   \
+      case 6: return CALL(8, 6, 2);                   \
+      case 7: return CALL(8, 7, 2);                   \
+      case 8: return CALL(8, 8, 2);                   \
+      default: return OFQ_ERR_UNSUPPORTED;            \
+    }                                                 \
+  } while (0)
+
 }  // namespace
 
 bool gemv_m1_supported(const LinearArgs& a) {
@@ -44,22 +105,43 @@ bool gemv_m1_supported(const LinearArgs& a) {
 // (4096 x 11008: 6.3 against 6.7 us), with short rows the second staging of x costs more than
 // that gains (4096 x 4096: 3.55 against 3.8 us).
 int launch_gemv_m1(hipStream_t st, const LinearArgs& a) {
-  const int h = (int)((a.k / 2 + 1023) / 1024);
-  if (a.k <= 4096) {
-    switch (h) {
-      case 1: return launch_m1_inst<16, 1, 1>(st, a);
-      default: return launch_m1_inst<16, 2, 1>(st, a);
+#define OFQ_M1_PLAIN(NW, H, XU) launch_m1_inst<NW, H, XU>(st, a)
+  OFQ_M1_DISPATCH(a.k, OFQ_M1_PLAIN);
+#undef OFQ_M1_PLAIN
+}
+
+// Two weights of equal shape on one x (hidden, gate) + the gating, one launch.
+int launch_gemv_m1_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act) {
+  if (!gemv_m1_supported(a) || !gemv_m1_supported(g)) return OFQ_ERR_UNSUPPORTED;
+  if (g.n != a.n || g.k != a.k || g.x != a.x || g.group_size != a.group_size) {
+    return OFQ_ERR_UNSUPPORTED;
+  }
+  M1Glu glu;
+  glu.w2 = static_cast<const uint8_t*>(g.w);
+  glu.scale2 = static_cast<const f16*>(g.scale);
+  glu.bias2 = static_cast<const f16*>(g.bias);
+  glu.out2 = static_cast<f16*>(g.out);
+  glu.y = static_cast<f16*>(y);
+  glu.act = act;
+#define OFQ_M1_GLU(NW, H, XU) launch_m1_glu_inst<NW, H, XU>(st, a, glu)
+  OFQ_M1_DISPATCH(a.k, OFQ_M1_GLU);
+#undef OFQ_M1_GLU
+}
+
+// Up to kGemvMaxProblems problems of equal k and group size, one launch.
+int launch_gemv_m1_grouped(hipStream_t st, const LinearArgs* pr, int count) {
+  if (count < 1 || count > kGemvMaxProblems) return OFQ_ERR_UNSUPPORTED;
+  int64_t blocks = 0;
+  for (int i = 0; i < count; ++i) {
+    if (!gemv_m1_supported(pr[i]) || pr[i].k != pr[0].k || pr[i].group_size != pr[0].group_size) {
+      return OFQ_ERR_UNSUPPORTED;
     }
+    blocks += (pr[i].n + 7) / 8;
   }
-  switch (h) {
-    case 3: return launch_m1_inst<8, 3, 1>(st, a);
-    case 4: return launch_m1_inst<8, 4, 1>(st, a);
-    case 5: return launch_m1_inst<8, 5, 2>(st, a);
-    case 6: return launch_m1_inst<8, 6, 2>(st, a);
-    case 7: return launch_m1_inst<8, 7, 2>(st, a);
-    case 8: return launch_m1_inst<8, 8, 2>(st, a);
-    default: return OFQ_ERR_UNSUPPORTED;
-  }
+  if (blocks > 0x7FFFFFFF) return OFQ_ERR_UNSUPPORTED;
+#define OFQ_M1_GROUPED(NW, H, XU) launch_m1_grouped_inst<NW, H, XU>(st, pr, count)
+  OFQ_M1_DISPATCH(pr[0].k, OFQ_M1_GROUPED);
+#undef OFQ_M1_GROUPED
 }
 
 }  // namespace ofq

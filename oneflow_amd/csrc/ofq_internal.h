@@ -35,6 +35,8 @@ int launch_gemm_wq(hipStream_t st, const LinearArgs& a, void* workspace, size_t 
 // weight rows (contiguous requests, packed dot products, no cross-wave fold).
 bool gemv_m1_supported(const LinearArgs& a);
 int launch_gemv_m1(hipStream_t st, const LinearArgs& a);
+int launch_gemv_m1_grouped(hipStream_t st, const LinearArgs* problems, int count);
+int launch_gemv_m1_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act);
 
 // Skinny-M (m <= 16) MFMA GEMV that streams the weights once.
 bool gemv_wq_supported(const LinearArgs& a);
