@@ -245,6 +245,134 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
   }
 }
 
+// The same for MANY rows per wave (n beyond what one resident round of one-row waves covers): a
+// block owns rows_per_block consecutive rows, its wave w the rows w, w + NW, ..; x is staged once
+// per block; the requests of a row go out two rows ahead of its arithmetic, so that a wave always
+// has two rows (2 x H KB) in flight and the CU streams without the round trip a new block pays.
+// Every request is unconditional so that the wait counts stay exact: a slot past the wave's last
+// row reads one and the same 16 bytes in every lane (a single cached request).
+template<int NW, int H, int XU>
+__global__ void __launch_bounds__(NW * 64)
+gemv_w4_m1_stream(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+                  const f16* __restrict__ scale, const f16* __restrict__ bias,
+                  f16* __restrict__ out, M1Shape sh) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NTH = NW * 64;
+  constexpr bool kXInRegs = H <= 2;  // x operands stay in registers across rows
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int K = sh.K;
+  const int row_bytes = K >> 1;
+  asm volatile("" ::"s"(out));
+  const int row0 = blockIdx.x * sh.rows_per_block;
+  int rows_blk = sh.N - row0;
+  if (rows_blk > sh.rows_per_block) rows_blk = sh.rows_per_block;
+  const int nr = rows_blk > wave ? (rows_blk - wave + NW - 1) / NW : 0;  // rows of this wave
+
+  const int nunits = K >> 4;
+  const bool stage_wave = wave * 64 < nunits;  // wave-uniform
+  u32x4 xu[XU][2];
+  if (stage_wave) {
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+      int u = tid + i * NTH;
+      u = u < nunits ? u : nunits - 1;
+      const u32x4* src = reinterpret_cast<const u32x4*>(x) + (size_t)u * 2;
+      xu[i][0] = src[0];
+      xu[i][1] = src[1];
+    }
+  }
+  const uint8_t* wblk = w + (int64_t)row0 * row_bytes;
+  const f16* sblk = scale + (int64_t)row0 * sh.G;
+  bool valid[H];
+  uint32_t voff[H];
+  int goff[H];
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    valid[h] = h * 1024 + lane * 16 < row_bytes;
+    voff[h] = valid[h] ? (uint32_t)(h * 1024 + lane * 16) : 0u;
+    goff[h] = valid[h] ? (h * 2048 + lane * 32) >> sh.gshift : 0;
+  }
+  u32x4 wq[2][H];
+  f16 sc[2][H];
+  uint16_t braw[2];
+  auto issue = [&](int i, int buf) {
+    const bool live = i < nr;  // wave-uniform
+    const int row_l = live ? wave + i * NW : 0;
+    const uint8_t* rowp = wblk + (size_t)row_l * row_bytes;
+    const f16* srow = sblk + (size_t)row_l * sh.G;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      wq[buf][h] = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4*>(rowp + (live ? voff[h] : 0u)));
+    }
+#pragma unroll
+    for (int h = 0; h < H; ++h) sc[buf][h] = srow[live ? goff[h] : 0];
+    braw[buf] = bias != nullptr ? reinterpret_cast<const uint16_t*>(bias)[row0 + row_l] : (uint16_t)0;
+  };
+  issue(0, 0);
+  issue(1, 1);
+
+  float* corr_l = reinterpret_cast<float*>(smem + (size_t)H * 4096);
+#pragma unroll
+  for (int i = 0; i < XU; ++i) {
+    if (wave * 64 + i * NTH >= nunits) break;  // wave-uniform
+    const int u = tid + i * NTH;
+    const bool ok = u < nunits;
+    u32x4 lo, hi;
+    permute_unit(xu[i][0], xu[i][1], lo, hi);
+    const int h = u >> 7, l = (u >> 1) & 63, p = u & 1;
+    if (ok) {
+      *reinterpret_cast<u32x4*>(smem + (size_t)(((h * 4 + 2 * p) * 64 + l) * 16)) = lo;
+      *reinterpret_cast<u32x4*>(smem + (size_t)(((h * 4 + 2 * p + 1) * 64 + l) * 16)) = hi;
+    }
+    float cpart = ok ? unit_corr(lo, hi) : 0.f;
+    cpart += __shfl_xor(cpart, 1, 64);
+    if (ok && p == 0) corr_l[h * 64 + l] = -cpart;
+  }
+  __syncthreads();
+
+  u32x4 xr[kXInRegs ? H : 1][4];
+  float crr[kXInRegs ? H : 1];
+  if (kXInRegs) {
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        xr[h][t] = *reinterpret_cast<const u32x4*>(smem + (size_t)(((h * 4 + t) * 64 + lane) * 16));
+      }
+      crr[h] = corr_l[h * 64 + lane];
+    }
+  }
+  auto finish = [&](int i, int buf) {
+    float tot = 0.f;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      float term;
+      if (kXInRegs) {
+        term = m1_dot32(wq[buf][h], xr[h], crr[h]) * (float)sc[buf][h];
+      } else {
+        u32x4 xa[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          xa[t] = *reinterpret_cast<const u32x4*>(smem + (size_t)(((h * 4 + t) * 64 + lane) * 16));
+        }
+        term = m1_dot32(wq[buf][h], xa, corr_l[h * 64 + lane]) * (float)sc[buf][h];
+      }
+      tot += valid[h] ? term : 0.f;
+    }
+    const float sum = wave_sum_m1(tot);
+    if (lane == 0) out[row0 + wave + i * NW] = (f16)(sum + (float)bias_at_end(braw[buf]));
+  };
+  for (int i = 0; i < nr; i += 2) {
+    finish(i, 0);
+    issue(i + 2, 0);
+    if (i + 1 < nr) finish(i + 1, 1);
+    issue(i + 3, 1);
+  }
+}
+
 template<int NW, int RPW, int H, int XU = 1>
 __global__ void __launch_bounds__(NW * 64)
 gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,

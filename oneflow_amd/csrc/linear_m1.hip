@@ -30,6 +30,27 @@ int launch_m1_inst(hipStream_t st, const LinearArgs& a) {
   return ofq_check_launch();
 }
 
+// many rows per wave: one block of 16 waves per CU, two from 128 rows per block on
+template<int H>
+int launch_m1_stream_inst(hipStream_t st, const LinearArgs& a) {
+  constexpr int NW = 16;
+  int grid = 256;
+  if ((a.n + grid - 1) / grid >= 128) grid = 512;
+  const int rpb = (int)((a.n + grid - 1) / grid);
+  grid = (int)((a.n + rpb - 1) / rpb);
+  M1Shape sh;
+  sh.N = (int)a.n;
+  sh.K = (int)a.k;
+  sh.rows_per_block = rpb;
+  sh.gshift = log2_exact(a.group_size);
+  sh.G = (int)(a.k / a.group_size);
+  gemv_w4_m1_stream<NW, H, 1><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
+      static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
+      static_cast<const f16*>(a.scale), static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
+      sh);
+  return ofq_check_launch();
+}
+
 template<int NW, int H, int XU>
 int launch_m1_glu_inst(hipStream_t st, const LinearArgs& a, const M1Glu& glu) {
   M1Shape sh;
@@ -104,7 +125,13 @@ bool gemv_m1_supported(const LinearArgs& a) {
 // longer rows two small blocks per CU, each with its own barrier, run ahead of one large one
 // (4096 x 11008: 6.3 against 6.7 us), with short rows the second staging of x costs more than
 // that gains (4096 x 4096: 3.55 against 3.8 us).
+// One row per wave while one resident round of blocks covers n (n <= 4096); beyond that, for rows
+// of at most 2 KB of codes, the streaming kernel (11008 x 4096: 6.2 against 6.4 us; 128256 x
+// 4096: 41.5 against 50 us, 6.5 TB/s).
 int launch_gemv_m1(hipStream_t st, const LinearArgs& a) {
+  if (a.n > 4096 && a.k <= 4096) {
+    return a.k <= 2048 ? launch_m1_stream_inst<1>(st, a) : launch_m1_stream_inst<2>(st, a);
+  }
 #define OFQ_M1_PLAIN(NW, H, XU) launch_m1_inst<NW, H, XU>(st, a)
   OFQ_M1_DISPATCH(a.k, OFQ_M1_PLAIN);
 #undef OFQ_M1_PLAIN
