@@ -9,7 +9,7 @@ weights (32 layers = 3.3 GB of packed weights, far beyond L2 + Infinity Cache, s
 streams its weights from HBM).  value = algorithmic bytes of all launches / wall time of the step.
 
 The same JSON line carries
-  roofline      for the dominant kernel (the 16-wave instance of the MFMA GEMV, which serves the
+  roofline      for the dominant kernel (gemv_w4_m1, the decode kernel for one row of x, on the
                 4096-row shapes: four 4096x4096 and one 4096x11008 per layer): algorithmic bytes
                 per launch / average launch duration, timed live with events on the launch stream
                 over a region that contains only that kernel's launches;
@@ -177,7 +177,7 @@ def main():
     avg_launch_us = ev_k_ms * 1e3 / (args.steps * launches_k4096)
     achieved = (bytes_k4096 / launches_k4096) / (avg_launch_us * 1e-6) / 1e9
     roofline = {
-        "kernel": "gemv_w4s_f16<16 waves, staged x> (n=4096 shapes: 4096x4096 x4, 4096x11008 x1 per layer)",
+        "kernel": "gemv_w4_m1 (a wave owns whole weight rows; n=4096 shapes: 4096x4096 x4, 4096x11008 x1 per layer)",
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "traffic": PMC_TRAFFIC_BYTES_PER_LAUNCH_M1 if (M == 1 and args.layers == 32) else None,
@@ -248,6 +248,23 @@ def main():
             "launches_per_step": 5 * args.layers,
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                          "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
+        # per shape: the GEMV alone over all layers, and beside it a plain read of the same weight
+        # tensors (torch.sum over their int32 view; its result is not used) in the same
+        # graph-replay harness: what a kernel that only reads those bytes takes on this box
+        by_shape = {}
+        for name, n, k, cnt in LLAMA7B_LAYER:
+            mats_s = [mat for mats in layers for mat in mats if mat[0] == name]
+            run_s = make_runner(lambda: [launch(mat) for mat in mats_s])
+            ev_s, _ = time_region(run_s, 10, 2)
+            us_s = ev_s * 1e3 / (10 * len(mats_s))
+            views = [mat[3].view(torch.int32) for mat in mats_s]
+            run_r = make_runner(lambda: [torch.sum(v) for v in views])
+            ev_r, _ = time_region(run_r, 10, 2)
+            gb_s = gemv_bytes(M, n, k) / (us_s * 1e-6) / 1e9
+            by_shape[f"{n}x{k}"] = {"us": round(us_s, 2), "gbps": round(gb_s, 1),
+                                    "frac": round(gb_s / HBM_PEAK_GBPS, 4),
+                                    "read_floor_us": round(ev_r * 1e3 / (10 * len(views)), 2)}
+        other[f"decode_w4a16_m{M}_by_shape"] = by_shape
         del layers
         torch.cuda.empty_cache()
         result["secondary"] = {**other, **secondary(L, _lib, torch, dev, args)}

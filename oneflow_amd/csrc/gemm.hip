@@ -20,16 +20,19 @@ namespace ofq {
 
 // Width of the weight tile under a 256-row tile of x.  The blocks run in rounds of one per CU;
 // a round costs about in proportion to the tile width, so the candidate with the smallest
-// (rounds x width) wins, the wider one on a tie (less L2 -> LDS traffic per MFMA).  352 is open
-// to the copy-fed GEMMs only (2048x11008: 8 x 32 = 256 tiles, exactly one round); 192 turns the
-// 258 or 344 tiles of m = 768 / 1024 at n = 11008 (two rounds of 128-wide tiles, the second
-// nearly empty) into one round of 174 / 232: 160 -> 115 us in-tile.
-int pick_tile_width(int64_t m, int64_t n, bool allow_352) {
+// (rounds x width) wins, the wider one on a tie (less L2 -> LDS traffic per MFMA).  384 (waves
+// 4 x 2, 64 x 192 per wave: 12 MFMAs per 8 fragment reads) is open to the copy-fed GEMMs only and
+// runs about a tenth faster per column than the narrower tiles on random operands (2048 x 11008
+// x 4096 bf16: 163 us against 182 us for 352-wide tiles on 8 x 1 waves, whose waves read 12
+// fragments per 11 MFMAs), which its cost is credited with; 192 turns the 258 or 344 tiles of
+// m = 768 / 1024 at n = 11008 (two rounds of 128-wide tiles, the second nearly empty) into one
+// round of 174 / 232: 160 -> 115 us in-tile.
+int pick_tile_width(int64_t m, int64_t n, bool allow_wide) {
   const int64_t m_tiles = (m + 255) / 256;
   auto cost = [&](int64_t bn) { return ((m_tiles * ((n + bn - 1) / bn) + 255) / 256) * bn; };
   int best = 128;
   if (cost(192) <= cost(best)) best = 192;
-  if (allow_352 && cost(352) <= cost(best)) best = 352;
+  if (allow_wide && cost(384) * 9 <= cost(best) * 10) best = 384;
   return best;
 }
 
@@ -48,8 +51,8 @@ int launch_plain(hipStream_t st, const LinearArgs& a, const void* wt) {
   ep.bias = static_cast<const S*>(a.bias);
   ep.out = static_cast<S*>(a.out);
   switch (pick_tile_width(a.m, a.n, true)) {
-    case 352:
-      return launch_core2<MF, B2Copy<352, 512>, EP, 256, 352, 8, 1>(st, a.x, a.k * 2, bp, ep, a.m,
+    case 384:
+      return launch_core2<MF, B2Copy<384, 512>, EP, 256, 384, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
                                                                     a.n, a.k / 64);
     case 192:
       return launch_core2<MF, B2Copy<192, 512>, EP, 256, 192, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
@@ -476,8 +479,8 @@ extern "C" int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, c
     ep.bias = static_cast<const TT<T>::storage*>(bias);                                        \
     ep.out = static_cast<TT<T>::storage*>(out);                                                \
     const int bn = m > 128 ? pick_tile_width(m, n, true) : 128;                                \
-    if (bn == 352) {                                                                           \
-      return launch_core2<MfmaI8, B2Copy<352, 512>, EP, 256, 352, 8, 1>(st, a, k, bp, ep, m,   \
+    if (bn == 384) {                                                                           \
+      return launch_core2<MfmaI8, B2Copy<384, 512>, EP, 256, 384, 4, 2>(st, a, k, bp, ep, m,   \
                                                                         n, k / 128);           \
     }                                                                                          \
     if (bn == 192) {                                                                           \
