@@ -65,7 +65,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="for a `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` run: a few direct launches of "
-                         "the hot path plus an elementwise kernel of known traffic (1 GiB read, "
+                         "the hot path (plain and fused step) plus an elementwise kernel of known traffic (1 GiB read, "
                          "1 GiB written) to scale the counters by; prints no result line")
     ap.add_argument("--pmc-gemm", action="store_true",
                     help="for a `rocprofv3 --pmc` run on the MFMA kernels: three launches each of the "
@@ -126,6 +126,33 @@ def main():
                 if mat[1] == 4096:
                     launch(mat)
 
+    # the same step with the block's neighbouring ops fused: q/k/v as one grouped launch,
+    # o, gate|up with the SiLU gating as one launch, down: 5 launches per layer, not 7 (+ gating)
+    glu_y = torch.empty((max(M, 8), 11008), dtype=torch.float16, device=dev)
+    vp = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    i64 = lambda v: (ctypes.c_int64 * len(v))(*v)
+
+    def step_fused(m=M):
+        stream = torch.cuda.current_stream().cuda_stream
+        for mats in layers:
+            qkv, o, gate, up, down = mats[0:3], mats[3], mats[4], mats[5], mats[6]
+            x4 = x_by_k[4096]
+            st = L.ofq_grouped_linear_gq(
+                stream, 3, vp([x4] * 3), vp([q[3] for q in qkv]), vp([q[4] for q in qkv]), None,
+                vp([q[5] for q in qkv]), vp([q[6] for q in qkv]), i64([m] * 3), i64([4096] * 3),
+                i64([4096] * 3), _lib.I8, _lib.F16, 4, 1, 1, 128)
+            if st != 0:
+                raise RuntimeError(f"ofq_grouped_linear_gq status {st}")
+            launch(o, m)
+            st = L.ofq_fused_glu_gq(stream, x4.data_ptr(), up[3].data_ptr(), up[4].data_ptr(), None,
+                                    up[5].data_ptr(), gate[3].data_ptr(), gate[4].data_ptr(), None,
+                                    gate[5].data_ptr(), glu_y.data_ptr(), up[6].data_ptr(),
+                                    gate[6].data_ptr(), 5, _lib.I8, _lib.F16, 4, 1, 1, 128, m,
+                                    11008, 4096)
+            if st != 0:
+                raise RuntimeError(f"ofq_fused_glu_gq status {st}")
+            launch(down, m)
+
     def make_runner(fn):
         if args.no_graph:
             return fn
@@ -159,6 +186,8 @@ def main():
             torch.add(src, 1.0, out=dst)  # vectorized_elementwise_kernel: 2^30 B in, 2^30 B out
         for _ in range(2):
             step_all()
+        for _ in range(2):
+            step_fused()
         torch.cuda.synchronize()
         return
 
@@ -214,57 +243,43 @@ def main():
                 "ms_per_step": round(wall_m / 10, 4), "gbps": round(gbps, 1),
                 "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                              "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
-        # the same step with the block's neighbouring ops fused: q/k/v as one grouped launch,
-        # o, gate|up with the SiLU gating as one launch, down: 5 launches per layer, not 7 (+ gating)
-        glu_y = torch.empty((max(M, 8), 11008), dtype=torch.float16, device=dev)
-        vp = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
-        i64 = lambda v: (ctypes.c_int64 * len(v))(*v)
+        for m in sorted({M, 4, 8}):
+            run_f = make_runner(lambda: step_fused(m))
+            _, wall_f = time_region(run_f, 10, 2)
+            b_m = sum(gemv_bytes(m, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER) * args.layers
+            gbps = (b_m + args.layers * m * 11008 * 2) / (wall_f / 10 * 1e-3) / 1e9
+            other[f"decode_w4a16_m{m}_grouped_qkv_and_glu"] = {
+                "ms_per_step": round(wall_f / 10, 4), "gbps": round(gbps, 1),
+                "launches_per_step": 5 * args.layers,
+                "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+                             "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
+        # per shape: the GEMV alone over all layers for 1, 4 and 8 rows of x, and beside it a
+        # kernel that only reads the codes of the same weight tensors (ofq_probe_read; 97% of the
+        # bytes the GEMV reads, in one launch per tensor) in the same graph-replay harness: what
+        # reading those bytes once takes on this box
+        sink = torch.zeros(1, dtype=torch.int32, device=dev)
 
-        def step_fused(m=M):
+        def read_only(mats):
             stream = torch.cuda.current_stream().cuda_stream
-            for mats in layers:
-                qkv, o, gate, up, down = mats[0:3], mats[3], mats[4], mats[5], mats[6]
-                x4 = x_by_k[4096]
-                st = L.ofq_grouped_linear_gq(
-                    stream, 3, vp([x4] * 3), vp([q[3] for q in qkv]), vp([q[4] for q in qkv]), None,
-                    vp([q[5] for q in qkv]), vp([q[6] for q in qkv]), i64([m] * 3), i64([4096] * 3),
-                    i64([4096] * 3), _lib.I8, _lib.F16, 4, 1, 1, 128)
+            for mat in mats:
+                st = L.ofq_probe_read(stream, mat[3].data_ptr(), mat[3].numel(), sink.data_ptr())
                 if st != 0:
-                    raise RuntimeError(f"ofq_grouped_linear_gq status {st}")
-                launch(o, m)
-                st = L.ofq_fused_glu_gq(stream, x4.data_ptr(), up[3].data_ptr(), up[4].data_ptr(), None,
-                                        up[5].data_ptr(), gate[3].data_ptr(), gate[4].data_ptr(), None,
-                                        gate[5].data_ptr(), glu_y.data_ptr(), up[6].data_ptr(),
-                                        gate[6].data_ptr(), 5, _lib.I8, _lib.F16, 4, 1, 1, 128, m,
-                                        11008, 4096)
-                if st != 0:
-                    raise RuntimeError(f"ofq_fused_glu_gq status {st}")
-                launch(down, m)
-        run_f = make_runner(step_fused)
-        _, wall_f = time_region(run_f, 10, 2)
-        gbps = (bytes_step + args.layers * M * 11008 * 2) / (wall_f / 10 * 1e-3) / 1e9
-        other[f"decode_w4a16_m{M}_grouped_qkv_and_glu"] = {
-            "ms_per_step": round(wall_f / 10, 4), "gbps": round(gbps, 1),
-            "launches_per_step": 5 * args.layers,
-            "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
-                         "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
-        # per shape: the GEMV alone over all layers, and beside it a plain read of the same weight
-        # tensors (torch.sum over their int32 view; its result is not used) in the same
-        # graph-replay harness: what a kernel that only reads those bytes takes on this box
-        by_shape = {}
-        for name, n, k, cnt in LLAMA7B_LAYER:
-            mats_s = [mat for mats in layers for mat in mats if mat[0] == name]
-            run_s = make_runner(lambda: [launch(mat) for mat in mats_s])
-            ev_s, _ = time_region(run_s, 10, 2)
-            us_s = ev_s * 1e3 / (10 * len(mats_s))
-            views = [mat[3].view(torch.int32) for mat in mats_s]
-            run_r = make_runner(lambda: [torch.sum(v) for v in views])
-            ev_r, _ = time_region(run_r, 10, 2)
-            gb_s = gemv_bytes(M, n, k) / (us_s * 1e-6) / 1e9
-            by_shape[f"{n}x{k}"] = {"us": round(us_s, 2), "gbps": round(gb_s, 1),
-                                    "frac": round(gb_s / HBM_PEAK_GBPS, 4),
-                                    "read_floor_us": round(ev_r * 1e3 / (10 * len(views)), 2)}
-        other[f"decode_w4a16_m{M}_by_shape"] = by_shape
+                    raise RuntimeError(f"ofq_probe_read status {st}")
+        for m in sorted({M, 1, 4, 8}):
+            by_shape = {}
+            for name, n, k, cnt in LLAMA7B_LAYER:
+                mats_s = [mat for mats in layers for mat in mats if mat[0] == name]
+                run_s = make_runner(lambda: [launch(mat, m) for mat in mats_s])
+                ev_s, _ = time_region(run_s, 10, 2)
+                us_s = ev_s * 1e3 / (10 * len(mats_s))
+                gb_s = gemv_bytes(m, n, k) / (us_s * 1e-6) / 1e9
+                by_shape[f"{n}x{k}"] = {"us": round(us_s, 2), "gbps": round(gb_s, 1),
+                                        "frac": round(gb_s / HBM_PEAK_GBPS, 4)}
+                if m == M:
+                    run_r = make_runner(lambda: read_only(mats_s))
+                    ev_r, _ = time_region(run_r, 10, 2)
+                    by_shape[f"{n}x{k}"]["read_floor_us"] = round(ev_r * 1e3 / (10 * len(mats_s)), 2)
+            other[f"decode_w4a16_m{m}_by_shape"] = by_shape
         del layers
         torch.cuda.empty_cache()
         result["secondary"] = {**other, **secondary(L, _lib, torch, dev, args)}

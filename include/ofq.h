@@ -312,6 +312,15 @@ int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, const float*
                         const float* b_scale, const void* bias, void* out, int out_dtype,
                         int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes);
 
+/*
+ * Measurement aid, no counterpart in the reference: a kernel that reads `bytes` (rounded down to
+ * 16) from buf once, one 16-byte request per lane, and computes nothing.  What it takes is the
+ * time below which no kernel that reads those bytes once can finish on this device; a benchmark
+ * reports it beside the decode kernels.  buf 16-byte aligned; sink: 4 writable bytes (left
+ * untouched in practice).
+ */
+int ofq_probe_read(void* stream, const void* buf, size_t bytes, void* sink);
+
 #ifdef __cplusplus
 }
 #endif

@@ -140,6 +140,42 @@ def test_glu_all_activations(t, m, n, k, split, g):
                     assert (yf != yr).mean() < 0.02, act
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 1000, 4096), (2, 344, 2048), (3, 136, 5120), (4, 2000, 4096),
+                                   (5, 37, 3072), (8, 1100, 4096), (8, 33, 11008), (4, 65, 11008)])
+def test_glu_and_grouped_few_rows_of_x_symmetric_int4_fp16(m, n, k):
+    """fp16, symmetric int4 in an int8 container, groups of 128, 1 .. 8 rows of x at real row
+    lengths (the decode case of both ops; one row of x takes the kernel in which a wave owns
+    whole weight rows).  Split GLU + a grouped call with three row counts on a shared x."""
+    import torch
+    import oneflow_amd as flow
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    rng = np.random.Generator(np.random.PCG64(m * 7 + n + k))
+    x, w, ws, _, b = _problem(rng, m, n, k, 4, True, np.int8, 128, "f16")
+    _, v, vs, _, c = _problem(rng, m, n, k, 4, True, np.int8, 128, "f16")
+    for act in ("fast_gelu", "silu", "none"):
+        y, wx, vx = _glu_call(L, _lib, torch, x, w, ws, None, b, v, vs, None, c, act, _lib.I8,
+                              _lib.F16, 4, True, 128, m, n, k)
+        r, _ = H.assert_linear_parity(wx, O.fused_linear(x, w, ws, None, b, 4, True, 1, 128), "f16", "wx")
+        assert r < 5e-4
+        r, _ = H.assert_linear_parity(vx, O.fused_linear(x, v, vs, None, c, 4, True, 1, 128), "f16", "vx")
+        assert r < 5e-4
+        y_ref = O.glu_gate(wx, vx, act)
+        yf, yr = O.to_f32(y).astype(np.float64), O.to_f32(y_ref).astype(np.float64)
+        assert (np.abs(yf - yr) <= 2.0001 * H.ulp_of(yr, "f16") + 1e-7).all(), act
+    ns = (n, max(1, n // 4), n + 13)
+    probs = [_problem(rng, m, nn, k, 4, True, np.int8, 128, "f16", bias=(i != 1))
+             for i, nn in enumerate(ns)]
+    tt = H.to_torch
+    outs = flow._C.grouped_linear_with_groupwise_quantized_weight(
+        [tt(x)] * 3, [tt(p[1]) for p in probs], [tt(p[2]) for p in probs], w_zeros=None,
+        bs=[tt(p[4]) for p in probs], num_bits=4, symmetric=True, group_dim=1, group_size=128)
+    for p, out in zip(probs, outs):
+        ref = O.fused_linear(x, p[1], p[2], None, p[4], 4, True, 1, 128)
+        r, _ = H.assert_linear_parity(H.to_numpy(out), ref, "f16", f"grouped n={p[1].shape[0]}")
+        assert r < 5e-4
+
+
 def test_glu_functional_matches_reference_style_composition():
     """flow._C.fused_glu_with_groupwise_quantized_weight against dequantize -> matmul -> gate in
     float64 (how the reference test builds its expectation, test_fused_glu.py:31-83), Llama

@@ -93,6 +93,29 @@ def test_decode_m1_row_per_wave_shapes(n, k, g, with_bias):
     assert r < 5e-4
 
 
+@pytest.mark.parametrize("m,n,k,g,with_bias", [
+    (2, 4096, 4096, 128, True), (3, 4099, 2048, 256, True), (4, 1000, 3072, 128, False),
+    (5, 300, 5120, 128, True), (6, 2048, 8192, 1024, True), (7, 64, 11008, 128, True),
+    (8, 4096, 4096, 128, True), (8, 129, 7936, 128, False), (4, 77, 13824, 128, True),
+    (3, 33, 16384, 128, True), (2, 50, 14336, 256, False), (8, 20000, 256, 128, True),
+    (8, 64, 11008, 128, True), (5, 64, 16384, 128, True),
+])
+def test_decode_few_rows_of_x_long_and_ragged_rows(m, n, k, g, with_bias):
+    """2 .. 8 rows of x, fp16, symmetric int4 in an int8 container: every row length up to 16384
+    (with lengths that are not a multiple of 2048), group sizes above 128, row counts off the
+    block sizes, and the shapes whose x does not fit LDS."""
+    rng = np.random.default_rng(n * 31 + k + m)
+    x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), "f16")
+    codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    w = H.pack_int4(codes)
+    scale = H.as_T(rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float32), "f16")
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), "f16") if with_bias else None
+    ref = O.fused_linear(x, w, scale, None, b, 4, True, 1, g)
+    got = _run(x, w, scale, None, b, 4, True, 1, g)
+    r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k} g={g}")
+    assert r < 5e-4
+
+
 @pytest.mark.parametrize("m", [1, 8])
 def test_same_weights_in_both_containers_differ_by_rounding_of_w_only(m):
     """The same symmetric 4-bit weights stored as int8 codes q and as uint8 codes q + 7: the int8
