@@ -12,6 +12,7 @@
 // min with 128-bit loads and wave shuffles and stores one (max,min) pair in the workspace; a
 // second tiny launch folds the pairs and does the scale / zero-point arithmetic.  No atomics,
 // no initialisation pass, and the result does not depend on block scheduling.
+#include <type_traits>
 #include "ofq_device.h"
 
 namespace ofq {
@@ -275,13 +276,35 @@ struct QParams {
   C upper, lower;
 };
 
-template<typename C, int MODE, bool FAKE>
-__device__ __forceinline__ C quant_one(C x, C scale, C zp, C upper, C lower) {
+// a / b for a that came from an fp16 value and a reciprocal y = 1 / b formed once per tensor (IEEE
+// division), b within [2^-60, 2^60]: the product a * y corrected twice with the exact remainder
+// (Markstein's division steps) is the correctly rounded quotient, bit for bit what `a / b`
+// gives, at 5 fused operations instead of the 11 of the division sequence the compiler emits
+// (which made the fp16 -> int8 kernel compute-bound).  Nothing over- or underflows: |a| is 0 or
+// in [2^-24, 65504].  Zero keeps its sign through a * y, infinity and NaN their class.
+__device__ __forceinline__ float div_of_half_value(float a, float b, float y) {
+  const float q0 = a * y;
+  const float r0 = __builtin_fmaf(-b, q0, a);
+  const float q1 = __builtin_fmaf(r0, y, q0);
+  const float r1 = __builtin_fmaf(-b, q1, a);
+  const float q = __builtin_fmaf(r1, y, q1);
+  // normal or subnormal a (class bits 3, 4, 7, 8): the corrected quotient
+  return __builtin_amdgcn_classf(a, 0x198) ? q : q0;
+}
+
+template<typename C, int MODE, bool FAKE, bool RECIP = false>
+__device__ __forceinline__ C quant_one(C x, C scale, C zp, C upper, C lower, C recip = 0) {
   C o;
-  if (MODE == kModeSym) {
-    o = t_rint<C>(x / scale);
+  C q;
+  if constexpr (RECIP) {
+    q = div_of_half_value(x, scale, recip);
   } else {
-    o = t_rint<C>(x / scale + zp);
+    q = x / scale;
+  }
+  if (MODE == kModeSym) {
+    o = t_rint<C>(q);
+  } else {
+    o = t_rint<C>(q + zp);
   }
   o = o > upper ? upper : o;
   o = o < lower ? lower : o;
@@ -310,7 +333,12 @@ struct Elem<double> {
 template<>
 struct Elem<f16> {
   static __device__ __forceinline__ float ld(const f16* p) { return (float)*p; }
-  static __device__ __forceinline__ void st(f16* p, float v) { *p = (f16)v; }
+  // The empty asm keeps the narrowing apart from a multiplication that produced v: fused, the
+  // compiler emits v_fma_mixlo_f16 with a +0 addend, which turns a product of -0 into +0.
+  static __device__ __forceinline__ void st(f16* p, float v) {
+    asm volatile("" : "+v"(v));
+    *p = (f16)v;
+  }
 };
 template<>
 struct Elem<bf16> {
@@ -358,6 +386,15 @@ quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
   C s0 = scale[0];
   if (cambricon) s0 = (C)exp2((double)(int)s0);  // scale = 2^int(shift)
   const C zp0 = MODE == kModeSym ? (C)0 : effective_zp<C, MODE>(zero_point[0]);
+  // fp16 input and one scale for the tensor: the division becomes a corrected multiplication
+  constexpr bool kHalfIn = std::is_same<IN, f16>::value && std::is_same<C, float>::value;
+  bool recip_ok = false;
+  C recip = 0;
+  if constexpr (kHalfIn) {
+    const float mag = __builtin_fabsf(s0);
+    recip_ok = per_tensor && mag >= 0x1p-60f && mag <= 0x1p60f;  // same for every lane
+    if (recip_ok) recip = 1.0f / s0;
+  }
   for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < n_packs; p += step) {
     const int64_t base = p * V;
     C s = s0, zp = zp0;
@@ -381,10 +418,44 @@ quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
       for (int e = 0; e < V; ++e) xin[e] = in[base + e];
     }
     OUT r[V];
+    if (recip_ok) {
+      if constexpr (kHalfIn && sizeof(OUT) == 1 && !FAKE && V % 4 == 0) {
+        // byte codes: the clamp moves behind the conversion (v_cvt_i32_f32 saturates and turns
+        // NaN into 0, which lies inside every code range), one integer median instead of two
+        // compares and two selects, and the bytes are merged in registers
+        const int lo = (int)lower, hi = (int)upper;
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const C x = (C)Elem<IN>::ld(&xin[e]);
-      Elem<OUT>::st(&r[e], quant_one<C, MODE, FAKE>(x, s, zp, upper, lower));
+        for (int e4 = 0; e4 < V; e4 += 4) {
+          uint32_t b[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float x = (float)Elem<IN>::ld(&xin[e4 + j]);
+            float q = div_of_half_value(x, s, recip);
+            if (MODE != kModeSym) q = q + zp;
+            const float t = t_rint<float>(q);
+            int v;
+            asm("v_cvt_i32_f32 %0, %1" : "=v"(v) : "v"(t));
+            v = v < lo ? lo : v;
+            b[j] = (uint32_t)(v > hi ? hi : v);
+          }
+          // low bytes of b[0..3] -> one word
+          const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+          const uint32_t hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+          reinterpret_cast<uint32_t*>(r)[e4 / 4] = lo2 | hi2;
+        }
+      } else if constexpr (kHalfIn) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const C x = (C)Elem<IN>::ld(&xin[e]);
+          Elem<OUT>::st(&r[e], quant_one<C, MODE, FAKE, true>(x, s, zp, upper, lower, recip));
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const C x = (C)Elem<IN>::ld(&xin[e]);
+        Elem<OUT>::st(&r[e], quant_one<C, MODE, FAKE>(x, s, zp, upper, lower));
+      }
     }
     constexpr int kOutBytes = V * (int)sizeof(OUT);
     if (kOutBytes % 16 == 0) {
@@ -400,6 +471,60 @@ quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
     } else {
 #pragma unroll
       for (int e = 0; e < V; ++e) out[base + e] = r[e];
+    }
+  }
+}
+
+// fp16 -> byte codes with one scale for the tensor (the activation quantisation in front of an
+// int8 matmul): a wave owns 1024 consecutive elements per turn and takes them as two contiguous
+// 1 KB requests (lane l: elements 8l.. and 512 + 8l..), so that every request and both 8-byte
+// stores of a wave are whole cache lines; the generic kernel's 32 bytes per lane make each request
+// touch half of every line.  elem_cnt a multiple of 1024.  Arithmetic as in quantize_kernel.
+template<typename OUT, int MODE>
+__global__ void __launch_bounds__(256)
+quantize_half_to_bytes_kernel(const f16* __restrict__ in, const float* __restrict__ scale,
+                              const float* __restrict__ zero_point, OUT* __restrict__ out,
+                              int64_t tiles, float upper, float lower, int cambricon) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t nwaves = (int64_t)gridDim.x * 4;
+  float s = scale[0];
+  if (cambricon) s = (float)exp2((double)(int)s);
+  const float zp = MODE == kModeSym ? 0.f : effective_zp<float, MODE>(zero_point[0]);
+  const float mag = __builtin_fabsf(s);
+  const bool recip_ok = mag >= 0x1p-60f && mag <= 0x1p60f;
+  const float recip = recip_ok ? 1.0f / s : 0.f;
+  const int lo = (int)lower, hi = (int)upper;
+  for (int64_t tile = wave; tile < tiles; tile += nwaves) {
+    const f16* src = in + tile * 1024 + lane * 8;
+    u32x4 raw[2];
+    raw[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
+    raw[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 512));
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const f16x8 xv = __builtin_bit_cast(f16x8, raw[hf]);
+      uint32_t words[2];
+#pragma unroll
+      for (int e4 = 0; e4 < 8; e4 += 4) {
+        uint32_t b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float x = (float)xv[e4 + j];
+          float q = recip_ok ? div_of_half_value(x, s, recip) : x / s;
+          if (MODE != kModeSym) q = q + zp;
+          const float t = t_rint<float>(q);
+          int v;
+          asm("v_cvt_i32_f32 %0, %1" : "=v"(v) : "v"(t));  // saturates; NaN -> 0
+          v = v < lo ? lo : v;
+          b[j] = (uint32_t)(v > hi ? hi : v);
+        }
+        const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+        const uint32_t hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+        words[e4 / 4] = lo2 | hi2;
+      }
+      u32x2 w2 = {words[0], words[1]};
+      __builtin_nontemporal_store(
+          w2, reinterpret_cast<u32x2*>(out + tile * 1024 + hf * 512 + lane * 8));
     }
   }
 }
@@ -423,6 +548,15 @@ int launch_quant(hipStream_t st, const void* in, const void* scale, const void* 
   OUT* o = static_cast<OUT*>(out);
   const C* s = static_cast<const C*>(scale);
   const C* z = static_cast<const C*>(zp);
+  if constexpr (std::is_same<IN, f16>::value && std::is_same<C, float>::value && sizeof(OUT) == 1
+                && !FAKE) {
+    if (scale_size == 1 && elem_cnt % 1024 == 0) {
+      const int64_t tiles = elem_cnt / 1024;
+      quantize_half_to_bytes_kernel<OUT, MODE><<<grid_for(tiles, 4), 256, 0, st>>>(
+          i, s, z, o, tiles, upper, lower, cambricon);
+      return ofq_check_launch();
+    }
+  }
   if (panel % V == 0 && elem_cnt % V == 0) {
     quantize_kernel<IN, C, OUT, MODE, FAKE, V><<<grid_for(elem_cnt / V, 256), 256, 0, st>>>(
         i, s, z, o, elem_cnt, panel, scale_size, upper, lower, cambricon);

@@ -126,6 +126,50 @@ def test_layer_norm_exact_statistics_rows_bit_exact(t, cols):
         assert H.to_numpy(s)[0] == s_ref[0]
 
 
+def _scale_with_mantissa(exp, mant):
+    return np.array([(np.uint32(exp + 127) << np.uint32(23)) | np.uint32(mant)], dtype=np.uint32).view(np.float32)
+
+
+@pytest.mark.parametrize("scheme", ["symmetric", "affine"])
+def test_quantization_of_every_fp16_value_bit_exact(scheme):
+    """fp16 input with one scale per tensor replaces the division by a multiplication with the
+    reciprocal and two exact-remainder corrections.  Every finite fp16 value and the infinities
+    (both zeros, subnormals included) against scales whose mantissas are the hard cases of a
+    division (all ones, just above a power of two, random), scales of either sign, and scales
+    outside the range the corrected multiplication is used for: int8 codes, codes stored as fp16
+    and fake quantization, all bit for bit what `x / scale` gives in the oracle."""
+    import oneflow_amd as flow
+    import torch
+    bits16 = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    x = bits16.view(np.float16)
+    x = x[~np.isnan(x)]
+    x = np.tile(x, 2)[: (2 * x.size) // 16 * 16].reshape(-1, 16)  # whole 16-element packs
+    rng = np.random.default_rng(11)
+    scales = [_scale_with_mantissa(e, m) for e, m in
+              [(-7, 0x7FFFFF), (-7, 0x7FFFFE), (-3, 0), (-3, 1), (2, 0x7FFFFD), (-12, 0x555555),
+               (9, 0x2AAAAA), (-59, 0x7FFFFF), (59, 3), (-70, 0x123456), (70, 0x654321)]]
+    scales += [np.array([v], dtype=np.float32) for v in rng.uniform(1e-4, 50.0, size=6)]
+    scales += [-scales[0], -scales[5]]
+    xf = x.astype(np.float32)
+    for sc in scales:
+        zp = np.array([0.0 if scheme == "symmetric" else 3.0], dtype=np.float32)
+        ref = O.quantization(xf, sc, zp, "google", 8, scheme, zp_mode="cuda")
+        ref_fake = O.fake_quantization(xf, sc, zp, "google", 8, scheme, zp_mode="cuda")
+        xt, st, zt = H.to_torch(x), H.to_torch(sc), H.to_torch(zp)
+        got_f16 = H.to_numpy(flow._C.quantization(xt, st, zt, "google", 8, scheme))
+        assert np.array_equal(got_f16.view(np.uint16), ref.astype(np.float16).view(np.uint16)), sc
+        got_fake = H.to_numpy(flow._C.fake_quantization(xt, st, zt, "google", 8, scheme))
+        assert np.array_equal(got_fake.view(np.uint16),
+                              ref_fake.astype(np.float16).view(np.uint16)), sc
+        # byte codes: whole 1024-element tiles (the kernel with two 1 KB requests per wave) and a
+        # size that is not a multiple of 1024 (the generic kernel)
+        code_dt, code_np = (torch.int8, np.int8) if scheme == "symmetric" else (torch.uint8, np.uint8)
+        for rows in (x.shape[0], x.shape[0] - 1):
+            got_b = H.to_numpy(flow._C.quantization(H.to_torch(x[:rows]), st, zt, "google", 8,
+                                                    scheme, out_dtype=code_dt))
+            assert np.array_equal(got_b, ref[:rows].astype(code_np)), (sc, rows)
+
+
 def test_dynamic_quantize_and_matmul_quant():
     import oneflow_amd as flow
     import torch
