@@ -349,6 +349,141 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
   if (lane == 0 && gw < rows) wave_absmax[gw] = amax;
 }
 
+// Rows of exactly 512 * NP elements of a 16-bit type, gamma and beta both present, no residual:
+// the same one-wave-per-row scheme with nothing conditional inside the row (no partial packs, no
+// null checks), the deviations kept in registers between the variance and the normalisation, the
+// fp16 row sum formed with packed dot products, and, when a wave walks several rows (LOOP), the
+// next row requested before the current one is worked on.  At 2048 x 4096 the general kernel
+// spends about 1100 vector instructions per row, this one about half; both are bound by that
+// arithmetic once the row has arrived, not by HBM.
+template<typename T, int NP, bool LOOP>
+__global__ void __launch_bounds__(kLnBlock)
+ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
+                      const typename TT<T>::storage* __restrict__ gamma,
+                      const typename TT<T>::storage* __restrict__ beta,
+                      typename TT<T>::storage* __restrict__ y, float* __restrict__ wave_absmax,
+                      int64_t rows, float eps) {
+  static_assert(sizeof(typename TT<T>::storage) == 2, "16-bit types only");
+  constexpr int kCols = NP * 512;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t gw = (int64_t)blockIdx.x * (kLnBlock / kWave) + (threadIdx.x >> 6);
+  const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / kWave);
+  if (gw >= rows) return;
+  u32x4 cur[NP], nxt[LOOP ? NP : 1], gr[NP], br[NP];
+  {
+    const typename TT<T>::storage* xr = x + gw * kCols + lane * 8;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      cur[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr + i * 512));
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    gr[i] = *reinterpret_cast<const u32x4*>(gamma + lane * 8 + i * 512);
+    br[i] = *reinterpret_cast<const u32x4*>(beta + lane * 8 + i * 512);
+  }
+  float amax = 0.0f;
+  f16x8 amax8 = {(f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f};
+  for (int64_t row = gw; row < rows; row += nwaves) {
+    bool more = false;
+    if constexpr (LOOP) {
+      more = row + nwaves < rows;  // the same for every lane
+      if (more) {
+        const typename TT<T>::storage* xn = x + (row + nwaves) * kCols + lane * 8;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          nxt[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xn + i * 512));
+        }
+      }
+    }
+    float f[NP][8];
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      RawPack<T> rp;
+      rp.q[0] = cur[i];
+      widen<T>(rp, f[i]);
+      if constexpr (TT<T>::dtype == OFQ_F16) {
+        // (1, 1) held in a register: with the constant as a literal operand the compiler emits
+        // the four dot products of a pack with one and the same source register
+        uint32_t ones_bits = 0x3c003c00u;
+        asm volatile("" : "+v"(ones_bits));
+        const f16x2 ones = __builtin_bit_cast(f16x2, ones_bits);
+        // (pairs taken from the whole-vector bit cast: `bit_cast<f16x2>(cur[i][w])` came out of
+        // the compiler as word 0 for every w)
+        const f16x8 h = __builtin_bit_cast(f16x8, cur[i]);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 0, 1), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 2, 3), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 4, 5), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 6, 7), ones, sum, false);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += f[i][e];
+      }
+    }
+    sum = wave_reduce(sum, OpSum());
+    const float mean = sum / (float)kCols;
+    float m2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        f[i][e] = f[i][e] - mean;
+        m2 = __builtin_fmaf(f[i][e], f[i][e], m2);
+      }
+    }
+    m2 = wave_reduce(m2, OpSum());
+    const float var = fmaxf(m2 / (float)kCols, 0.0f);
+    const float inv = 1.0f / __builtin_sqrtf(var + eps);
+    typename TT<T>::storage* yr = y + row * kCols + lane * 8;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      if constexpr (TT<T>::dtype == OFQ_F16) {
+        f16x8 t;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = (f16)(f[i][e] * inv);
+        t = t * __builtin_bit_cast(f16x8, gr[i]);
+        t = t + __builtin_bit_cast(f16x8, br[i]);
+        // |t| by clearing the sign bits of the four words (elementwise abs of the vector comes
+        // out as three instructions per pair)
+        const u32x4 tb = __builtin_bit_cast(u32x4, t);
+        const u32x4 ab = {tb[0] & 0x7FFF7FFFu, tb[1] & 0x7FFF7FFFu, tb[2] & 0x7FFF7FFFu,
+                          tb[3] & 0x7FFF7FFFu};
+        amax8 = __builtin_elementwise_max(amax8, __builtin_bit_cast(f16x8, ab));
+        *reinterpret_cast<u32x4*>(yr + i * 512) = tb;
+      } else {
+        RawPack<T> gp, bp;
+        gp.q[0] = gr[i];
+        bp.q[0] = br[i];
+        float g[8], b[8], o[8];
+        widen<T>(gp, g);
+        widen<T>(bp, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float t = TT<T>::round(f[i][e] * inv);
+          t = TT<T>::round(t * g[e]);
+          t = TT<T>::round(t + b[e]);
+          o[e] = t;
+          amax = fmaxf(amax, fabsf(t));
+        }
+        store8<T>(yr + i * 512, o);
+      }
+    }
+    if constexpr (LOOP) {
+      if (more) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) cur[i] = nxt[i];
+      }
+    }
+  }
+  if constexpr (TT<T>::dtype == OFQ_F16) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, (float)amax8[e]);
+  }
+  amax = wave_reduce(amax, OpMax());
+  if (lane == 0) wave_absmax[gw] = amax;
+}
+
 // any cols: three passes over the row through L2 (the row was just read, so only the first
 // pass touches HBM), scalar accesses.
 template<typename T, bool SKIP>
@@ -452,6 +587,34 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
   constexpr int kWavesPerBlock = kLnBlock / kWave;
   // fp32 rows beyond 2048 elements would not fit a lane's registers at two waves per SIMD
   const int64_t wave_packs = (sizeof(S) == 4 ? 4 : 8) * kWave;
+  if constexpr (sizeof(S) == 2 && !SKIP) {
+    const int np = (int)(cols / 512);
+    if (vec_ok && gamma != nullptr && beta != nullptr && cols % 512 == 0
+        && (np == 1 || np == 2 || np == 4 || np == 8)) {
+      // one row per wave while the rows fit 16 waves per CU; beyond that 8 waves per CU walk the
+      // rows with the next row in flight
+      const bool loop = rows > 256 * 16;
+      const int64_t waves = loop ? 256 * 8 : rows;
+      const int grid = (int)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+      nparts = waves;
+#define OFQ_LN_FULL(NPV)                                                                        \
+  if (loop) {                                                                                    \
+    ln_observer_wave_full<T, NPV, true><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, eps); \
+  } else {                                                                                       \
+    ln_observer_wave_full<T, NPV, false><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows,    \
+                                                                    eps);                        \
+  }
+      switch (np) {
+        case 1: OFQ_LN_FULL(1) break;
+        case 2: OFQ_LN_FULL(2) break;
+        case 4: OFQ_LN_FULL(4) break;
+        default: OFQ_LN_FULL(8) break;
+      }
+#undef OFQ_LN_FULL
+      ln_observer_finalize<<<1, kWave, 0, st>>>(ws, nparts, bits, scale, zero_point);
+      return ofq_check_launch();
+    }
+  }
   if (vec_ok && npacks <= wave_packs) {
     // about 32 KB of rows in flight per CU streams best: 4 waves per CU for 8 KB rows, up to 16
     // for rows of 2 KB and less (16384 x 1024 fp16: 33 -> 23 us); with more rows than waves a
