@@ -416,9 +416,31 @@ def secondary(L, _lib, torch, dev, args):
                                                         g, m, n, k, None, 0), "prefill"))
     flops = 2.0 * m * n * k
     tf = flops / (us * 1e-6) / 1e12
+    # Two yardsticks for the same shape, measured here so that they can be checked: (1) the same
+    # call on operands that toggle few bits (x = 0, all codes equal): MFMA throughput on this part
+    # depends on the data (power and clock), and the headline above is quoted on random operands;
+    # (2) the vendor GEMM (torch.matmul, bf16 x bf16 with the weights already dequantised, i.e.
+    # without the dequantisation this op has to do) on random operands of the same shape.
+    x0 = torch.zeros_like(x)
+    w0 = torch.full_like(w, 128)
+    us_const = timeit(lambda: chk(L.ofq_fused_linear_gq(cs(), x0.data_ptr(), w0.data_ptr(),
+                                                        sc.data_ptr(), ze.data_ptr(), None,
+                                                        o.data_ptr(), _lib.U8, _lib.BF16, 8, 0, 1,
+                                                        g, m, n, k, ws.data_ptr(), ws_bytes),
+                                  "prefill, constant operands"))
+    del x0, w0
+    us_vendor = None
+    try:
+        wd = torch.randn((n, k), device=dev).to(torch.bfloat16)
+        us_vendor = timeit(lambda: torch.matmul(x, wd.t(), out=o))
+        del wd
+    except Exception as e:  # the yardstick must not take the benchmark down
+        print(f"bench.py: vendor GEMM yardstick failed: {e}", file=sys.stderr)
     out["prefill_w8a16_bf16_m2048"] = {
         "us": round(us, 2), "tflops": round(tf, 1), "workspace_bytes": ws_bytes,
         "us_without_workspace": round(us_fused, 2),
+        "us_same_call_constant_operands": round(us_const, 2),
+        "us_vendor_gemm_bf16_same_shape_random_operands": None if us_vendor is None else round(us_vendor, 2),
         "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS["bf16"],
                      "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS["bf16"], 4)}}
     del x, w, sc, ze, o, ws

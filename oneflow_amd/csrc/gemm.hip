@@ -332,8 +332,15 @@ int mq_splits(int64_t m, int64_t n, int64_t k) {
   // long rows (k >= 8192) already pay for slices from 33 rows of a on: 4096 x 11008 at m = 64
   // streams in 33 us and runs in 22 us as slices
   if (m <= (k >= 8192 ? kMatmulQuantRowsMaxM / 2 : kMatmulQuantRowsMaxM) || k % 128 != 0) return 1;
-  const int64_t bm = m > 128 ? 256 : 128;
-  const int64_t slots = m > 128 ? 256 : 512;
+  int64_t bm = m > 128 ? 256 : 128;
+  int64_t slots = m > 128 ? 256 : 512;
+  // up to 512 rows on a weight with few column tiles: 128-row tiles and fewer, longer slices
+  // write half the partial sums (256 x 4096 x 4096: 21.2 -> 18.8 us, 128 rows: 18.2 -> 15.1 us)
+  const bool few_tiles = m <= 512 && ((m + 127) / 128) * ((n + 127) / 128) <= 128;
+  if (few_tiles) {
+    bm = 128;
+    slots = m <= 128 ? 128 : 256;
+  }
   const int64_t blocks = ((m + bm - 1) / bm) * ((n + 127) / 128);
   int64_t s = slots / blocks;
   const int64_t kt = k / 128;
@@ -386,7 +393,8 @@ int launch_mq_split(hipStream_t st, const void* a, const BCopyParams& bp, const 
   EpPartialI32::Params pp;
   pp.out = partials;
   int rc;
-  if (m > 128) {
+  const bool few_tiles = m <= 512 && ((m + 127) / 128) * ((n + 127) / 128) <= 128;  // as mq_splits
+  if (m > 128 && !few_tiles) {
     rc = launch_core2<MfmaI8, B2Copy<128, 512>, EpPartialI32, 256, 128, 4, 2>(st, a, k, bp, pp, m,
                                                                              n, k / 128, splits);
   } else {
