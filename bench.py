@@ -32,12 +32,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the dominant kernel (mean over its launches of one step) from two
-# `rocprofv3 --pmc` runs of `bench.py --pmc-calibration` (FETCH_SIZE, then WRITE_SIZE, each scaled
-# by what the same counter reads for an elementwise kernel of known size: x2.0 and x1.0); the
-# summary is profiles/gemv_w4s_f16__llama7b_decode_m1__hbm_traffic_pmc.txt (11,816,70x B, the last
-# digits move from run to run; rounded to 1000 B here).  Valid for m = 1 only.
-PMC_TRAFFIC_BYTES_PER_LAUNCH_M1 = 11817000
+# HBM bytes per launch of the dominant kernel (mean over the launches of the roofline region: four
+# of 4096x4096 to one of 4096x11008) from two `rocprofv3 --pmc` runs of `bench.py --pmc-calibration`
+# (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for an elementwise
+# kernel of known size: x2.0 and x1.0); the summary is
+# profiles/gemv_w4_m1__llama7b_decode_m1__hbm_traffic_pmc.txt (11,767,863 B; rounded to 1000 B
+# here).  Valid for m = 1 only.
+PMC_TRAFFIC_BYTES_PER_LAUNCH_M1 = 11768000
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "i8": 5000.0}
 
 LLAMA7B_LAYER = [  # (name, n, k, count per decoder layer)

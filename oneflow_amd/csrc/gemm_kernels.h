@@ -310,9 +310,7 @@ struct B2Dequant {
 };
 
 // NSTAGE LDS stages; the copies of tile t are issued at the top of iteration t-(NSTAGE-1).
-// DBG (experiments only): 1 = no MFMA, 2 = no global traffic after the prologue,
-// 5 = codes are fetched but not converted
-template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2, int DBG = 0>
+template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
            typename EP::Params ep, int M, int N, int KT_total, int kt_split, int m_tiles,
@@ -400,8 +398,8 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
   // Issue order per iteration: code loads first, copies last, so that "at most kCopyOps
   // outstanding" at the end retires everything except the copies just issued.
   auto iteration = [&](int kt, typename BP::Regs& st_regs, typename BP::Regs& ld_regs) {
-    const bool more_copies = DBG != 2 && kt + D < KT;
-    if (DBG != 2 && !BP::kDirect && kt + 2 < KT)
+    const bool more_copies = kt + D < KT;
+    if (!BP::kDirect && kt + 2 < KT)
       BP::load(bp, n0, kt_base + kt + 2, wave, lane, tid, ld_regs, nullptr);
     if (more_copies) issue_copies(kt + D, ld_regs);
     uint8_t* cur = stage_of(kt);
@@ -434,16 +432,12 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          if (DBG == 1) {
-            acc[i][j][0] += af[set][i][0] + bf[set][j][0];
-          } else {
-            // weights as the first operand: the 32x32 result is D[n][m], so a lane ends up with
-            // 4 CONSECUTIVE n per register quad -- what the row-major output wants
-            acc[i][j] = MF::mma(bf[set][j], af[set][i], acc[i][j]);
-          }
+          // weights as the first operand: the 32x32 result is D[n][m], so a lane ends up with
+          // 4 CONSECUTIVE n per register quad -- what the row-major output wants
+          acc[i][j] = MF::mma(bf[set][j], af[set][i], acc[i][j]);
         }
       // a quarter of the conversions per k-step, in the shadow of the MFMAs just issued
-      if (store_b && DBG != 5) BP::store_part(bp, st_regs, nxt + kABytes, tid, ks);
+      if (store_b) BP::store_part(bp, st_regs, nxt + kABytes, tid, ks);
     }
     // tile kt+1 must be complete: its copies are older than those issued in this iteration
     if (D > 1 && more_copies) {
@@ -539,7 +533,7 @@ gemm_core2(const uint8_t* __restrict__ A, int64_t lda, typename BP::Params bp,
   }
 }
 
-template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2, int DBG = 0>
+template<class MF, class BP, class EP, int BM, int BN, int WM, int WN, int NSTAGE = 2>
 int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::Params& bp,
                  const typename EP::Params& ep, int64_t M, int64_t N, int64_t KT,
                  int splits = 1) {
@@ -547,7 +541,7 @@ int launch_core2(hipStream_t st, const void* A, int64_t lda, const typename BP::
   const int n_tiles = (int)((N + BN - 1) / BN);
   // the stages; the epilogue stages its output panels in the same memory
   const size_t lds_bytes = NSTAGE * (size_t)(BM + BN) * kStageRow;
-  auto kern = gemm_core2<MF, BP, EP, BM, BN, WM, WN, NSTAGE, DBG>;
+  auto kern = gemm_core2<MF, BP, EP, BM, BN, WM, WN, NSTAGE>;
   if (lds_bytes > 64 * 1024) {
     static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
     if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), (int)lds_bytes, lds_allowed)) return OFQ_ERR_LAUNCH;

@@ -233,8 +233,6 @@ __device__ __forceinline__ float unit_corr_of(const u32x4 a, const u32x4 b) {
   return unit_corr(lo, hi);
 }
 
-// DBG (timing experiments only, results are then wrong): 1 = no MFMA/bit work, 2 = no LDS x
-// operand reads, 4 = no cross-wave reduction, 8 = no x staging.
 // Pins the widening of a prefetched bias value to the place of use: without the empty asm the
 // compiler sinks the conversion (and the wait for every load issued so far) up to the load.
 __device__ __forceinline__ f16 bias_at_end(uint16_t raw) {
@@ -243,7 +241,7 @@ __device__ __forceinline__ f16 bias_at_end(uint16_t raw) {
   return __builtin_bit_cast(f16, (uint16_t)v);
 }
 
-template<int NWAVES, int UNROLL, bool STAGED, int DBG = 0>
+template<int NWAVES, int UNROLL, bool STAGED>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
              const f16* __restrict__ scale, const f16* __restrict__ bias,
@@ -274,7 +272,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const bool has_x = r < M;
 
   // ---- loads that feed LDS are issued first so that they return before the weights ---------
-  const int nunits = (STAGED && !(DBG & 8)) ? (M * K) >> 4 : 0;
+  const int nunits = STAGED ? (M * K) >> 4 : 0;
   u32x4 xu[kGemvMaxUnits][2];
   if (STAGED) {
 #pragma unroll
@@ -386,10 +384,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
       const int c = chunk_of(p0, u);
       if (c < nchunks) {
         u32x4 xa[4];
-        if (DBG & 2) {
-#pragma unroll
-          for (int t = 0; t < 4; ++t) xa[t] = u32x4{0x3c003c00u + (uint32_t)c, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
-        } else if (STAGED) {
+        if (STAGED) {
           const u32x4* xp = reinterpret_cast<const u32x4*>(xrec + c * xrec_stride);
 #pragma unroll
           for (int t = 0; t < 4; ++t) xa[t] = xp[t];
@@ -405,13 +400,9 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
         // the accumulator starts at -corr (staged), or corr is built alongside (not staged)
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         f32x4 corr = {0.f, 0.f, 0.f, 0.f};
-        if (STAGED && !(DBG & 2)) acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
-        if (DBG & 1) {
-          acc[0] += __builtin_bit_cast(float, wq[u][0] ^ wq[u][1] ^ xa[0][0]);
-          acc[1] += __builtin_bit_cast(float, wq[u][2] ^ wq[u][3] ^ xa[1][0] ^ xa[2][1] ^ xa[3][2]);
-        }
+        if (STAGED) acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
 #pragma unroll
-        for (int h = 0; h < 2 && !(DBG & 1); ++h) {
+        for (int h = 0; h < 2; ++h) {
           const uint32_t w0 = wq[u][2 * h];
           const uint32_t w1 = wq[u][2 * h + 1];
           const uint32_t w0s = w0 >> 8, w1s = w1 >> 8;
@@ -449,10 +440,6 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
     }
   }
   // lane holds D[m = 4*kb + v][n = n0 + r]; only rows m < M travel through LDS
-  if (DBG & 4) {
-    if (wave == 0 && kb == 0 && n0 + r < N) out[n0 + r] = (f16)(total[0] + total[1] + total[2] + total[3]);
-    return;
-  }
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     const int m = 4 * kb + v;
