@@ -66,7 +66,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="for a `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` run: a few direct launches of "
-                         "the hot path (plain and fused step) plus an elementwise kernel of known traffic (1 GiB read, "
+                         "the hot path (plain and fused step), the LayerNorm -> quantize pair, plus an elementwise kernel of known traffic (1 GiB read, "
                          "1 GiB written) to scale the counters by; prints no result line")
     ap.add_argument("--pmc-gemm", action="store_true",
                     help="for a `rocprofv3 --pmc` run on the MFMA kernels: three launches each of the "
@@ -189,6 +189,27 @@ def main():
             step_all()
         for _ in range(2):
             step_fused()
+        # the activation front end of the int8 path: LayerNorm + observer, then quantisation of the
+        # y just written, on fresh buffers each time (is y re-read from HBM or from the caches?)
+        mm, kk = 2048, 4096
+        gam = torch.randn(kk, device=dev).to(torch.float16)
+        bet = torch.randn(kk, device=dev).to(torch.float16)
+        sc1 = torch.empty(1, dtype=torch.float32, device=dev)
+        zp1 = torch.empty(1, dtype=torch.float32, device=dev)
+        lws = torch.empty(mm * 4, dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream().cuda_stream
+        for _ in range(4):
+            xa = torch.randn((mm, kk), device=dev).to(torch.float16)
+            ya = torch.empty_like(xa)
+            qa = torch.empty((mm, kk), dtype=torch.int8, device=dev)
+            st = L.ofq_fused_layer_norm_min_max_observer(stream, xa.data_ptr(), gam.data_ptr(),
+                                                         bet.data_ptr(), ya.data_ptr(), sc1.data_ptr(),
+                                                         zp1.data_ptr(), _lib.F16, mm, kk, 1e-5, 8,
+                                                         lws.data_ptr(), mm * 4)
+            st |= L.ofq_quantization(stream, ya.data_ptr(), sc1.data_ptr(), zp1.data_ptr(),
+                                     qa.data_ptr(), _lib.F16, _lib.I8, mm * kk, 1, 8, 0, 0, 0)
+            if st != 0:
+                raise RuntimeError(f"layer norm / quantization status {st}")
         torch.cuda.synchronize()
         return
 
