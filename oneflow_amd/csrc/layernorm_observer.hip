@@ -356,14 +356,18 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
 // next row requested before the current one is worked on.  At 2048 x 4096 the general kernel
 // spends about 1100 vector instructions per row, this one about half; both are bound by that
 // arithmetic once the row has arrived, not by HBM.
-template<typename T, int NP, bool LOOP>
+// SKIP: the normalised row is (x + bias[c]) + skip * T(alpha) (see the top of the file), formed
+// as the row arrives and kept in storage format in place of x; the next row is then not
+// requested ahead (LOOP must be false), the registers hold the residual inputs instead.
+template<typename T, int NP, bool LOOP, bool SKIP = false>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
                       const typename TT<T>::storage* __restrict__ gamma,
                       const typename TT<T>::storage* __restrict__ beta,
                       typename TT<T>::storage* __restrict__ y, float* __restrict__ wave_absmax,
-                      int64_t rows, float eps) {
+                      int64_t rows, float eps, SkipArgs<T> sk = SkipArgs<T>()) {
   static_assert(sizeof(typename TT<T>::storage) == 2, "16-bit types only");
+  static_assert(!(SKIP && LOOP), "the residual variant does not prefetch");
   constexpr int kCols = NP * 512;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t gw = (int64_t)blockIdx.x * (kLnBlock / kWave) + (threadIdx.x >> 6);
@@ -393,6 +397,50 @@ ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
           nxt[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xn + i * 512));
+        }
+      }
+    }
+    if constexpr (SKIP) {
+      if (row != gw) {  // (rows after the wave's first: x was not requested ahead)
+        const typename TT<T>::storage* xr2 = x + row * kCols + lane * 8;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          cur[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr2 + i * 512));
+        }
+      }
+      u32x4 sr[NP], bb[NP];
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        if (sk.skip) {
+          sr[i] = __builtin_nontemporal_load(
+              reinterpret_cast<const u32x4*>(sk.skip + row * kCols + lane * 8 + i * 512));
+        }
+        if (sk.bias) bb[i] = *reinterpret_cast<const u32x4*>(sk.bias + lane * 8 + i * 512);
+      }
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        if constexpr (TT<T>::dtype == OFQ_F16) {
+          // native packed fp16 arithmetic rounds once per operation, which is what rounding the
+          // fp32 result of each operation to fp16 gives as well (an absent input enters as +0)
+          f16x8 v = __builtin_bit_cast(f16x8, cur[i]);
+          const f16x8 zero8 = {(f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f};
+          v = v + (sk.bias ? __builtin_bit_cast(f16x8, bb[i]) : zero8);
+          const f16 a = (f16)sk.alpha;
+          const f16x8 sa = sk.skip ? __builtin_bit_cast(f16x8, sr[i]) * a : zero8 * a;
+          v = v + sa;
+          cur[i] = __builtin_bit_cast(u32x4, v);
+        } else {
+          RawPack<T> xp, sp, bp;
+          xp.q[0] = cur[i];
+          float fx[8], fb[8], fs[8], o[8];
+          widen<T>(xp, fx);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) fb[e] = fs[e] = 0.f;
+          if (sk.bias) { bp.q[0] = bb[i]; widen<T>(bp, fb); }
+          if (sk.skip) { sp.q[0] = sr[i]; widen<T>(sp, fs); }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] = skip_sum<T>(fx[e], fb[e], fs[e], sk.alpha);
+          cur[i] = narrow<T>(o).q[0];
         }
       }
     }
@@ -587,18 +635,22 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
   constexpr int kWavesPerBlock = kLnBlock / kWave;
   // fp32 rows beyond 2048 elements would not fit a lane's registers at two waves per SIMD
   const int64_t wave_packs = (sizeof(S) == 4 ? 4 : 8) * kWave;
-  if constexpr (sizeof(S) == 2 && !SKIP) {
+  if constexpr (sizeof(S) == 2) {
     const int np = (int)(cols / 512);
     if (vec_ok && gamma != nullptr && beta != nullptr && cols % 512 == 0
         && (np == 1 || np == 2 || np == 4 || np == 8)) {
       // one row per wave while the rows fit 16 waves per CU; beyond that 8 waves per CU walk the
       // rows with the next row in flight
       const bool loop = rows > 256 * 16;
+      // (the residual variant at NP = 8 holds 230 registers: 8 waves per CU there as well)
       const int64_t waves = loop ? 256 * 8 : rows;
       const int grid = (int)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
       nparts = waves;
 #define OFQ_LN_FULL(NPV)                                                                        \
-  if (loop) {                                                                                    \
+  if (SKIP) {                                                                                    \
+    ln_observer_wave_full<T, NPV, false, SKIP><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws,    \
+                                                                          rows, eps, sk);        \
+  } else if (loop) {                                                                             \
     ln_observer_wave_full<T, NPV, true><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, eps); \
   } else {                                                                                       \
     ln_observer_wave_full<T, NPV, false><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows,    \
