@@ -275,6 +275,50 @@ def main():
                 "launches_per_step": 5 * args.layers,
                 "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                              "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
+        # the offline tile-major copy of the weights (ofq_groupwise_repack) for 4 and 8 rows of x;
+        # a shape the tiled call does not serve at that m (8 rows of 11008 do not fit LDS) keeps
+        # the row-major call, as a caller would
+        tiled = {}
+        for mats in layers:
+            for mat in mats:
+                nb = L.ofq_groupwise_repack_bytes(4, mat[1], mat[2])
+                t = torch.empty(nb, dtype=torch.int8, device=dev)
+                st = L.ofq_groupwise_repack(torch.cuda.current_stream().cuda_stream, mat[3].data_ptr(),
+                                            t.data_ptr(), 4, mat[1], mat[2])
+                if st != 0:
+                    raise RuntimeError(f"ofq_groupwise_repack status {st}")
+                tiled[id(mat)] = t
+
+        def launch_tiled(mat, m):
+            name, n, k, w, scale, bias, out = mat
+            st = L.ofq_fused_linear_gq_tiled(torch.cuda.current_stream().cuda_stream,
+                                             x_by_k[k].data_ptr(), tiled[id(mat)].data_ptr(),
+                                             scale.data_ptr(), None, bias.data_ptr(), out.data_ptr(),
+                                             _lib.I8, _lib.F16, 4, 1, 1, 128, m, n, k)
+            if st == 5:  # OFQ_ERR_UNSUPPORTED
+                launch(mat, m)
+                return False
+            if st != 0:
+                raise RuntimeError(f"ofq_fused_linear_gq_tiled status {st}")
+            return True
+        for m in (4, 8):
+            run_t = make_runner(lambda: [launch_tiled(mat, m) for mats in layers for mat in mats])
+            _, wall_t = time_region(run_t, 10, 2)
+            b_m = sum(gemv_bytes(m, n, k) * cnt for _, n, k, cnt in LLAMA7B_LAYER) * args.layers
+            gbps = b_m / (wall_t / 10 * 1e-3) / 1e9
+            by_shape = {}
+            for name, n, k, cnt in LLAMA7B_LAYER:
+                mats_s = [mat for mats in layers for mat in mats if mat[0] == name]
+                served = launch_tiled(mats_s[0], m)
+                run_s = make_runner(lambda: [launch_tiled(mat, m) for mat in mats_s])
+                ev_s, _ = time_region(run_s, 10, 2)
+                by_shape[f"{n}x{k}"] = {"us": round(ev_s * 1e3 / (10 * len(mats_s)), 2),
+                                        "tiled_call_serves_it": served}
+            other[f"decode_w4a16_m{m}_tile_major_weights"] = {
+                "ms_per_step": round(wall_t / 10, 4), "gbps": round(gbps, 1), "by_shape": by_shape,
+                "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+                             "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
+        del tiled
         # per shape: the GEMV alone over all layers for 1, 4 and 8 rows of x, and beside it a
         # kernel that only reads the codes of the same weight tensors (ofq_probe_read; 97% of the
         # bytes the GEMV reads, in one launch per tensor) in the same graph-replay harness: what

@@ -313,6 +313,33 @@ int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, const float*
                         int64_t m, int64_t n, int64_t k, void* workspace, size_t workspace_bytes);
 
 /*
+ * Offline tile-major copy of 4-bit weights for the decode kernels at 2 to 16 rows of x.  No
+ * counterpart in the reference, whose only weight format is the row-major [n, k/2] array of
+ * python/oneflow/test/modules/test_groupwise_quantization.py:26-81; this is the pre-shuffled
+ * variant of that format.  The row-balanced decode kernel gives every block of its grid
+ * rows_per_block consecutive weight rows (a function of n alone) and walks them as 16-row
+ * tiles, a lane (k-slot kb, row r) taking 16 bytes of each 64-byte chunk of its row: in the
+ * row-major array one request of a wave is 16 pieces of 64 bytes.  The copy stores, for block b,
+ * tile t and chunk c, those 64 x 16 bytes as one contiguous KB in lane order,
+ *   tiled[((b * tiles_per_block + t) * (k/128) + c) * 1024 + (kb * 16 + r) * 16 + 0..15]
+ *     = w[b * rows_per_block + 16 t + r][64 c + 16 kb + 0..15],
+ * zeros for rows beyond the block's share.  Scales, zeros and bias keep the reference layout.
+ * ofq_groupwise_repack_bytes: size of the copy (0: no tile-major form for this shape; 4-bit
+ * codes and 128 | k only).  ofq_fused_linear_gq_tiled: ofq_fused_linear_gq on the copy, same
+ * argument meaning, same bits in `out` as the row-major call (tested); OFQ_ERR_UNSUPPORTED
+ * outside fp16, groups of a multiple of 128 along K, m <= 16 and m * k * 2 bytes of x within
+ * LDS -- callers keep the row-major array for everything else (prefill, one row of x, where the
+ * kernel that reads whole rows is the faster one).
+ */
+size_t ofq_groupwise_repack_bytes(int num_bits, int64_t n, int64_t k);
+int ofq_groupwise_repack(void* stream, const void* w, void* w_tiled, int num_bits, int64_t n,
+                         int64_t k);
+int ofq_fused_linear_gq_tiled(void* stream, const void* x, const void* w_tiled,
+                              const void* w_scale, const void* w_zero, const void* b, void* out,
+                              int w_dtype, int t_dtype, int num_bits, int symmetric,
+                              int group_dim, int64_t group_size, int64_t m, int64_t n, int64_t k);
+
+/*
  * Measurement aid, no counterpart in the reference: a kernel that reads `bytes` (rounded down to
  * 16) from buf once, one 16-byte request per lane, and computes nothing.  What it takes is the
  * time below which no kernel that reads those bytes once can finish on this device; a benchmark

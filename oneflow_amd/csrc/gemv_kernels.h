@@ -510,14 +510,19 @@ __device__ __forceinline__ float glu_activation(float v, int act) {
   }
 }
 
+// TILED: w is the tile-major copy ofq_groupwise_repack writes (see w4p_tiled_bytes): the 64-byte
+// chunk c of the 16 rows of the block's tile t is one contiguous KB in the order the lanes take
+// it, [k-slot 0..3][row 0..15][16 bytes], at ((block * tiles_per_block + t) * nchunks + c) * 1024.
+// A request of a wave is then 1 KB of consecutive bytes instead of 16 pieces of 64.
 template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
-         int ZMODE = kZeroNone, bool GLU = false>
+         int ZMODE = kZeroNone, bool GLU = false, bool TILED = false>
 __device__ __forceinline__ void
 gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
               const f16* __restrict__ scale, const f16* __restrict__ zero,
               const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
               int group_size, int cpg_shift, int rows_per_block, GluArgs glu = GluArgs()) {
   static_assert(EXACT || (SIGNED && ZMODE == kZeroNone), "the unrounded path has no zero term");
+  static_assert(!(GLU && TILED), "the tile-major layout serves the plain linear only");
   constexpr int NMAT = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
@@ -541,11 +546,12 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   auto trow_of = [&](int vt) { return (GLU && vt >= ntiles ? vt - ntiles : vt) * 16; };
   auto srow_of = [&](int vt) { return (GLU && vt >= ntiles ? rows_per_block : 0) + trow_of(vt); };
 
-  // LDS: [red ntiles*NWAVES*M*16 f32][scales NMAT*rows_per_block*G halves, padded to 16 B]
+  // LDS: [red NMAT*tiles_per_block*NWAVES*M*16 f32][scales NMAT*rows_per_block*G halves, padded to 16 B]
   //      [zeros, same size (asymmetric only)][corr nchunks*16 f32 (unrounded path only)]
   //      [64 zero bytes][x records M*nchunks*256 B]
   float* red = reinterpret_cast<float*>(smem);
-  const int red_floats = kW4pMaxTiles * NWAVES * M * 16;
+  const int tiles_per_block = (rows_per_block + 15) >> 4;
+  const int red_floats = NMAT * tiles_per_block * NWAVES * M * 16;  // <= kW4pMaxTiles tiles
   const int tile_bytes = (NMAT * rows_per_block * G * 2 + 15) & ~15;
   f16* sl = reinterpret_cast<f16*>(smem + (size_t)red_floats * 4);
   f16* zl = reinterpret_cast<f16*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
@@ -613,6 +619,17 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   // reads one and the same 16 bytes in every lane, a single cached request; lanes past the
   // block's rows re-read its first row (their outputs are never stored).
   auto issue = [&](int tile, int pair, u32x4 (&dst)[2], bool live) {
+    if constexpr (TILED) {
+      const uint8_t* tbase = w + ((int64_t)block * tiles_per_block + tile) * nchunks * 1024
+                             + lane * 16;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int c = 2 * pair + u;
+        const uint8_t* q = tbase + (int64_t)(c < nchunks ? c : 0) * 1024;
+        dst[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(live ? q : w));
+      }
+      return;
+    }
     const int row_l = trow_of(tile) + r;
     const bool ok = row_l < rows_blk;
     const uint8_t* p = (mat_of(tile) ? wbase2 : wbase) + (int64_t)(ok ? row_l : 0) * (K >> 1);
@@ -875,15 +892,14 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
 }
 
 template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
-         int ZMODE = kZeroNone>
+         int ZMODE = kZeroNone, bool TILED = false>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
              const f16* __restrict__ scale, const f16* __restrict__ zero,
              const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
              int group_size, int cpg_shift, int rows_per_block) {
-  gemv_w4p_body<NWAVES, kW4pDepth, EXACT, SIGNED, ZMODE>(blockIdx.x, x, w, scale, zero, bias, out,
-                                                         M, N, K, group_size, cpg_shift,
-                                                         rows_per_block);
+  gemv_w4p_body<NWAVES, kW4pDepth, EXACT, SIGNED, ZMODE, false, TILED>(
+      blockIdx.x, x, w, scale, zero, bias, out, M, N, K, group_size, cpg_shift, rows_per_block);
 }
 
 // Several problems of equal m, k and quantisation in one launch: the grid is the concatenation
@@ -957,7 +973,7 @@ gemv_w4p_f16_glu(const f16* __restrict__ x, const uint8_t* __restrict__ w,
 inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,
                                  bool exact, bool asym, int nmat = 1) {
   const int G = K / group_size;
-  return (size_t)kW4pMaxTiles * nwaves * M * 16 * 4
+  return (size_t)nmat * ((rows_per_block + 15) / 16) * nwaves * M * 16 * 4
          + (size_t)(asym ? 2 : 1) * ((nmat * rows_per_block * G * 2 + 15) & ~15)
          + (exact ? 0 : (size_t)(K >> 7) * 64) + 64 + (size_t)M * (K * 2 + 16);
 }

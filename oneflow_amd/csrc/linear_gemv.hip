@@ -120,10 +120,10 @@ bool w4s_supported(const LinearArgs& a) {
 
 // Row-balanced kernel: grid = a whole number of blocks per CU (or one 16-row tile per block when
 // n is small), rows_per_block <= 64.
-template<int NW, bool EXACT, bool SIGNED, int ZMODE>
+template<int NW, bool EXACT, bool SIGNED, int ZMODE, bool TILED = false>
 int launch_w4p_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block, size_t lds,
                     int cpg_shift) {
-  auto kern = gemv_w4p_f16<NW, 1, EXACT, SIGNED, ZMODE>;
+  auto kern = gemv_w4p_f16<NW, 1, EXACT, SIGNED, ZMODE, TILED>;
   static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
   if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
@@ -142,18 +142,27 @@ bool w4p_supported(const LinearArgs& a) {
          && a.n <= 0x7FFFFFFF - 16 && (a.symmetric || !a.w_signed);
 }
 
-// OFQ_ERR_UNSUPPORTED when the shape does not fit the row-balanced kernel
-int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift) {
+// The row split of the row-balanced kernel, a function of n alone (the tile-major weight copy is
+// laid out by it): one block per CU of a 256-CU part when that keeps a block within 64 rows (a
+// single 16-row tile per block when n is small), else two, else as many 64-row blocks as it takes.
+void w4p_row_split(int64_t n, int64_t* grid_out, int* rows_per_block_out) {
   constexpr int kCUs = 256;
   const int64_t max_rows = 16 * kW4pMaxTiles;
-  // one block per CU when that keeps a block within 64 rows (a single 16-row tile per block
-  // when n is small), else two, else as many 64-row blocks as it takes
   int64_t grid = kCUs;
-  if ((a.n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
-  if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
-  int rpb = (int)((a.n + grid - 1) / grid);
+  if ((n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
+  if ((n + grid - 1) / grid > max_rows) grid = (n + max_rows - 1) / max_rows;
+  int rpb = (int)((n + grid - 1) / grid);
   if (rpb < 16) rpb = 16;
-  grid = (a.n + rpb - 1) / rpb;
+  *grid_out = (n + rpb - 1) / rpb;
+  *rows_per_block_out = rpb;
+}
+
+// OFQ_ERR_UNSUPPORTED when the shape does not fit the row-balanced kernel
+int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift, bool tiled) {
+  constexpr int kCUs = 256;
+  int64_t grid;
+  int rpb;
+  w4p_row_split(a.n, &grid, &rpb);
   const bool two_per_cu = grid > kCUs;
   const int nw = two_per_cu ? 8 : 16;
   if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
@@ -163,18 +172,18 @@ int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift) {
   const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
                                         !a.symmetric);
   if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
-#define OFQ_W4P(NWV)                                                                         \
-  if (nw == NWV) {                                                                           \
+#define OFQ_W4P(NWV, TL)                                                                     \
+  if (nw == NWV && tiled == TL) {                                                            \
     if (!exact)                                                                              \
-      return launch_w4p_inst<NWV, false, true, kZeroNone>(st, a, (int)grid, rpb, lds,        \
-                                                          cpg_shift);                        \
+      return launch_w4p_inst<NWV, false, true, kZeroNone, TL>(st, a, (int)grid, rpb, lds,    \
+                                                              cpg_shift);                    \
     if (a.symmetric)                                                                         \
-      return launch_w4p_inst<NWV, true, false, kZeroSymU>(st, a, (int)grid, rpb, lds,        \
-                                                          cpg_shift);                        \
-    return launch_w4p_inst<NWV, true, false, kZeroAsym>(st, a, (int)grid, rpb, lds,          \
-                                                        cpg_shift);                          \
+      return launch_w4p_inst<NWV, true, false, kZeroSymU, TL>(st, a, (int)grid, rpb, lds,    \
+                                                              cpg_shift);                    \
+    return launch_w4p_inst<NWV, true, false, kZeroAsym, TL>(st, a, (int)grid, rpb, lds,      \
+                                                            cpg_shift);                      \
   }
-  OFQ_W4P(16) OFQ_W4P(8)
+  OFQ_W4P(16, false) OFQ_W4P(8, false) OFQ_W4P(16, true) OFQ_W4P(8, true)
 #undef OFQ_W4P
   return OFQ_ERR_UNSUPPORTED;
 }
@@ -274,7 +283,7 @@ int launch_w4s(hipStream_t st, const LinearArgs& a) {
   // More than one 16-row tile per CU, or an x too large to stage per 16 rows: the row-balanced
   // kernel (equal bytes per block, x staged once per block) is the faster one.
   if (tiles > 256 || !staged) {
-    int rc = launch_w4p(st, a, cpg_shift);
+    int rc = launch_w4p(st, a, cpg_shift, false);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
     // x too large for either staged kernel: the natural-order kernel reads x from L2 once per
     // block, the one below once per 16 rows
@@ -696,7 +705,7 @@ int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
   } else if (w4p_supported(a)) {
     // uint8 container / asymmetric: the row-balanced kernel with the reference's roundings
-    const int rc = launch_w4p(st, a, ilog2_exact(a.group_size / 128));
+    const int rc = launch_w4p(st, a, ilog2_exact(a.group_size / 128), false);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
   }
   if (rows_supported(a)) {
@@ -825,4 +834,115 @@ extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
     }
   }
   return launch_linear_generic(st, a);
+}
+
+// ---- tile-major weight copy -------------------------------------------------------------------
+namespace ofq {
+namespace {
+
+// one lane moves the 16 bytes it will later request: lane (k-slot kb, row r) of chunk c of tile t
+// of block b <- row b * rows_per_block + 16 t + r, bytes [64 c + 16 kb, +16); rows past the
+// block's share (or past n) become zeros
+__global__ void __launch_bounds__(256)
+repack_w4_tiles(const uint8_t* __restrict__ w, uint8_t* __restrict__ tiled, int N, int K,
+                int rows_per_block, int tiles_per_block, int64_t pieces) {
+  const int nchunks = K >> 7;
+  const int row_bytes = K >> 1;
+  for (int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x; p < pieces;
+       p += (int64_t)gridDim.x * 256) {
+    const int lane = (int)(p & 63);
+    const int64_t kb_index = p >> 6;  // (block * tiles_per_block + t) * nchunks + c
+    const int c = (int)(kb_index % nchunks);
+    const int64_t tile_index = kb_index / nchunks;
+    const int t = (int)(tile_index % tiles_per_block);
+    const int64_t b = tile_index / tiles_per_block;
+    const int r = lane & 15, kb = lane >> 4;
+    const int row_l = 16 * t + r;
+    const int64_t row = b * rows_per_block + row_l;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (row_l < rows_per_block && row < N) {
+      v = *reinterpret_cast<const u32x4*>(w + row * row_bytes + c * 64 + kb * 16);
+    }
+    reinterpret_cast<u32x4*>(tiled)[p] = v;
+  }
+}
+
+bool tiled_shape_ok(int num_bits, int64_t n, int64_t k) {
+  return num_bits == 4 && n >= 1 && k >= 128 && k % 128 == 0 && k <= (1 << 20)
+         && n <= 0x7FFFFFFF - 16;
+}
+
+}  // namespace
+}  // namespace ofq
+
+extern "C" size_t ofq_groupwise_repack_bytes(int num_bits, int64_t n, int64_t k) {
+  if (!tiled_shape_ok(num_bits, n, k)) return 0;
+  int64_t grid;
+  int rpb;
+  w4p_row_split(n, &grid, &rpb);
+  return (size_t)grid * (size_t)((rpb + 15) / 16) * 16 * (size_t)(k / 2);
+}
+
+extern "C" int ofq_groupwise_repack(void* stream, const void* w, void* w_tiled, int num_bits,
+                                    int64_t n, int64_t k) {
+  OFQ_RETURN_IF(num_bits != 4 && num_bits != 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(n <= 0 || k <= 0, OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(!tiled_shape_ok(num_bits, n, k), OFQ_ERR_UNSUPPORTED);
+  OFQ_RETURN_IF(w == nullptr || w_tiled == nullptr, OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(!ofq_aligned16(w) || !ofq_aligned16(w_tiled), OFQ_ERR_MISALIGNED);
+  int64_t grid;
+  int rpb;
+  w4p_row_split(n, &grid, &rpb);
+  const int tpb = (rpb + 15) / 16;
+  const int64_t pieces = grid * tpb * (k / 128) * 64;
+  int64_t blocks = (pieces + 255) / 256;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  repack_w4_tiles<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const uint8_t*>(w), static_cast<uint8_t*>(w_tiled), (int)n, (int)k, rpb, tpb,
+      pieces);
+  return ofq_check_launch();
+}
+
+extern "C" int ofq_fused_linear_gq_tiled(void* stream, const void* x, const void* w_tiled,
+                                         const void* w_scale, const void* w_zero, const void* b,
+                                         void* out, int w_dtype, int t_dtype, int num_bits,
+                                         int symmetric, int group_dim, int64_t group_size,
+                                         int64_t m, int64_t n, int64_t k) {
+  OFQ_RETURN_IF(num_bits != 4 && num_bits != 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(group_dim != 0 && group_dim != 1, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(w_dtype != OFQ_U8 && w_dtype != OFQ_I8, OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(!symmetric && w_dtype != OFQ_U8, OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(t_dtype != OFQ_F16 && t_dtype != OFQ_BF16 && t_dtype != OFQ_F32,
+                OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(m < 0 || n < 0 || k <= 0 || group_size <= 0, OFQ_ERR_BAD_SHAPE);
+  if (m == 0 || n == 0) return OFQ_OK;
+  const int64_t group_dim_size = group_dim == 0 ? n : k;
+  OFQ_RETURN_IF(group_size > group_dim_size || group_dim_size % group_size != 0,
+                OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(x == nullptr || w_tiled == nullptr || w_scale == nullptr || out == nullptr,
+                OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF((symmetric != 0) != (w_zero == nullptr), OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(!ofq_aligned16(x) || !ofq_aligned16(w_tiled) || !ofq_aligned16(w_scale)
+                    || !ofq_aligned16(w_zero) || !ofq_aligned16(b) || !ofq_aligned16(out),
+                OFQ_ERR_MISALIGNED);
+  LinearArgs a;
+  a.x = x;
+  a.w = w_tiled;
+  a.scale = w_scale;
+  a.zero = w_zero;
+  a.bias = b;
+  a.out = out;
+  a.t_dtype = t_dtype;
+  a.w_signed = w_dtype == OFQ_I8;
+  a.bits = num_bits;
+  a.symmetric = symmetric != 0;
+  a.group_dim = group_dim;
+  a.group_size = group_size;
+  a.m = m;
+  a.n = n;
+  a.k = k;
+  // what the row-balanced kernel takes: fp16, 4 bits, groups of a multiple of 128 along K, at
+  // most 16 rows of x whose m * k halves fit LDS
+  if (!w4p_supported(a) || !tiled_shape_ok(num_bits, n, k)) return OFQ_ERR_UNSUPPORTED;
+  return launch_w4p(static_cast<hipStream_t>(stream), a, ilog2_exact(a.group_size / 128), true);
 }

@@ -226,6 +226,54 @@ def fused_linear_with_groupwise_quantized_weight(x, w, w_scale, *, w_zero=None, 
     return out
 
 
+def groupwise_repack(w, num_bits=4):
+    """Extension (no counterpart in the reference): the tile-major copy of row-major 4-bit codes
+    ``w`` [n, k/2] that ``fused_linear_with_tiled_groupwise_quantized_weight`` reads, as a flat
+    uint8 / int8 tensor of ``ofq_groupwise_repack_bytes`` elements.  Done once, offline."""
+    _check(w.dim() == 2 and w.dtype in (torch.int8, torch.uint8), "w should be 2-D int8 / uint8 codes")
+    _check(num_bits == 4, "only 4-bit codes have a tile-major form")
+    _require_gpu(w)
+    w = _contig(w)
+    n, k = w.shape[0], w.shape[1] * 2
+    L = _lib.lib()
+    nbytes = L.ofq_groupwise_repack_bytes(num_bits, n, k)
+    _check(nbytes > 0, f"no tile-major form for n={n}, k={k} (k should be a multiple of 128)")
+    tiled = torch.empty(nbytes, dtype=w.dtype, device=w.device)
+    st = L.ofq_groupwise_repack(_stream(w), _ptr(w), _ptr(tiled), num_bits, n, k)
+    _lib.check("ofq_groupwise_repack", st)
+    return tiled
+
+
+def fused_linear_with_tiled_groupwise_quantized_weight(x, w_tiled, w_scale, *, w_zero=None, b=None,
+                                                       num_bits=4, symmetric=True, group_dim=-1,
+                                                       group_size=-1):
+    """``fused_linear_with_groupwise_quantized_weight`` on the copy ``groupwise_repack`` made of
+    ``w`` (n and k are taken from ``w_scale`` and ``x``); the same bits as the row-major call.
+    For up to 16 rows of ``x`` in fp16 with groups of a multiple of 128 along K; raises
+    ``OfqError`` (unsupported) otherwise -- keep the row-major weight for those calls."""
+    _check(x.dim() >= 2 or x.dim() == 1, "x should have at least one dimension")
+    k = x.shape[-1]
+    m = x.numel() // k
+    n = w_scale.shape[0]
+    gd = group_dim if group_dim >= 0 else group_dim + 2
+    _check(gd == 1, "the tile-major copy serves groups along K only")
+    gs = group_size if group_size >= 0 else k
+    _check(w_tiled.dim() == 1 and w_tiled.dtype in (torch.int8, torch.uint8),
+           "w_tiled should be the flat tensor groupwise_repack returns")
+    _check((w_zero is None) == bool(symmetric), "w_zero is given exactly when symmetric is False")
+    _require_gpu(x, w_tiled, w_scale, w_zero, b)
+    L = _lib.lib()
+    _check(w_tiled.numel() == L.ofq_groupwise_repack_bytes(num_bits, n, k),
+           "w_tiled does not have the size of the tile-major copy of an [n, k] weight")
+    x, w_scale, w_zero, b = map(_contig, (x, w_scale, w_zero, b))
+    out = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=x.dtype, device=x.device)
+    st = L.ofq_fused_linear_gq_tiled(_stream(x), _ptr(x), _ptr(w_tiled), _ptr(w_scale),
+                                     _ptr(w_zero), _ptr(b), _ptr(out), _dt(w_tiled), _dt(x),
+                                     num_bits, int(symmetric), gd, gs, m, n, k)
+    _lib.check("ofq_fused_linear_gq_tiled", st)
+    return out
+
+
 def grouped_linear_with_groupwise_quantized_weight(xs, ws, w_scales, *, w_zeros=None, bs=None,
                                                    num_bits=8, symmetric=True, group_dim=-1,
                                                    group_size=-1):

@@ -5,6 +5,7 @@ fake_quantization.py, moving_average_min_max_observer.py:119-153); each forwards
 import torch
 
 from . import functional as _C
+from ._lib import OfqError
 
 
 class MinMaxObserver(torch.nn.Module):
@@ -126,7 +127,26 @@ class QuantizedLinear(torch.nn.Module):
             mod.bias = linear.bias.detach().clone()
         return mod
 
+    def make_decode_copy(self):
+        """Extension: keeps a tile-major copy of the 4-bit weight beside the row-major one
+        (``_C.groupwise_repack``; not part of ``state_dict``).  ``forward`` then reads it for 2 to
+        16 rows of fp16 ``x`` and the row-major weight for everything else."""
+        self.weight_tiled = _C.groupwise_repack(self.weight, self.num_bits)
+        return self
+
     def forward(self, x):
+        tiled = getattr(self, "weight_tiled", None)
+        if tiled is not None and x.dtype == torch.float16 and self.group_size % 128 == 0:
+            m = x.numel() // x.shape[-1]
+            if 2 <= m <= 16:
+                try:
+                    return _C.fused_linear_with_tiled_groupwise_quantized_weight(
+                        x, tiled, self.weight_scale, w_zero=self.weight_zero, b=self.bias,
+                        num_bits=self.num_bits, symmetric=self.symmetric, group_dim=1,
+                        group_size=self.group_size)
+                except OfqError as e:  # e.g. m * k beyond what the kernel stages in LDS
+                    if e.status != 5:  # OFQ_ERR_UNSUPPORTED
+                        raise
         return _C.fused_linear_with_groupwise_quantized_weight(
             x, self.weight, self.weight_scale, w_zero=self.weight_zero, b=self.bias,
             num_bits=self.num_bits, symmetric=self.symmetric, group_dim=1,
