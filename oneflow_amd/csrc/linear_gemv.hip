@@ -37,58 +37,136 @@
 namespace ofq {
 namespace {
 
-// ---- any shape, any grouping: one wave per output element --------------------------------
-template<typename T, int BITS, bool SIGNED>
+// ---- any shape, any grouping: one wave per weight row and up to MT rows of x ----------------
+// The fallback for what the streaming kernels do not take (k off their chunk grid, odd group
+// sizes).  A wave owns weight row n, its lanes walk k (two adjacent codes of a byte per step for
+// 4-bit weights, so that a wave's requests are 64 consecutive bytes of codes), every element is
+// dequantised once with the reference's roundings and meets the rows m0 .. m0+MT-1 of x;
+// indices are 32-bit (the entry point bounds m*k, n*k and m*n by 2^31).
+template<typename T, int BITS, bool SIGNED, int MT>
 __global__ void __launch_bounds__(256)
 linear_generic(const typename TT<T>::storage* __restrict__ x, const uint8_t* __restrict__ w,
                const typename TT<T>::storage* __restrict__ scale,
                const typename TT<T>::storage* __restrict__ zero,
                const typename TT<T>::storage* __restrict__ bias,
-               typename TT<T>::storage* __restrict__ out, int64_t M, int64_t N, int64_t K,
-               int group_dim, int64_t group_size, int symmetric) {
+               typename TT<T>::storage* __restrict__ out, int M, int N, int K, int group_dim,
+               int group_size, int symmetric) {
+  constexpr int E = BITS == 4 ? 2 : 1;
   const int lane = threadIdx.x & 63;
-  const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int64_t m = blockIdx.y;
+  const int n = (int)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int m0 = (int)blockIdx.y * MT;
   if (n >= N) return;
-  const int64_t G = group_dim == 1 ? K / group_size : 0;
-  float acc = 0.f;
-  for (int64_t k = lane; k < K; k += 64) {
-    const int64_t si = group_dim == 1 ? n * G + k / group_size : (n / group_size) * K + k;
-    const float s = TT<T>::load(scale + si);
-    float z;
-    if (!symmetric) {
-      z = TT<T>::load(zero + si);
-    } else if (SIGNED) {
-      z = 0.f;
-    } else {
-      z = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * s);
-    }
-    const float q = (float)code_at<BITS, SIGNED>(w, n * K + k);
+  float acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = 0.f;
+  auto zero_term = [&](float s, int si) -> float {
+    if (!symmetric) return TT<T>::load(zero + si);
+    if (SIGNED) return 0.f;
+    return TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * s);
+  };
+  auto element = [&](int k, float s, float z) {
+    const float q = (float)code_at<BITS, SIGNED>(w, (int64_t)n * K + k);
     const float wv = TT<T>::round(TT<T>::round(q * s) + z);
-    acc = __builtin_fmaf(TT<T>::load(x + m * K + k), wv, acc);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      if (m0 + i < M) acc[i] = __builtin_fmaf(TT<T>::load(x + (m0 + i) * K + k), wv, acc[i]);
+    }
+  };
+  if (group_dim == 1) {
+    // group by group: scale and zero are the same for the whole wave (one broadcast request per
+    // group instead of one per element, no division per element).  Items (group, step of 64*E
+    // elements within it) are taken four at a time with all their requests issued before any is
+    // used: a wave walks its row alone, and one memory round trip per item would bound it.
+    const int G = K / group_size;
+    const int spg = (group_size + 64 * E - 1) / (64 * E);  // steps per group
+    const int items = G * spg;
+    constexpr int B = 4;
+    for (int it0 = 0; it0 < items; it0 += B) {
+      float sv[B], zv[B];
+      int kk[B][E];
+      bool ok[B][E];
+      int code[B][E];
+      float xv[B][E][MT];
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int it = it0 + b < items ? it0 + b : items - 1;
+        const int gi = it / spg;  // (the same for every lane)
+        const int st = it - gi * spg;
+        const int si = n * G + gi;
+        sv[b] = TT<T>::load(scale + si);
+        zv[b] = zero_term(sv[b], si);
+        const int kend = (gi + 1) * group_size;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const int k = gi * group_size + st * 64 * E + lane * E + e;
+          ok[b][e] = it0 + b < items && k < kend;
+          kk[b][e] = ok[b][e] ? k : 0;
+          code[b][e] = code_at<BITS, SIGNED>(w, (int64_t)n * K + kk[b][e]);
+#pragma unroll
+          for (int i = 0; i < MT; ++i) {
+            xv[b][e][i] = TT<T>::load(x + (m0 + i < M ? m0 + i : m0) * K + kk[b][e]);
+          }
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const float wv = TT<T>::round(TT<T>::round((float)code[b][e] * sv[b]) + zv[b]);
+#pragma unroll
+          for (int i = 0; i < MT; ++i) {
+            if (ok[b][e] && m0 + i < M) acc[i] = __builtin_fmaf(xv[b][e][i], wv, acc[i]);
+          }
+        }
+      }
+    }
+  } else {
+    const int srow = (n / group_size) * K;
+    for (int k0 = lane * E; k0 < K; k0 += 64 * E) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const int k = k0 + e;
+        if (k < K) {
+          const float s = TT<T>::load(scale + srow + k);
+          element(k, s, zero_term(s, srow + k));
+        }
+      }
+    }
   }
-  acc = wave_reduce(acc, OpSum());
-  if (lane == 0) {
-    if (bias != nullptr) acc += TT<T>::load(bias + n);
-    TT<T>::store(out + m * N + n, acc);
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const float sum = wave_reduce(acc[i], OpSum());
+    if (lane == 0 && m0 + i < M) {
+      float r = sum;
+      if (bias != nullptr) r += TT<T>::load(bias + n);
+      TT<T>::store(out + (m0 + i) * N + n, r);
+    }
   }
 }
 
 template<typename T>
 int launch_generic_t(hipStream_t st, const LinearArgs& a) {
   typedef typename TT<T>::storage S;
-  dim3 grid((unsigned)((a.n + 3) / 4), (unsigned)a.m);
-#define OFQ_G(B, SG)                                                                         \
-  if (a.bits == B && a.w_signed == SG) {                                                     \
-    linear_generic<T, B, SG><<<grid, 256, 0, st>>>(                                          \
+  if (a.group_size > 0x7FFFFFFF) return OFQ_ERR_UNSUPPORTED;
+#define OFQ_G1(B, SG, MTV)                                                                   \
+  {                                                                                          \
+    dim3 grid((unsigned)((a.n + 3) / 4), (unsigned)((a.m + MTV - 1) / MTV));                 \
+    linear_generic<T, B, SG, MTV><<<grid, 256, 0, st>>>(                                     \
         static_cast<const S*>(a.x), static_cast<const uint8_t*>(a.w),                        \
         static_cast<const S*>(a.scale), static_cast<const S*>(a.zero),                       \
-        static_cast<const S*>(a.bias), static_cast<S*>(a.out), a.m, a.n, a.k, a.group_dim,   \
-        a.group_size, a.symmetric ? 1 : 0);                                                  \
+        static_cast<const S*>(a.bias), static_cast<S*>(a.out), (int)a.m, (int)a.n, (int)a.k, \
+        a.group_dim, (int)a.group_size, a.symmetric ? 1 : 0);                                \
     return ofq_check_launch();                                                               \
+  }
+#define OFQ_G(B, SG)                                                                         \
+  if (a.bits == B && a.w_signed == SG) {                                                     \
+    if (a.m == 1) OFQ_G1(B, SG, 1)                                                           \
+    if (a.m <= 4) OFQ_G1(B, SG, 4)                                                           \
+    OFQ_G1(B, SG, 8)                                                                         \
   }
   OFQ_G(4, false) OFQ_G(4, true) OFQ_G(8, false) OFQ_G(8, true)
 #undef OFQ_G
+#undef OFQ_G1
   return OFQ_ERR_UNSUPPORTED;
 }
 
