@@ -117,6 +117,133 @@ matmul_quant_rows(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
   }
 }
 
+// ---- 1 to 4 rows of a: a wave owns whole rows of b -------------------------------------------
+// With so few rows the matrix core adds nothing and its operand layout costs (a request of 16
+// rows x 64 bytes instead of whole rows, a fold across the waves that split K).  Here lane l
+// holds bytes [h * 1024 + 16 l, +16) of every row of a in registers (h < H = ceil(k / 1024)),
+// a wave walks the rows w, w + NW, .. of the block's share of b with the requests of two rows in
+// flight, meets each row with v_dot4_i32_i8 (exact int32) and sums across the lanes; no LDS, no
+// barrier.  Same int32 sums and the same epilogue as the other paths, hence the same bits.
+__device__ __forceinline__ int wave_sum_i32(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+  v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+  v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, false);  // row_half_mirror
+  v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, false);  // row_mirror
+  return (__builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16))
+         + (__builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48));
+}
+
+template<typename T, int NW, int H, int MR>
+__global__ void __launch_bounds__(NW * 64)
+matmul_quant_wave_rows(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                       const float* __restrict__ a_scale, const float* __restrict__ b_scale,
+                       const typename TT<T>::storage* __restrict__ bias,
+                       typename TT<T>::storage* __restrict__ out, int M, int N, int K,
+                       int rows_per_block) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int row0 = blockIdx.x * rows_per_block;
+  int rows_blk = N - row0;
+  if (rows_blk > rows_per_block) rows_blk = rows_per_block;
+  const int nr = rows_blk > wave ? (rows_blk - wave + NW - 1) / NW : 0;  // rows of this wave
+  bool valid[H];
+  uint32_t voff[H];
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    valid[h] = h * 1024 + lane * 16 < K;
+    voff[h] = valid[h] ? (uint32_t)(h * 1024 + lane * 16) : 0u;
+  }
+  const uint8_t* bblk = b + (int64_t)row0 * K;
+  i32x4 wq[2][H];
+  auto issue = [&](int i, int buf) {
+    const bool live = i < nr;  // the same for every lane
+    const uint8_t* rowp = bblk + (size_t)(live ? wave + i * NW : 0) * K;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      wq[buf][h] = __builtin_nontemporal_load(
+          reinterpret_cast<const i32x4*>(rowp + (live ? voff[h] : 0u)));
+    }
+  };
+  // the rows of a first (they come from L2 and every row of b needs them), then two rows of b
+  i32x4 av[MR][H];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const uint8_t* arow = a + (size_t)(m < M ? m : 0) * K;
+#pragma unroll
+    for (int h = 0; h < H; ++h) av[m][h] = *reinterpret_cast<const i32x4*>(arow + voff[h]);
+  }
+  issue(0, 0);
+  issue(1, 1);
+  const float sa = a_scale[0];
+  auto finish = [&](int i, int buf) {
+    const int n = row0 + wave + i * NW;
+    const float sb = b_scale[n];
+    float bv = 0.f;
+    if (bias != nullptr) bv = TT<T>::load(bias + n);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      int acc = 0;
+#pragma unroll
+      for (int h = 0; h < H; ++h) {
+        int part = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          part = __builtin_amdgcn_sdot4(av[m][h][j], wq[buf][h][j], part, false);
+        }
+        acc += valid[h] ? part : 0;
+      }
+      const int sum = wave_sum_i32(acc);
+      if (lane == 0 && m < M) {
+        float v = (float)sum * (sa * sb);
+        if (bias != nullptr) v = v + bv;
+        TT<T>::store(out + (int64_t)m * N + n, v);
+      }
+    }
+  };
+  for (int i = 0; i < nr; i += 2) {
+    finish(i, 0);
+    issue(i + 2, 0);
+    if (i + 1 < nr) finish(i + 1, 1);
+    issue(i + 3, 1);
+  }
+}
+
+template<typename T, int H, int MR>
+int launch_wave_rows_inst(hipStream_t st, const uint8_t* a, const uint8_t* b, const float* a_scale,
+                          const float* b_scale, const void* bias, void* out, int m, int64_t n,
+                          int64_t k) {
+  typedef typename TT<T>::storage S;
+  constexpr int NW = 16;
+  // one block per CU, two from 128 rows per block on; a wave then walks its rows two ahead
+  int64_t grid = 256;
+  if ((n + grid - 1) / grid >= 128) grid = 512;
+  int rpb = (int)((n + grid - 1) / grid);
+  if (rpb < NW) rpb = NW;
+  grid = (n + rpb - 1) / rpb;
+  matmul_quant_wave_rows<T, NW, H, MR><<<(unsigned)grid, NW * 64, 0, st>>>(
+      a, b, a_scale, b_scale, static_cast<const S*>(bias), static_cast<S*>(out), m, (int)n, (int)k,
+      rpb);
+  return ofq_check_launch();
+}
+
+// m <= 4, 16 | k <= 8192 (the rows of a are held in registers: 4 H m of them)
+template<typename T>
+int launch_wave_rows(hipStream_t st, const uint8_t* a, const uint8_t* b, const float* a_scale,
+                     const float* b_scale, const void* bias, void* out, int m, int64_t n,
+                     int64_t k) {
+  const int h = (int)((k + 1023) / 1024);
+#define OFQ_WR(HV)                                                                             \
+  case HV:                                                                                     \
+    if (m == 1) return launch_wave_rows_inst<T, HV, 1>(st, a, b, a_scale, b_scale, bias, out, m, n, k); \
+    if (m == 2) return launch_wave_rows_inst<T, HV, 2>(st, a, b, a_scale, b_scale, bias, out, m, n, k); \
+    return launch_wave_rows_inst<T, HV, 4>(st, a, b, a_scale, b_scale, bias, out, m, n, k);
+  switch (h) {
+    OFQ_WR(1) OFQ_WR(2) OFQ_WR(3) OFQ_WR(4) OFQ_WR(5) OFQ_WR(6) OFQ_WR(7) OFQ_WR(8)
+    default: return OFQ_ERR_UNSUPPORTED;
+  }
+#undef OFQ_WR
+}
+
 template<typename T, int NW, int MT>
 int launch_inst(hipStream_t st, const uint8_t* a, const uint8_t* b, const float* a_scale,
                 const float* b_scale, const void* bias, void* out, int m, int64_t n, int64_t k,
@@ -136,6 +263,10 @@ int launch_inst(hipStream_t st, const uint8_t* a, const uint8_t* b, const float*
 template<typename T>
 int launch_part(hipStream_t st, const uint8_t* a, const uint8_t* b, const float* a_scale,
                 const float* b_scale, const void* bias, void* out, int m, int64_t n, int64_t k) {
+  if (m <= 4 && k <= 8192 && k % 16 == 0) {
+    const int rc = launch_wave_rows<T>(st, a, b, a_scale, b_scale, bias, out, m, n, k);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   constexpr int kCUs = 256;
   const int64_t max_rows = 16 * kI8MaxTiles;
   int64_t grid = kCUs;
