@@ -20,15 +20,19 @@
 namespace ofq {
 namespace {
 
-template<bool SYM, bool SIGNED, int BITS>
-__device__ __forceinline__ int quant_code(float v, float sc, float mn) {
+// HALF: v is the value of an fp16 element and `recip` = 1 / sc (IEEE division, once per group):
+// the symmetric quotient v / sc is then the twice-corrected product of div_of_half_value, bit for
+// bit the division (sc = absmax / 7 or / 127 of fp16 values lies far inside its range).  With 11
+// instructions per division this kernel was bound by its arithmetic, not by HBM.
+template<bool SYM, bool SIGNED, int BITS, bool HALF = false>
+__device__ __forceinline__ int quant_code(float v, float sc, float mn, float recip = 0.f) {
   constexpr float kSignedMax = (float)((1 << (BITS - 1)) - 1);
   constexpr float kOffset = SYM ? (SIGNED ? 0.0f : kSignedMax) : 0.0f;
   float r;
   if (sc == 0.0f) {
     r = kOffset;
   } else if (SYM) {
-    const float d = v / sc;
+    const float d = HALF ? div_of_half_value(v, sc, recip) : v / sc;
     r = __builtin_rintf(d + kOffset);
   } else {
     const float d = v - mn;
@@ -52,8 +56,9 @@ quantize_pack_rows(const typename TT<T>::storage* __restrict__ x, uint8_t* __res
                    typename TT<T>::storage* __restrict__ zero, int64_t total_groups, int L) {
   typedef typename TT<T>::storage S;
   const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t grp = slot / L;
-  const int l = (int)(slot - grp * L);
+  const int lshift = __builtin_ctz((unsigned)L);  // L is a power of two
+  const int64_t grp = slot >> lshift;
+  const int l = (int)(slot & (L - 1));
   const bool live = grp < total_groups;
   const int64_t base = (live ? grp : 0) * (int64_t)L * 8 + (int64_t)l * 8;
   S raw[8];
@@ -83,8 +88,19 @@ quantize_pack_rows(const typename TT<T>::storage* __restrict__ x, uint8_t* __res
     if (!SYM) TT<T>::store(&zero[grp], mn);
   }
   uint32_t c[8];
+  constexpr bool kHalf = SYM && TT<T>::dtype == OFQ_F16;
+  // (an infinite element makes the scale infinite: that group keeps the division)
+  const bool fast = kHalf && sc > 0.0f && sc <= 0x1p60f;
+  if (fast) {
+    const float recip = 1.0f / sc;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) c[e] = (uint32_t)quant_code<SYM, SIGNED, BITS>(v[e], sc, mn);
+    for (int e = 0; e < 8; ++e) {
+      c[e] = (uint32_t)quant_code<SYM, SIGNED, BITS, true>(v[e], sc, mn, recip);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) c[e] = (uint32_t)quant_code<SYM, SIGNED, BITS>(v[e], sc, mn);
+  }
   if (BITS == 8) {
     u32x2 w;
     w[0] = (c[0] & 0xFF) | ((c[1] & 0xFF) << 8) | ((c[2] & 0xFF) << 16) | (c[3] << 24);

@@ -43,6 +43,32 @@ def test_bit_exact_against_the_oracle(bits, symmetric, signed, t, n, k, group_di
         assert np.array_equal(O.to_f32(z), O.to_f32(zr))  # by value: the sign of a zero minimum is free
 
 
+@pytest.mark.parametrize("bits,signed", [(4, True), (4, False), (8, True), (8, False)])
+def test_symmetric_fp16_groups_of_arbitrary_bit_patterns(bits, signed):
+    """Symmetric quantisation of fp16 weights divides by the group scale through a corrected
+    multiplication with its reciprocal.  Groups of random fp16 bit patterns (every exponent,
+    subnormals, both zeros, the largest values; infinities in a few groups, which keep the
+    division) against the oracle's `x / scale`, bit for bit."""
+    rng = np.random.default_rng(bits * 2 + signed)
+    bits16 = rng.integers(0, 65536, size=(6000, 128)).astype(np.uint16)
+    x = bits16.view(np.float16)
+    x[np.isnan(x)] = np.float16(0.0)
+    keep_inf = np.zeros(x.shape[0], bool)
+    keep_inf[:5] = True
+    x[np.isinf(x) & ~keep_inf[:, None]] = np.float16(65504.0)
+    # narrow the spread inside most groups so that the codes are not all 0 or the extremes
+    for r in range(100, x.shape[0]):
+        e = int(rng.integers(1, 28))
+        x[r] = (x[r].view(np.uint16) & np.uint16(0x83FF) | np.uint16(e << 10)).view(np.float16)
+    x[5] = np.float16(0.0)
+    x[6, :4] = np.array([6e-8, -6e-8, 1.2e-7, 0.0], np.float16)
+    qr, sr, _ = O.groupwise_quantize(x, bits, True, 1, 128, signed)
+    q, s, _ = _run(x, bits, True, 1, 128, signed)
+    rows = ~keep_inf  # (a group with an infinite element has scale inf and codes from 0 * nan)
+    assert np.array_equal(q.view(np.uint8)[rows], qr.view(np.uint8)[rows])
+    assert np.array_equal(s.view(np.uint16)[rows], sr.view(np.uint16)[rows])
+
+
 def test_constant_and_zero_groups_and_ties():
     """scale 0 groups get the code of value 0; exact .5 quotients round to even."""
     x = np.zeros((4, 64), np.float32)
