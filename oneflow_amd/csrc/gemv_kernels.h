@@ -199,6 +199,13 @@ gemv_f16_mfma(const f16* __restrict__ x, const uint8_t* __restrict__ w,
 // ---------------------------------------------------------------------------------------------
 constexpr int kGemvMaxUnits = 4;  // 32-byte x units a thread may stage
 
+// (2 v * ceil(2^31 / d)) >> 32 == v / d for v < 2^17 and 1 <= d <= 2^13: the row of x a staging
+// unit belongs to, without an integer division per unit
+__device__ __forceinline__ uint32_t row_of_inv(int d) { return 0x7FFFFFFFu / (uint32_t)d + 1u; }
+__device__ __forceinline__ int row_of(int v, uint32_t inv) {
+  return (int)__umulhi((uint32_t)v << 1, inv);
+}
+
 // x of one 16-k unit (two 128-bit words, natural order) -> low-nibble operand and high-nibble
 // operand, the latter divided by 16
 __device__ __forceinline__ void permute_unit(const u32x4 a, const u32x4 b, u32x4& lo, u32x4& hi) {
@@ -251,6 +258,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
   const int nchunks = K >> 7;
+  const uint32_t inv_chunks = row_of_inv(nchunks);
   const int npairs = (nchunks + 1) >> 1;
   const int G = K / group_size;
   // LDS: [reduction NWAVES*64*4 f32][scale tile 16*G halves, padded to 16 B]
@@ -339,7 +347,8 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
         // unit u = (m, chunk, j): j -> kb = j/2, t = 2*(j%2) + {0: lo, 1: hi}; 32 bytes per unit
         // rows of x are skewed by 16 bytes each: the lanes of different m that read the same
         // chunk then hit different LDS bank groups (their records are a multiple of 256 B apart)
-        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32 + ((u >> 3) / nchunks) * 16);
+        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32
+                                              + row_of(u >> 3, inv_chunks) * 16);
         dst[0] = lo;
         dst[1] = hi;
       }
@@ -349,7 +358,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
       cpart += __shfl_xor(cpart, 2, 64);
       cpart += __shfl_xor(cpart, 4, 64);
       if (u < nunits && (u & 7) == 0) {
-        const int m = (u >> 3) / nchunks;
+        const int m = row_of(u >> 3, inv_chunks);
         const int c = (u >> 3) - m * nchunks;
         corr_l[c * 16 + m] = -cpart;  // negated: it seeds the MFMA accumulator
       }
@@ -527,6 +536,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
   const int nchunks = K >> 7;
+  const uint32_t inv_chunks = row_of_inv(nchunks);
   const int npairs = (nchunks + 1) >> 1;
   const int G = K / group_size;
   const int tid = threadIdx.x;
@@ -717,7 +727,8 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
       if (u < nunits) {
         // rows of x are skewed by 16 bytes each: the lanes of different m that read the same
         // chunk then hit different LDS bank groups (their records are a multiple of 256 B apart)
-        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32 + ((u >> 3) / nchunks) * 16);
+        u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32
+                                              + row_of(u >> 3, inv_chunks) * 16);
         dst[0] = permute_x4(xu[i][0]);
         dst[1] = permute_x4(xu[i][1]);
       }
@@ -726,7 +737,8 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     if (u < nunits) {
       u32x4 lo, hi;
       permute_unit(xu[i][0], xu[i][1], lo, hi);
-      u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32 + ((u >> 3) / nchunks) * 16);
+      u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32
+                                            + row_of(u >> 3, inv_chunks) * 16);
       dst[0] = lo;
       dst[1] = hi;
     }
@@ -735,7 +747,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     cpart += __shfl_xor(cpart, 2, 64);
     cpart += __shfl_xor(cpart, 4, 64);
     if (u < nunits && (u & 7) == 0) {
-      const int m = (u >> 3) / nchunks;
+      const int m = row_of(u >> 3, inv_chunks);
       const int c = (u >> 3) - m * nchunks;
       corr_l[c * 16 + m] = -cpart;
     }
