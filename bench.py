@@ -697,10 +697,13 @@ def secondary(L, _lib, torch, dev, args):
                                   "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBPS, 4)}}
     del wsrc, qo
 
-    # ---- decode through the natural-order kernel: bf16 W4 asymmetric g=128 and fp16 W8 g=64, --
-    # m = 1 and 16, gate/up shape; 8 weight sets cycled so that no launch finds its codes in cache
+    # ---- decode of the variants whose w~ is formed with the reference's roundings: W4 with a zero
+    # point g=128 in fp16 and bf16, fp16 W8 g=64; m = 1 (a wave owns whole rows) and 16 (MFMA,
+    # natural element order), gate/up shape; 8 weight sets cycled so that no launch finds its
+    # codes in cache
     n, k = 11008, 4096
-    for tag, tcode, tdt, bits, g in (("bf16_w4_asym_g128", _lib.BF16, torch.bfloat16, 4, 128),
+    for tag, tcode, tdt, bits, g in (("f16_w4_asym_g128", _lib.F16, torch.float16, 4, 128),
+                                     ("bf16_w4_asym_g128", _lib.BF16, torch.bfloat16, 4, 128),
                                      ("f16_w8_asym_g64", _lib.F16, torch.float16, 8, 64)):
         reps = 8
         ws = [torch.randint(0, 256, (n, k * bits // 8), dtype=torch.uint8, device=dev) for _ in range(reps)]

@@ -778,6 +778,10 @@ int launch_gemv_wq(hipStream_t st, const LinearArgs& a) {
     const int rc = launch_gemv_m1(st, a);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;
   }
+  if (gemv_m1_any_supported(a)) {
+    const int rc = launch_gemv_m1_any(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   if (w4s_supported(a)) {
     const int rc = launch_w4s(st, a);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;

@@ -38,6 +38,12 @@ int launch_gemv_m1(hipStream_t st, const LinearArgs& a);
 int launch_gemv_m1_grouped(hipStream_t st, const LinearArgs* problems, int count);
 int launch_gemv_m1_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act);
 
+// m = 1, fp16 or bf16, 4- or 8-bit codes in either container, symmetric or with a zero point,
+// groups along K of a power-of-two size: the same row-per-wave structure with the reference's
+// roundings of w~.
+bool gemv_m1_any_supported(const LinearArgs& a);
+int launch_gemv_m1_any(hipStream_t st, const LinearArgs& a);
+
 // Skinny-M (m <= 16) MFMA GEMV that streams the weights once.
 bool gemv_wq_supported(const LinearArgs& a);
 int launch_gemv_wq(hipStream_t st, const LinearArgs& a);

@@ -216,6 +216,64 @@ def test_decode_natural_order_kernel(m, n, k, group_size, num_bits, t):
         assert (np.abs(gf - rf) <= np.maximum(H.ulp_of(rf, t), 2e-4) * (1 + 1e-9)).all() or shortcut
 
 
+@pytest.mark.parametrize("n,k,group_size", [
+    (4096, 4096, 128), (11008, 4096, 128), (4096, 11008, 128), (5000, 256, 32), (4099, 1536, 64),
+    (40000, 2048, 256), (300, 8192, 1024), (130, 5120, 64), (17, 14336, 128), (9000, 416, 32),
+    (1, 64, 32)])
+@pytest.mark.parametrize("num_bits", [4, 8])
+@pytest.mark.parametrize("t", ["bf16", "f16"])
+def test_decode_single_row_of_x_every_variant(n, k, group_size, num_bits, t):
+    """m = 1 for both 16-bit types, both code widths and all three code variants: rows of 1 to
+    8 KB of codes (and beyond, where another kernel takes over), rows that end inside a KB, one
+    row per wave and many rows per wave, n not a multiple of the block's waves, groups from one
+    lane's share of a row up to 1024."""
+    rng = np.random.Generator(np.random.PCG64(n * 31 + k + num_bits))
+    x = H.as_T(rng.standard_normal((1, k)).astype(np.float32), t)
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), t)
+    for symmetric, qdt in VARIANTS:
+        w, scale, zero = H.quantize_groupwise(wf, num_bits, symmetric, 1, group_size, qdt, t)
+        ref = O.fused_linear(x, w, scale, zero, b, num_bits, symmetric, 1, group_size)
+        got = _run(x, w, scale, zero, b, num_bits, symmetric, 1, group_size)
+        what = f"{t} b{num_bits} n={n} k={k} g={group_size} {symmetric} {qdt}"
+        r, e = H.assert_linear_parity(got, ref, t, what)
+        shortcut = t == "f16" and num_bits == 4 and qdt == np.int8 and group_size % 128 == 0
+        # w~ formed with the oracle's roundings: what is left is the order of the fp32 sum, which
+        # moves a few per cent of the outputs by one rounding of T (5e-4 relative in fp16)
+        assert r < (3e-3 if t == "bf16" else 5e-4 if shortcut else 2e-4), (r, what)
+        gf, rf = O.to_f32(got).astype(np.float64), O.to_f32(ref).astype(np.float64)
+        assert (np.abs(gf - rf) <= np.maximum(H.ulp_of(rf, t), 2e-4) * (1 + 1e-9)).all() or shortcut
+    # exact integer case through the same path (closed form, no oracle): scales 1, integer zero
+    # points, x in {-1, 0, 1} with so few non-zeros that every sum is an integer T represents
+    kk, nn = min(k, 2048), min(n, 600)
+    gsz = min(group_size, kk)
+    ones = H.as_T(np.ones((nn, kk // gsz), dtype=np.float32), t)
+    for symmetric, qdt in VARIANTS:
+        offset_127 = num_bits == 8 and symmetric and qdt == np.uint8  # w~ = code - 127
+        nnz = {"f16": 16 if offset_127 else 128, "bf16": 2 if offset_127 else 16}[t]
+        xi = np.zeros((1, kk), dtype=np.float32)
+        pos = rng.choice(kk, size=min(nnz, kk), replace=False)
+        xi[0, pos] = rng.choice([-1.0, 1.0], size=pos.size)
+        zero, zp = None, 0
+        if qdt == np.int8:
+            codes = rng.integers(-8, 8, size=(nn, kk)).astype(np.int8)
+            values = codes.astype(np.int64)
+        else:
+            codes = rng.integers(0, 16, size=(nn, kk)).astype(np.uint8)
+            values = codes.astype(np.int64)
+            if symmetric:
+                values = values - ((1 << (num_bits - 1)) - 1)
+            else:
+                zp = rng.integers(-8, 1, size=(nn, kk // gsz))
+                values = values + np.repeat(zp, gsz, axis=1)
+                zero = H.as_T(zp.astype(np.float32), t)
+        w = H.pack_int4(codes) if num_bits == 4 else codes
+        exact = xi.astype(np.int64) @ values.T
+        assert np.abs(exact).max() < (256 if t == "bf16" else 2048)
+        got = _run(H.as_T(xi, t), w, ones, zero, None, num_bits, symmetric, 1, gsz)
+        assert np.array_equal(O.to_f32(got).astype(np.int64), exact), (t, num_bits, symmetric, qdt)
+
+
 def test_decode_m_invariance_and_integer_case():
     """Row i of an m=8 call agrees with the m=1 call on that row (the two batch sizes take
     different code paths: x staged in LDS or not, so agreement is to fp32-accumulation noise, at
