@@ -613,8 +613,18 @@ def secondary(L, _lib, torch, dev, args):
                                                wsc.data_ptr(), None, o.data_ptr(), _lib.F16, m, n, k),
                             "matmul_quant"))
     tops = 2.0 * m * n * k / (us * 1e-6) / 1e12
+
+    # yardstick: the vendor int8 GEMM (torch._int_mm: int8 x int8 -> int32, without the scaling to
+    # fp16 that this op does in its epilogue) on the same operands
+    def vendor_int8(a_i8, w_i8):
+        try:
+            return round(timeit(lambda: torch._int_mm(a_i8, w_i8.t())), 2)
+        except Exception as e:  # the yardstick must not take the benchmark down
+            print(f"bench.py: vendor int8 GEMM yardstick failed: {e}", file=sys.stderr)
+            return None
     out["matmul_quant_i8_m2048"] = {
         "us": round(us, 2), "tops": round(tops, 1),
+        "us_vendor_gemm_int8_to_int32_same_operands": vendor_int8(a8[0], wq),
         "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": MFMA_PEAK_TFLOPS["i8"],
                      "unit": "TOP/s", "frac": round(tops / MFMA_PEAK_TFLOPS["i8"], 4)}}
     # a batch of 256 rows on a square weight: 32 x 1 tiles of 128 columns, so K is cut into slices
@@ -632,6 +642,7 @@ def secondary(L, _lib, torch, dev, args):
     tops = 2.0 * mm * nn * k / (us * 1e-6) / 1e12
     out["matmul_quant_i8_m256_4096x4096"] = {
         "us": round(us, 2), "tops": round(tops, 1), "workspace_bytes": int(mq_ws_bytes),
+        "us_vendor_gemm_int8_to_int32_same_operands": vendor_int8(a8[0][:mm], wsq),
         "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": MFMA_PEAK_TFLOPS["i8"],
                      "unit": "TOP/s", "frac": round(tops / MFMA_PEAK_TFLOPS["i8"], 4)}}
     del wsq, osq, mq_ws
