@@ -128,7 +128,7 @@ def main():
                     launch(mat)
 
     # the same step with the block's neighbouring ops fused: q/k/v as one grouped launch,
-    # o, gate|up with the SiLU gating as one launch, down: 5 launches per layer, not 7 (+ gating)
+    # o, gate|up with the SiLU gating as one launch, down: 4 launches per layer, not 7 (+ gating)
     glu_y = torch.empty((max(M, 8), 11008), dtype=torch.float16, device=dev)
     vp = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
     i64 = lambda v: (ctypes.c_int64 * len(v))(*v)
@@ -272,7 +272,7 @@ def main():
             gbps = (b_m + args.layers * m * 11008 * 2) / (wall_f / 10 * 1e-3) / 1e9
             other[f"decode_w4a16_m{m}_grouped_qkv_and_glu"] = {
                 "ms_per_step": round(wall_f / 10, 4), "gbps": round(gbps, 1),
-                "launches_per_step": 5 * args.layers,
+                "launches_per_step": 4 * args.layers,
                 "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                              "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
         # the offline tile-major copy of the weights (ofq_groupwise_repack) for 4 and 8 rows of x;

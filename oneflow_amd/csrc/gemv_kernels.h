@@ -523,8 +523,11 @@ __device__ __forceinline__ float glu_activation(float v, int act) {
 // chunk c of the 16 rows of the block's tile t is one contiguous KB in the order the lanes take
 // it, [k-slot 0..3][row 0..15][16 bytes], at ((block * tiles_per_block + t) * nchunks + c) * 1024.
 // A request of a wave is then 1 KB of consecutive bytes instead of 16 pieces of 64.
+// PH = 2: m * k is more than LDS holds at once (8 rows of 11008): the chunk pairs of a row are
+// walked in two halves, each with its own staging of x; the x of the second half is requested
+// while the first is worked on, and the sums of a (tile, wave) add up in `red`.
 template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
-         int ZMODE = kZeroNone, bool GLU = false, bool TILED = false>
+         int ZMODE = kZeroNone, bool GLU = false, bool TILED = false, int PH = 1>
 __device__ __forceinline__ void
 gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
               const f16* __restrict__ scale, const f16* __restrict__ zero,
@@ -532,12 +535,17 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
               int group_size, int cpg_shift, int rows_per_block, GluArgs glu = GluArgs()) {
   static_assert(EXACT || (SIGNED && ZMODE == kZeroNone), "the unrounded path has no zero term");
   static_assert(!(GLU && TILED), "the tile-major layout serves the plain linear only");
+  static_assert(PH == 1 || PH == 2, "one staging of x or two");
   constexpr int NMAT = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
   const int nchunks = K >> 7;
-  const uint32_t inv_chunks = row_of_inv(nchunks);
-  const int npairs = (nchunks + 1) >> 1;
+  const int npairs_all = (nchunks + 1) >> 1;
+  // the phase being worked on: its chunk pairs [., + npairs), its chunks [cbeg, cbeg + ncs)
+  int npairs = PH == 2 ? (npairs_all + 1) >> 1 : npairs_all;
+  int cbeg = 0;
+  int ncs = PH == 2 ? 2 * npairs : nchunks;
+  uint32_t inv_chunks = row_of_inv(ncs);
   const int G = K / group_size;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -558,7 +566,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
 
   // LDS: [red NMAT*tiles_per_block*NWAVES*M*16 f32][scales NMAT*rows_per_block*G halves, padded to 16 B]
   //      [zeros, same size (asymmetric only)][corr nchunks*16 f32 (unrounded path only)]
-  //      [64 zero bytes][x records M*nchunks*256 B]
+  //      [64 zero bytes][x records M*ncs*256 B, ncs = chunks of a phase]
   float* red = reinterpret_cast<float*>(smem);
   const int tiles_per_block = (rows_per_block + 15) >> 4;
   const int red_floats = NMAT * tiles_per_block * NWAVES * M * 16;  // <= kW4pMaxTiles tiles
@@ -571,18 +579,29 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   uint8_t* xs = zrec + 64;
 
   // ---- requests that feed LDS go out first ----------------------------------------------------
-  const int nunits = (M * K) >> 4;
+  int nunits = M * ncs * 8;  // 32-byte units of x of the phase, row by row
   u32x4 xu[kGemvMaxUnits][2];
+  // unit u of a phase whose rows hold `cs` chunks from chunk `c0` on
+  auto request_x = [&](int units, int cs, int c0, uint32_t inv) {
 #pragma unroll
-  for (int i = 0; i < kGemvMaxUnits; ++i) {
-    if (wave * 64 + i * NT >= nunits) break;
-    const int u = tid + i * NT;
-    if (u < nunits) {
-      const u32x4* src = reinterpret_cast<const u32x4*>(x + (int64_t)u * 16);
-      xu[i][0] = src[0];
-      xu[i][1] = src[1];
+    for (int i = 0; i < kGemvMaxUnits; ++i) {
+      if (wave * 64 + i * NT >= units) break;
+      const int u = tid + i * NT;
+      if (u < units) {
+        const u32x4* src;
+        if constexpr (PH == 1) {
+          src = reinterpret_cast<const u32x4*>(x + (int64_t)u * 16);
+        } else {
+          const int m = row_of(u >> 3, inv);
+          const int cl = (u >> 3) - m * cs;
+          src = reinterpret_cast<const u32x4*>(x + ((int64_t)(m * nchunks + c0 + cl) * 8 + (u & 7)) * 16);
+        }
+        xu[i][0] = src[0];
+        xu[i][1] = src[1];
+      }
     }
-  }
+  };
+  request_x(nunits, ncs, cbeg, inv_chunks);
   // the scales of the block's rows are one contiguous piece
   const int tile_halves = rows_blk * G;
   const f16* stile = scale + (int64_t)row0 * G;
@@ -634,7 +653,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
                              + lane * 16;
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const int c = 2 * pair + u;
+        const int c = cbeg + 2 * pair + u;
         const uint8_t* q = tbase + (int64_t)(c < nchunks ? c : 0) * 1024;
         dst[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(live ? q : w));
       }
@@ -645,7 +664,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     const uint8_t* p = (mat_of(tile) ? wbase2 : wbase) + (int64_t)(ok ? row_l : 0) * (K >> 1);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int c = 2 * pair + u;
+      const int c = cbeg + 2 * pair + u;
       const uint8_t* q = p + (c < nchunks ? c : 0) * 64;
       dst[u] = __builtin_nontemporal_load(
           reinterpret_cast<const u32x4*>(live ? q : w + (int64_t)row0 * (K >> 1)));
@@ -660,18 +679,21 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   };
   int it_tile[kW4pDepth], it_pair[kW4pDepth];
   u32x4 wq[kW4pDepth][2];
+  auto first_items = [&]() {
 #pragma unroll
-  for (int d = 0; d < kW4pDepth; ++d) {
-    it_tile[d] = 0;
-    it_pair[d] = wave + d * NWAVES;
-    advance(it_tile[d], it_pair[d], 0);
-    // unconditional, so that the wait counts stay exact: a slot without an item reads one and
-    // the same 16 bytes in every lane (a single cached request)
-    {
-      const bool live = it_tile[d] < nvt;
-      issue(live ? it_tile[d] : 0, live ? it_pair[d] : 0, wq[d], live);
+    for (int d = 0; d < kW4pDepth; ++d) {
+      it_tile[d] = 0;
+      it_pair[d] = wave + d * NWAVES;
+      advance(it_tile[d], it_pair[d], 0);
+      // unconditional, so that the wait counts stay exact: a slot without an item reads one and
+      // the same 16 bytes in every lane (a single cached request)
+      {
+        const bool live = it_tile[d] < nvt;
+        issue(live ? it_tile[d] : 0, live ? it_pair[d] : 0, wq[d], live);
+      }
     }
-  }
+  };
+  first_items();
 
   // ---- fill LDS -------------------------------------------------------------------------------
   for (int e = tid; e < red_floats / 4; e += NT) reinterpret_cast<f32x4*>(red)[e] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -718,51 +740,65 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     }
   }
   if (tid < 16) reinterpret_cast<uint32_t*>(zrec)[tid] = 0u;
+  // x of the phase (held in xu) -> records in LDS
+  auto stage_x = [&]() {
 #pragma unroll
-  for (int i = 0; i < kGemvMaxUnits; ++i) {
-    if (wave * 64 + i * NT >= nunits) break;
-    const int u = tid + i * NT;
-    if (EXACT) {
-      // one record per code word: x in the pair order of unpack4_pairs
+    for (int i = 0; i < kGemvMaxUnits; ++i) {
+      if (wave * 64 + i * NT >= nunits) break;
+      const int u = tid + i * NT;
+      if (EXACT) {
+        // one record per code word: x in the pair order of unpack4_pairs
+        if (u < nunits) {
+          // rows of x are skewed by 16 bytes each: the lanes of different m that read the same
+          // chunk then hit different LDS bank groups (their records are a multiple of 256 B apart)
+          u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32
+                                                + row_of(u >> 3, inv_chunks) * 16);
+          dst[0] = permute_x4(xu[i][0]);
+          dst[1] = permute_x4(xu[i][1]);
+        }
+        continue;
+      }
       if (u < nunits) {
-        // rows of x are skewed by 16 bytes each: the lanes of different m that read the same
-        // chunk then hit different LDS bank groups (their records are a multiple of 256 B apart)
+        u32x4 lo, hi;
+        permute_unit(xu[i][0], xu[i][1], lo, hi);
         u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32
                                               + row_of(u >> 3, inv_chunks) * 16);
-        dst[0] = permute_x4(xu[i][0]);
-        dst[1] = permute_x4(xu[i][1]);
+        dst[0] = lo;
+        dst[1] = hi;
       }
-      continue;
+      float cpart = u < nunits ? unit_corr_of(xu[i][0], xu[i][1]) : 0.f;
+      cpart += __shfl_xor(cpart, 1, 64);
+      cpart += __shfl_xor(cpart, 2, 64);
+      cpart += __shfl_xor(cpart, 4, 64);
+      if (u < nunits && (u & 7) == 0) {
+        const int m = row_of(u >> 3, inv_chunks);
+        const int c = (u >> 3) - m * ncs;  // chunk within the phase
+        corr_l[c * 16 + m] = -cpart;
+      }
     }
-    if (u < nunits) {
-      u32x4 lo, hi;
-      permute_unit(xu[i][0], xu[i][1], lo, hi);
-      u32x4* dst = reinterpret_cast<u32x4*>(xs + (size_t)u * 32
-                                            + row_of(u >> 3, inv_chunks) * 16);
-      dst[0] = lo;
-      dst[1] = hi;
-    }
-    float cpart = u < nunits ? unit_corr_of(xu[i][0], xu[i][1]) : 0.f;
-    cpart += __shfl_xor(cpart, 1, 64);
-    cpart += __shfl_xor(cpart, 2, 64);
-    cpart += __shfl_xor(cpart, 4, 64);
-    if (u < nunits && (u & 7) == 0) {
-      const int m = row_of(u >> 3, inv_chunks);
-      const int c = (u >> 3) - m * nchunks;
-      corr_l[c * 16 + m] = -cpart;
-    }
+  };
+  stage_x();
+  if constexpr (PH == 2) {
+    // the second half's x goes out now; it is staged when the first half has been walked
+    const int ncs2 = nchunks - ncs;
+    request_x(M * ncs2 * 8, ncs2, ncs, row_of_inv(ncs2 > 0 ? ncs2 : 1));
   }
   __syncthreads();
 
-  const uint8_t* xrec = has_x ? xs + (size_t)r * (nchunks * 256 + 16) + kb * 64 : zrec;
+  const uint8_t* xrec = has_x ? xs + (size_t)r * (ncs * 256 + 16) + kb * 64 : zrec;
   const int xrec_stride = has_x ? 256 : 0;
+  bool add_to_red = false;  // second phase: the (tile, wave) slots already hold the first's sums
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
   f32x4 total1 = {0.f, 0.f, 0.f, 0.f};  // second accumulator of the exact path
   auto flush = [&](int t) {
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int m = 4 * kb + v;
-      if (m < M) red[((t * NWAVES + wave) * M + m) * 16 + r] = total[v] + total1[v];
+      if (m < M) {
+        float* slot = red + ((t * NWAVES + wave) * M + m) * 16 + r;
+        const float sum = total[v] + total1[v];
+        *slot = PH == 2 && add_to_red ? *slot + sum : sum;
+      }
     }
     total1 = f32x4{0.f, 0.f, 0.f, 0.f};
   };
@@ -772,9 +808,10 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     const f16* slr = sl + (srow_of(tile) + r) * G;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int c = 2 * pair + u;
+      const int cl = 2 * pair + u;  // chunk within the phase: the index of its x record
+      const int c = cbeg + cl;
       if (c < nchunks) {
-        const u32x4* xp = reinterpret_cast<const u32x4*>(xrec + c * xrec_stride);
+        const u32x4* xp = reinterpret_cast<const u32x4*>(xrec + cl * xrec_stride);
         u32x4 xa[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) xa[t] = xp[t];
@@ -809,7 +846,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
           continue;
         }
         const float s = (float)slr[grp];
-        f32x4 acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
+        f32x4 acc = *reinterpret_cast<const f32x4*>(corr_l + cl * 16 + kb * 4);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const uint32_t w0 = wq[d][u][2 * h];
@@ -840,40 +877,62 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
       total = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   };
-  // items of this wave: wave, wave + NWAVES, ... < nitems
-  const int nitems = nvt * npairs;
-  int left = nitems > wave ? (nitems - wave + NWAVES - 1) / NWAVES : 0;
-  // steady state: every slot is consumed and refilled unconditionally, so the compiler's wait
-  // before each slot is exact (the 2 * (kW4pDepth - 1) younger loads stay in flight)
-  while (left >= 2 * kW4pDepth) {
+  auto walk = [&]() {
+    // items of this wave: wave, wave + NWAVES, ... < nitems
+    const int nitems = nvt * npairs;
+    int left = nitems > wave ? (nitems - wave + NWAVES - 1) / NWAVES : 0;
+    // steady state: every slot is consumed and refilled unconditionally, so the compiler's wait
+    // before each slot is exact (the 2 * (kW4pDepth - 1) younger loads stay in flight)
+    while (left >= 2 * kW4pDepth) {
+#pragma unroll
+      for (int d = 0; d < kW4pDepth; ++d) {
+        const int tile = it_tile[d], pair = it_pair[d];
+        process(d, tile, pair);
+        advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
+        issue(it_tile[d], it_pair[d], wq[d], true);
+        next_or_flush(d, tile);
+      }
+      left -= kW4pDepth;
+    }
+    // tail: fewer than 2 * kW4pDepth items are left; at most kW4pDepth - 1 refills
 #pragma unroll
     for (int d = 0; d < kW4pDepth; ++d) {
       const int tile = it_tile[d], pair = it_pair[d];
-      process(d, tile, pair);
-      advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
-      issue(it_tile[d], it_pair[d], wq[d], true);
-      next_or_flush(d, tile);
+      if (d < left) {
+        process(d, tile, pair);
+        advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
+        if (d + kW4pDepth < left) issue(it_tile[d], it_pair[d], wq[d], true);
+        next_or_flush(d, tile);
+      }
     }
-    left -= kW4pDepth;
-  }
-  // tail: fewer than 2 * kW4pDepth items are left; at most kW4pDepth - 1 refills
 #pragma unroll
-  for (int d = 0; d < kW4pDepth; ++d) {
-    const int tile = it_tile[d], pair = it_pair[d];
-    if (d < left) {
-      process(d, tile, pair);
-      advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
-      if (d + kW4pDepth < left) issue(it_tile[d], it_pair[d], wq[d], true);
-      next_or_flush(d, tile);
+    for (int d = 0; d < kW4pDepth - 1; ++d) {
+      const int tile = it_tile[d], pair = it_pair[d];
+      if (d + kW4pDepth < left) {
+        process(d, tile, pair);
+        advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
+        next_or_flush(d, tile);
+      }
     }
-  }
-#pragma unroll
-  for (int d = 0; d < kW4pDepth - 1; ++d) {
-    const int tile = it_tile[d], pair = it_pair[d];
-    if (d + kW4pDepth < left) {
-      process(d, tile, pair);
-      advance(it_tile[d], it_pair[d], kW4pDepth * NWAVES);
-      next_or_flush(d, tile);
+  };
+  walk();
+  if constexpr (PH == 2) {
+    // second half of the chunk pairs: its first items are requested before the barrier behind
+    // which the x records are replaced
+    cbeg = ncs;
+    npairs = npairs_all - npairs;
+    ncs = nchunks - ncs;
+    if (ncs > 0) {
+      inv_chunks = row_of_inv(ncs);
+      nunits = M * ncs * 8;
+      add_to_red = true;
+      total = f32x4{0.f, 0.f, 0.f, 0.f};
+      first_items();
+      __syncthreads();  // every wave has read its last x record and correction of the first half
+      stage_x();
+      __syncthreads();
+      xrec = has_x ? xs + (size_t)r * (ncs * 256 + 16) + kb * 64 : zrec;
+      walk();
     }
   }
   __syncthreads();
@@ -904,13 +963,13 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
 }
 
 template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
-         int ZMODE = kZeroNone, bool TILED = false>
+         int ZMODE = kZeroNone, bool TILED = false, int PH = 1>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_w4p_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
              const f16* __restrict__ scale, const f16* __restrict__ zero,
              const f16* __restrict__ bias, f16* __restrict__ out, int M, int N, int K,
              int group_size, int cpg_shift, int rows_per_block) {
-  gemv_w4p_body<NWAVES, kW4pDepth, EXACT, SIGNED, ZMODE, false, TILED>(
+  gemv_w4p_body<NWAVES, kW4pDepth, EXACT, SIGNED, ZMODE, false, TILED, PH>(
       blockIdx.x, x, w, scale, zero, bias, out, M, N, K, group_size, cpg_shift, rows_per_block);
 }
 
@@ -982,12 +1041,20 @@ gemv_w4p_f16_glu(const f16* __restrict__ x, const uint8_t* __restrict__ w,
                                                        rows_per_block, glu);
 }
 
+// chunks of x a block holds at once: all of a row's, or (two stagings) the larger half of its
+// chunk pairs
+inline int gemv_w4p_phase_chunks(int K, int phases) {
+  const int nchunks = K >> 7;
+  return phases == 2 ? 2 * ((((nchunks + 1) >> 1) + 1) >> 1) : nchunks;
+}
+
 inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,
-                                 bool exact, bool asym, int nmat = 1) {
+                                 bool exact, bool asym, int nmat = 1, int phases = 1) {
   const int G = K / group_size;
   return (size_t)nmat * ((rows_per_block + 15) / 16) * nwaves * M * 16 * 4
          + (size_t)(asym ? 2 : 1) * ((nmat * rows_per_block * G * 2 + 15) & ~15)
-         + (exact ? 0 : (size_t)(K >> 7) * 64) + 64 + (size_t)M * (K * 2 + 16);
+         + (exact ? 0 : (size_t)(K >> 7) * 64) + 64
+         + (size_t)M * (gemv_w4p_phase_chunks(K, phases) * 256 + 16);
 }
 
 // dynamic LDS bytes of gemv_w4s_f16

@@ -198,10 +198,10 @@ bool w4s_supported(const LinearArgs& a) {
 
 // Row-balanced kernel: grid = a whole number of blocks per CU (or one 16-row tile per block when
 // n is small), rows_per_block <= 64.
-template<int NW, bool EXACT, bool SIGNED, int ZMODE, bool TILED = false>
+template<int NW, bool EXACT, bool SIGNED, int ZMODE, bool TILED = false, int PH = 1>
 int launch_w4p_inst(hipStream_t st, const LinearArgs& a, int grid, int rows_per_block, size_t lds,
                     int cpg_shift) {
-  auto kern = gemv_w4p_f16<NW, 1, EXACT, SIGNED, ZMODE, TILED>;
+  auto kern = gemv_w4p_f16<NW, 1, EXACT, SIGNED, ZMODE, TILED, PH>;
   static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
   if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
@@ -243,13 +243,25 @@ int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift, bool tiled) {
   w4p_row_split(a.n, &grid, &rpb);
   const bool two_per_cu = grid > kCUs;
   const int nw = two_per_cu ? 8 : 16;
-  if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
   // one thread folds one output of the block
   if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) return OFQ_ERR_UNSUPPORTED;
   const bool exact = !(a.symmetric && a.w_signed);
-  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
-                                        !a.symmetric);
-  if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
+  const size_t lds_cap = (two_per_cu ? 80u : 160u) * 1024u;
+  size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                                  !a.symmetric);
+  if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) {
+    // m * k beyond one staging of x: two stagings, each of half the chunk pairs of a row
+    // (the symmetric int8-container case on one block per CU only)
+    if (exact || nw != 16) return OFQ_ERR_UNSUPPORTED;
+    const int64_t half_units = a.m * gemv_w4p_phase_chunks((int)a.k, 2) * 8;
+    lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                             !a.symmetric, 1, 2);
+    if (half_units > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) return OFQ_ERR_UNSUPPORTED;
+    return tiled ? launch_w4p_inst<16, false, true, kZeroNone, true, 2>(st, a, (int)grid, rpb, lds,
+                                                                        cpg_shift)
+                 : launch_w4p_inst<16, false, true, kZeroNone, false, 2>(st, a, (int)grid, rpb,
+                                                                         lds, cpg_shift);
+  }
 #define OFQ_W4P(NWV, TL)                                                                     \
   if (nw == NWV && tiled == TL) {                                                            \
     if (!exact)                                                                              \

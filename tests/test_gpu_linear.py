@@ -168,11 +168,14 @@ def test_decode_w4a16_row_balanced_shapes(m, n, k, container):
     assert np.array_equal(got.astype(np.int64), exact)
 
 
-@pytest.mark.parametrize("m,n,k", [(16, 80, 8192), (8, 48, 11008), (13, 4096, 4096)])
+@pytest.mark.parametrize("m,n,k", [(16, 80, 8192), (8, 48, 11008), (13, 4096, 4096),
+                                   (8, 100, 11136), (5, 300, 16512), (6, 4096, 11008),
+                                   (16, 5000, 8192), (8, 11008, 11008), (7, 33, 22016)])
 @pytest.mark.parametrize("symmetric,qdt", VARIANTS)
 def test_decode_w4a16_large_x(m, n, k, symmetric, qdt):
-    """m * k too large for x to be staged in LDS: the kernels that read x from L2 per chunk, for
-    all three code variants."""
+    """m * k too large for x to be staged in LDS at once, for all three code variants: x staged
+    in two halves of a row's chunk pairs (symmetric int8 container; an odd number of chunks, one
+    and several tiles per block, two blocks per CU) or read from L2 per chunk."""
     rng = np.random.Generator(np.random.PCG64(m * 131 + n))
     x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), "f16")
     wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
@@ -182,6 +185,18 @@ def test_decode_w4a16_large_x(m, n, k, symmetric, qdt):
     got = _run(x, w, scale, zero, b, 4, symmetric, 1, 128)
     r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k}")
     assert r < (5e-4 if (symmetric and qdt == np.int8) else 1e-4)
+    if symmetric and qdt == np.int8:
+        # exact integer case through the same path (closed form, no oracle): scales 1, sparse
+        # small-integer x, every sum an integer below 2048
+        nn = min(n, 700)
+        xi = rng.integers(-2, 3, size=(m, k)).astype(np.float16)
+        xi[rng.random((m, k)) < 0.9] = 0
+        codes = rng.integers(-8, 8, size=(nn, k)).astype(np.int8)
+        ones = np.ones((nn, k // 128), dtype=np.float16)
+        exact = xi.astype(np.int64) @ codes.astype(np.int64).T
+        assert np.abs(exact).max() < 2048
+        got = _run(xi, H.pack_int4(codes), ones, None, None, 4, True, 1, 128)
+        assert np.array_equal(got.astype(np.int64), exact)
 
 
 @pytest.mark.parametrize("m,n,k,group_size", [
