@@ -1030,15 +1030,15 @@ gemv_w4p_f16_grouped(GemvGroup g, int M, int K, int group_size, int cpg_shift,
 }
 
 // two weights of equal shape (hidden state, gate), every block the same rows of both
-template<int NWAVES, bool EXACT, bool SIGNED, int ZMODE>
+template<int NWAVES, bool EXACT, bool SIGNED, int ZMODE, int PH = 1>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_w4p_f16_glu(const f16* __restrict__ x, const uint8_t* __restrict__ w,
                  const f16* __restrict__ scale, const f16* __restrict__ zero,
                  const f16* __restrict__ bias, f16* __restrict__ out, GluArgs glu, int M, int N,
                  int K, int group_size, int cpg_shift, int rows_per_block) {
-  gemv_w4p_body<NWAVES, 1, EXACT, SIGNED, ZMODE, true>(blockIdx.x, x, w, scale, zero, bias, out,
-                                                       M, N, K, group_size, cpg_shift,
-                                                       rows_per_block, glu);
+  gemv_w4p_body<NWAVES, 1, EXACT, SIGNED, ZMODE, true, false, PH>(
+      blockIdx.x, x, w, scale, zero, bias, out, M, N, K, group_size, cpg_shift, rows_per_block,
+      glu);
 }
 
 // chunks of x a block holds at once: all of a row's, or (two stagings) the larger half of its

@@ -654,10 +654,10 @@ int launch_w4p_grouped(hipStream_t st, const LinearArgs* pr, int count) {
   return OFQ_ERR_UNSUPPORTED;
 }
 
-template<int NW, bool EXACT, bool SIGNED, int ZMODE>
+template<int NW, bool EXACT, bool SIGNED, int ZMODE, int PH = 1>
 int launch_w4p_glu_inst(hipStream_t st, const LinearArgs& a, const GluArgs& glu, int grid,
                         int rows_per_block, size_t lds) {
-  auto kern = gemv_w4p_f16_glu<NW, EXACT, SIGNED, ZMODE>;
+  auto kern = gemv_w4p_f16_glu<NW, EXACT, SIGNED, ZMODE, PH>;
   static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
   if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
@@ -689,12 +689,19 @@ int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, vo
   grid = (a.n + rpb - 1) / rpb;
   const bool two_per_cu = grid > kCUs;
   const int nw = two_per_cu ? 8 : 16;
-  if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
   if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) return OFQ_ERR_UNSUPPORTED;
   const bool exact = !(a.symmetric && a.w_signed);
-  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
-                                        !a.symmetric, 2);
-  if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
+  const size_t lds_cap = (two_per_cu ? 80u : 160u) * 1024u;
+  size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                                  !a.symmetric, 2);
+  // x beyond one staging (8 rows of 4096 next to two blocks' worth of sums): two stagings
+  const bool two_stagings = a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap;
+  if (two_stagings) {
+    lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact, !a.symmetric,
+                             2, 2);
+    const int64_t half_units = a.m * gemv_w4p_phase_chunks((int)a.k, 2) * 8;
+    if (half_units > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) return OFQ_ERR_UNSUPPORTED;
+  }
   GluArgs glu;
   glu.w2 = static_cast<const uint8_t*>(g.w);
   glu.scale2 = static_cast<const f16*>(g.scale);
@@ -703,15 +710,18 @@ int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, vo
   glu.out2 = static_cast<f16*>(g.out);
   glu.y = static_cast<f16*>(y);
   glu.act = act;
-#define OFQ_W4PGLU(NWV)                                                                        \
-  if (nw == NWV) {                                                                             \
+#define OFQ_W4PGLU(NWV, PHV)                                                                   \
+  if (nw == NWV && two_stagings == (PHV == 2)) {                                               \
     if (!exact)                                                                                \
-      return launch_w4p_glu_inst<NWV, false, true, kZeroNone>(st, a, glu, (int)grid, rpb, lds); \
+      return launch_w4p_glu_inst<NWV, false, true, kZeroNone, PHV>(st, a, glu, (int)grid, rpb, \
+                                                                   lds);                       \
     if (a.symmetric)                                                                           \
-      return launch_w4p_glu_inst<NWV, true, false, kZeroSymU>(st, a, glu, (int)grid, rpb, lds); \
-    return launch_w4p_glu_inst<NWV, true, false, kZeroAsym>(st, a, glu, (int)grid, rpb, lds);  \
+      return launch_w4p_glu_inst<NWV, true, false, kZeroSymU, PHV>(st, a, glu, (int)grid, rpb, \
+                                                                   lds);                       \
+    return launch_w4p_glu_inst<NWV, true, false, kZeroAsym, PHV>(st, a, glu, (int)grid, rpb,   \
+                                                                 lds);                         \
   }
-  OFQ_W4PGLU(16) OFQ_W4PGLU(8)
+  OFQ_W4PGLU(16, 1) OFQ_W4PGLU(8, 1) OFQ_W4PGLU(16, 2) OFQ_W4PGLU(8, 2)
 #undef OFQ_W4PGLU
   return OFQ_ERR_UNSUPPORTED;
 }
