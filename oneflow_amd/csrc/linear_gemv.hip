@@ -679,29 +679,42 @@ int launch_gemv_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, vo
   if (!w4p_supported(a) || !w4p_supported(g)) return OFQ_ERR_UNSUPPORTED;
   if (g.n != a.n || g.k != a.k || g.m != a.m || g.x != a.x) return OFQ_ERR_UNSUPPORTED;
   constexpr int kCUs = 256;
-  // a block walks the same rows of both weights: half the tiles per weight
-  const int64_t max_rows = 16 * (kW4pMaxTiles / 2);
-  int64_t grid = kCUs;
-  if ((a.n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
-  if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
-  int rpb = (int)((a.n + grid - 1) / grid);
-  if (rpb < 16) rpb = 16;
-  grid = (a.n + rpb - 1) / rpb;
-  const bool two_per_cu = grid > kCUs;
-  const int nw = two_per_cu ? 8 : 16;
-  if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) return OFQ_ERR_UNSUPPORTED;
   const bool exact = !(a.symmetric && a.w_signed);
-  const size_t lds_cap = (two_per_cu ? 80u : 160u) * 1024u;
-  size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
-                                  !a.symmetric, 2);
-  // x beyond one staging (8 rows of 4096 next to two blocks' worth of sums): two stagings
-  const bool two_stagings = a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap;
-  if (two_stagings) {
+  // A block walks the same rows of both weights.  First choice: up to 64 rows of each per block,
+  // so that n = 11008 is one block of 16 waves per CU as in the plain linear (43 rows, three
+  // tiles per weight); that doubles the per-(tile, wave) sums in LDS, so with many rows of x it
+  // may not fit, and then a block owns at most 32 rows of each weight (two blocks per CU).
+  int64_t grid = 0;
+  int rpb = 0, nw = 0;
+  size_t lds = 0;
+  bool two_stagings = false, fits = false;
+  for (int tiles_per_weight = kW4pMaxTiles; tiles_per_weight >= kW4pMaxTiles / 2 && !fits;
+       tiles_per_weight -= kW4pMaxTiles / 2) {
+    const int64_t max_rows = 16 * tiles_per_weight;
+    grid = kCUs;
+    if ((a.n + grid - 1) / grid > max_rows) grid = 2 * kCUs;
+    if ((a.n + grid - 1) / grid > max_rows) grid = (a.n + max_rows - 1) / max_rows;
+    rpb = (int)((a.n + grid - 1) / grid);
+    if (rpb < 16) rpb = 16;
+    grid = (a.n + rpb - 1) / rpb;
+    const bool two_per_cu = grid > kCUs;
+    nw = two_per_cu ? 8 : 16;
+    // one thread folds one output of the block (per weight)
+    if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) continue;
+    const size_t lds_cap = (two_per_cu ? 80u : 160u) * 1024u;
     lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact, !a.symmetric,
-                             2, 2);
-    const int64_t half_units = a.m * gemv_w4p_phase_chunks((int)a.k, 2) * 8;
-    if (half_units > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) return OFQ_ERR_UNSUPPORTED;
+                             2);
+    // x beyond one staging (8 rows of 4096 next to the sums of two weights): two stagings
+    two_stagings = a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap;
+    if (two_stagings) {
+      lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                               !a.symmetric, 2, 2);
+      const int64_t half_units = a.m * gemv_w4p_phase_chunks((int)a.k, 2) * 8;
+      if (half_units > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) continue;
+    }
+    fits = true;
   }
+  if (!fits) return OFQ_ERR_UNSUPPORTED;
   GluArgs glu;
   glu.w2 = static_cast<const uint8_t*>(g.w);
   glu.scale2 = static_cast<const f16*>(g.scale);
