@@ -84,15 +84,15 @@ gemv_rows_body(int block, const uint16_t* __restrict__ x, const uint8_t* __restr
   const int ntiles = (rows_blk + 15) >> 4;
   const bool has_x = r < M;
 
-  // LDS: [red kRowsMaxTiles*NWAVES*M*16 f32][scales rows_per_block*G, padded to 16 B]
-  //      [zeros, same size (asymmetric only)][64 zero bytes][x: M rows of K*2+16 bytes (STAGED)]
-  float* red = reinterpret_cast<float*>(smem);
-  const int red_floats = kRowsMaxTiles * NWAVES * M * 16;
+  // LDS: [scales rows_per_block*G, padded to 16 B][zeros, same size (asymmetric only)]
+  //      [64 zero bytes][x: M rows of K*2+16 bytes (STAGED)]; the sums of the waves
+  //      (tiles*NWAVES*M*16 f32) take the place of x once every wave has walked its pairs
   const int tile_bytes = (rows_per_block * G * 2 + 15) & ~15;
-  uint16_t* sl = reinterpret_cast<uint16_t*>(smem + (size_t)red_floats * 4);
+  uint16_t* sl = reinterpret_cast<uint16_t*>(smem);
   uint16_t* zl = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
   uint8_t* zrec = reinterpret_cast<uint8_t*>(sl) + (ZMODE == kZeroAsym ? 2 : 1) * tile_bytes;
   uint8_t* xs = zrec + 64;
+  float* red = reinterpret_cast<float*>(xs);
   const int x_pitch = K * 2 + 16;  // rows skewed by 16 bytes: lanes of different m reading the
                                    // same k hit different LDS bank groups
 
@@ -250,7 +250,8 @@ gemv_rows_body(int block, const uint16_t* __restrict__ x, const uint8_t* __restr
     }
     pair += NWAVES;
   }
-  // every wave writes its sums of every tile (zeros when it had no pair)
+  // every wave writes its sums of every tile (zeros when it had no pair) where x was
+  if (STAGED) __syncthreads();  // ... which every wave has finished reading
 #pragma unroll
   for (int t = 0; t < kRowsMaxTiles; ++t) {
     if (t < ntiles) {
@@ -620,9 +621,10 @@ inline size_t gemv_rows_mt_lds_bytes(int nwaves, int mt, int K, int group_size,
 inline size_t gemv_rows_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,
                                   bool asym, bool staged) {
   const int G = K / group_size;
-  return (size_t)kRowsMaxTiles * nwaves * M * 16 * 4
-         + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15) + 64
-         + (staged ? (size_t)M * (K * 2 + 16) : 0);
+  const size_t red = (size_t)((rows_per_block + 15) / 16) * nwaves * M * 16 * 4;
+  const size_t xrows = staged ? (size_t)M * (K * 2 + 16) : 0;
+  return (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15) + 64
+         + (red > xrows ? red : xrows);
 }
 
 }  // namespace

@@ -345,6 +345,14 @@ int launch_rows(hipStream_t st, const LinearArgs& a) {
   const size_t cap = (two_per_cu ? 80u : 160u) * 1024u;
   // x goes to LDS when it fits there and in the staging registers; else it is read from L2
   bool staged = a.m * a.k / 8 <= (int64_t)kRowsMaxUnits * nw * 64;
+  // bf16 with 4-bit codes and a zero term is bound by the vector unit (eleven instructions per
+  // element pair); staging more than 64 KB of x adds to that (11008 x 4096 at 16 rows: 16.0
+  // against 15.2 us), where the 8-bit and the symmetric variants gain from it (fp16 W8: 14.2
+  // against 15.3 us)
+  if (a.t_dtype == OFQ_BF16 && a.bits == 4 && !(a.symmetric && a.w_signed)
+      && a.m * a.k * 2 > 65536) {
+    staged = false;
+  }
   size_t lds = gemv_rows_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb,
                                    !a.symmetric, staged);
   if (staged && lds > cap) {
