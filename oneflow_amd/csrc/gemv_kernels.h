@@ -1017,12 +1017,12 @@ __device__ __forceinline__ GemvProblem select_problem(const GemvGroup& g, int bl
   return pr;
 }
 
-template<int NWAVES, bool EXACT, bool SIGNED, int ZMODE>
+template<int NWAVES, bool EXACT, bool SIGNED, int ZMODE, int PH = 1>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_w4p_f16_grouped(GemvGroup g, int M, int K, int group_size, int cpg_shift,
                      int rows_per_block) {
   const GemvProblem pr = select_problem(g, (int)blockIdx.x);
-  gemv_w4p_body<NWAVES, 1, EXACT, SIGNED, ZMODE>(
+  gemv_w4p_body<NWAVES, 1, EXACT, SIGNED, ZMODE, false, false, PH>(
       (int)blockIdx.x - pr.first_block, static_cast<const f16*>(pr.x), pr.w,
       static_cast<const f16*>(pr.scale), static_cast<const f16*>(pr.zero),
       static_cast<const f16*>(pr.bias), static_cast<f16*>(pr.out), M, pr.N, K, group_size,

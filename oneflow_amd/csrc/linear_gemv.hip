@@ -579,10 +579,10 @@ int launch_rows_grouped_t(hipStream_t st, const LinearArgs& a, const GemvGroup& 
   return OFQ_ERR_UNSUPPORTED;
 }
 
-template<int NW, bool EXACT, bool SIGNED, int ZMODE>
+template<int NW, bool EXACT, bool SIGNED, int ZMODE, int PH = 1>
 int launch_w4p_grouped_inst(hipStream_t st, const GemvGroup& g, int grid, int m, int k,
                             int group_size, int rows_per_block, size_t lds) {
-  auto kern = gemv_w4p_f16_grouped<NW, EXACT, SIGNED, ZMODE>;
+  auto kern = gemv_w4p_f16_grouped<NW, EXACT, SIGNED, ZMODE, PH>;
   static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
   if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(g, m, k, group_size, ilog2_exact(group_size / 128),
@@ -638,26 +638,33 @@ int launch_w4p_grouped(hipStream_t st, const LinearArgs* pr, int count) {
   if (grid > 0x7FFFFFFF) return OFQ_ERR_UNSUPPORTED;
   const bool two_per_cu = grid > 256;
   const int nw = two_per_cu ? 8 : 16;
-  if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64) return OFQ_ERR_UNSUPPORTED;
   if ((int64_t)((rpb + 15) / 16) * a.m * 16 > nw * 64) return OFQ_ERR_UNSUPPORTED;
   const bool exact = !(a.symmetric && a.w_signed);
-  const size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
-                                        !a.symmetric);
-  if (lds > (two_per_cu ? 80u : 160u) * 1024u) return OFQ_ERR_UNSUPPORTED;
+  const size_t lds_cap = (two_per_cu ? 80u : 160u) * 1024u;
+  size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                                  !a.symmetric);
+  // x beyond one staging: two stagings, each of half the chunk pairs of a row
+  const bool two_stagings = a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap;
+  if (two_stagings) {
+    lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact, !a.symmetric,
+                             1, 2);
+    const int64_t half_units = a.m * gemv_w4p_phase_chunks((int)a.k, 2) * 8;
+    if (half_units > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) return OFQ_ERR_UNSUPPORTED;
+  }
   GemvGroup g{};
   fill_group(g, pr, count, rpb);
-#define OFQ_W4PG(NWV)                                                                        \
-  if (nw == NWV) {                                                                           \
+#define OFQ_W4PG(NWV, PHV)                                                                   \
+  if (nw == NWV && two_stagings == (PHV == 2)) {                                             \
     if (!exact)                                                                              \
-      return launch_w4p_grouped_inst<NWV, false, true, kZeroNone>(                           \
+      return launch_w4p_grouped_inst<NWV, false, true, kZeroNone, PHV>(                      \
           st, g, (int)grid, (int)a.m, (int)a.k, (int)a.group_size, rpb, lds);                \
     if (a.symmetric)                                                                         \
-      return launch_w4p_grouped_inst<NWV, true, false, kZeroSymU>(                           \
+      return launch_w4p_grouped_inst<NWV, true, false, kZeroSymU, PHV>(                      \
           st, g, (int)grid, (int)a.m, (int)a.k, (int)a.group_size, rpb, lds);                \
-    return launch_w4p_grouped_inst<NWV, true, false, kZeroAsym>(                             \
+    return launch_w4p_grouped_inst<NWV, true, false, kZeroAsym, PHV>(                        \
         st, g, (int)grid, (int)a.m, (int)a.k, (int)a.group_size, rpb, lds);                  \
   }
-  OFQ_W4PG(16) OFQ_W4PG(8)
+  OFQ_W4PG(16, 1) OFQ_W4PG(8, 1) OFQ_W4PG(16, 2) OFQ_W4PG(8, 2)
 #undef OFQ_W4PG
   return OFQ_ERR_UNSUPPORTED;
 }
