@@ -99,9 +99,11 @@ int ofq_groupwise_dequantize(void* stream, const void* in, const void* scale, co
  *   int8 container (no zero term), groups along K with 128 | group_size, m <= 16 -- the Llama
  *   decode case.  There the group scale multiplies the exact fp32 sum of x*q over the group, so
  *   q*scale is never rounded to fp16; the result is closer to exact arithmetic and differs from
- *   the composition above by ~3e-4 rel-L2 (contract: 1e-3).  Every other combination (uint8
- *   container, a zero term, 8 bit, bf16, fp32, m > 16, groups along N) forms w~ with the two
- *   roundings of groupwise_dequantize.  The same weights in the two containers can therefore
+ *   the composition above by ~3e-4 rel-L2 (contract: 1e-3).  The same codes with groups along
+ *   N (16 | group_size, 256 | k) at m = 1 take a kernel of that family in which the scale meets
+ *   x instead (x*scale is rounded to fp16 once per k, q*scale never): the same ~3e-4.  Every
+ *   other combination (uint8 container, a zero term, 8 bit, bf16, fp32, m > 16, groups along N
+ *   otherwise) forms w~ with the two roundings of groupwise_dequantize.  The same weights in the two containers can therefore
  *   differ in the last bits of the output.
  * Any m is accepted (the reference kernel has no m limit either, :473,590).
  * workspace: optional.  ofq_fused_linear_gq_workspace_bytes() is non-zero only for large m on the

@@ -38,6 +38,7 @@ struct M1Shape {
   int rows_per_block;
   int gshift;  // log2(group_size)
   int G;       // groups per row
+  int gn;      // groups along N (GN kernels): rows per group, a multiple of rows_per_block
 };
 
 // LDS: [x operands H x 4 pieces x 64 lanes x 16 B] [corr H x 64 f32]
@@ -102,7 +103,11 @@ struct M1Glu {
 // NW waves per block; RPW rows per wave (rows wave, wave + NW, ..); H = KB of codes per row,
 // rounded up (a lane owns bytes [h*1024 + lane*16, +16) of a row for h < H); XU units of x per
 // thread at staging; NM = 1, or 2 for the GLU (hidden and gate).
-template<int NW, int RPW, int H, int XU, int NM>
+// GN: groups run along N (scale [N / gn, K], one value per k, shared by the gn rows of a group;
+// a block's rows lie in one group).  The scale then meets x instead of the codes: the block
+// stages x * s (one fp16 rounding per k, where the reference rounds q * s per element) and the
+// rows need no scale of their own.
+template<int NW, int RPW, int H, int XU, int NM, bool GN = false>
 __device__ __forceinline__ void
 m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
         const f16* __restrict__ scale, const f16* __restrict__ bias, f16* __restrict__ out, int N,
@@ -122,6 +127,7 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const int nunits = K >> 4;  // 32-byte units of x; XU per thread (K <= 16 * XU * NW * 64)
   const bool stage_wave = wave * 64 < nunits;  // wave-uniform
   u32x4 xu[XU][2];
+  u32x4 su[GN ? XU : 1][2];
   if (stage_wave) {
 #pragma unroll
     for (int i = 0; i < XU; ++i) {
@@ -130,6 +136,12 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
       const u32x4* src = reinterpret_cast<const u32x4*>(x) + (size_t)u * 2;
       xu[i][0] = src[0];
       xu[i][1] = src[1];
+      if (GN) {
+        const u32x4* ssrc =
+            reinterpret_cast<const u32x4*>(scale + (size_t)(row0 / sh.gn) * K) + (size_t)u * 2;
+        su[GN ? i : 0][0] = ssrc[0];
+        su[GN ? i : 0][1] = ssrc[1];
+      }
     }
   }
   uint16_t bias_raw[NM][RPW];
@@ -174,7 +186,7 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
 #pragma unroll
       for (int h = 0; h < H; ++h) {
         const int g = valid[h] ? (h * 2048 + lane * 32) >> sh.gshift : 0;
-        sc[q][i][h] = srow[g];
+        sc[q][i][h] = GN ? (f16)1.0f : srow[g];
       }
     }
   }
@@ -186,6 +198,18 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
     if (wave * 64 + i * NTH >= nunits) break;  // wave-uniform
     const int u = tid + i * NTH;
     const bool ok = u < nunits;
+    if (GN) {
+#pragma unroll
+      for (int p2 = 0; p2 < 2; ++p2) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // (each word through a scalar of its own, see dequant8_b4_v)
+          const uint32_t xw = xu[i][p2][e];
+          const uint32_t sw = su[GN ? i : 0][p2][e];
+          xu[i][p2][e] = as_u32(as_h2(xw) * as_h2(sw));
+        }
+      }
+    }
     u32x4 lo, hi;
     permute_unit(xu[i][0], xu[i][1], lo, hi);
     const int h = u >> 7, l = (u >> 1) & 63, p = u & 1;
@@ -219,7 +243,7 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
 #pragma unroll
       for (int i = 0; i < RPW; ++i) {
         const float acc = m1_dot32(wq[q][i][h], xa, cr);
-        const float term = acc * (float)sc[q][i][h];
+        const float term = GN ? acc : acc * (float)sc[q][i][h];
         tot[q][i] += valid[h] ? term : 0.f;
       }
     }
@@ -380,6 +404,16 @@ gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,
            M1Shape sh) {
   asm volatile("" ::"s"(out));  // fetch the output pointer with the other arguments
   m1_body<NW, RPW, H, XU, 1>(blockIdx.x, x, w, scale, bias, out, sh.N, sh, M1Glu());
+}
+
+// groups along N: scale [N / sh.gn, K]
+template<int NW, int H, int XU = 1>
+__global__ void __launch_bounds__(NW * 64)
+gemv_w4_m1_gn(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+              const f16* __restrict__ scale, const f16* __restrict__ bias, f16* __restrict__ out,
+              M1Shape sh) {
+  asm volatile("" ::"s"(out));
+  m1_body<NW, 1, H, XU, 1, true>(blockIdx.x, x, w, scale, bias, out, sh.N, sh, M1Glu());
 }
 
 // hidden = x w~^T + b, gate = x v~^T + c, y = hidden * act(gate): one launch, one wave per row pair

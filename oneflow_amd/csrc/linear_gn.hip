@@ -156,6 +156,10 @@ bool gemv_gn_supported(const LinearArgs& a) {
 
 int launch_gemv_gn(hipStream_t st, const LinearArgs& a) {
   if (a.t_dtype == OFQ_F32) return launch_gn_f32(st, a);
+  if (gemv_m1_gn_supported(a)) {
+    const int rc = launch_gemv_m1_gn(st, a);
+    if (rc != OFQ_ERR_UNSUPPORTED) return rc;
+  }
   for (int64_t m0 = 0; m0 < a.m; m0 += 64) {
     const int m = (int)(a.m - m0 < 64 ? a.m - m0 : 64);
     const int rc = launch_gn_part(st, a, m0, m);

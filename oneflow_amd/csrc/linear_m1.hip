@@ -22,6 +22,7 @@ int launch_m1_inst(hipStream_t st, const LinearArgs& a) {
   sh.rows_per_block = NW;  // one row per wave
   sh.gshift = log2_exact(a.group_size);
   sh.G = (int)(a.k / a.group_size);
+  sh.gn = 1;
   const int grid = (int)((a.n + NW - 1) / NW);
   gemv_w4_m1<NW, 1, H, XU><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
       static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
@@ -44,7 +45,26 @@ int launch_m1_stream_inst(hipStream_t st, const LinearArgs& a) {
   sh.rows_per_block = rpb;
   sh.gshift = log2_exact(a.group_size);
   sh.G = (int)(a.k / a.group_size);
+  sh.gn = 1;
   gemv_w4_m1_stream<NW, H, 1><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
+      static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
+      static_cast<const f16*>(a.scale), static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
+      sh);
+  return ofq_check_launch();
+}
+
+// groups along N: one row per wave, the block's rows inside one group
+template<int NW, int H, int XU>
+int launch_m1_gn_inst(hipStream_t st, const LinearArgs& a) {
+  M1Shape sh;
+  sh.N = (int)a.n;
+  sh.K = (int)a.k;
+  sh.rows_per_block = NW;
+  sh.gshift = 0;
+  sh.G = 0;
+  sh.gn = (int)a.group_size;
+  const int grid = (int)((a.n + NW - 1) / NW);
+  gemv_w4_m1_gn<NW, H, XU><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
       static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
       static_cast<const f16*>(a.scale), static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
       sh);
@@ -59,6 +79,7 @@ int launch_m1_glu_inst(hipStream_t st, const LinearArgs& a, const M1Glu& glu) {
   sh.rows_per_block = NW;
   sh.gshift = log2_exact(a.group_size);
   sh.G = (int)(a.k / a.group_size);
+  sh.gn = 1;
   const int grid = (int)((a.n + NW - 1) / NW);
   gemv_w4_m1_glu<NW, H, XU><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
       static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
@@ -89,6 +110,7 @@ int launch_m1_grouped_inst(hipStream_t st, const LinearArgs* pr, int count) {
   sh.rows_per_block = NW;
   sh.gshift = log2_exact(pr[0].group_size);
   sh.G = (int)(pr[0].k / pr[0].group_size);
+  sh.gn = 1;
   gemv_w4_m1_grouped<NW, H, XU><<<first, NW * 64, gemv_m1_lds_bytes(H), st>>>(g, sh);
   return ofq_check_launch();
 }
@@ -135,6 +157,23 @@ int launch_gemv_m1(hipStream_t st, const LinearArgs& a) {
 #define OFQ_M1_PLAIN(NW, H, XU) launch_m1_inst<NW, H, XU>(st, a)
   OFQ_M1_DISPATCH(a.k, OFQ_M1_PLAIN);
 #undef OFQ_M1_PLAIN
+}
+
+// Groups along N (scale [n / group_size, k]): the scale is applied to x once per block.
+bool gemv_m1_gn_supported(const LinearArgs& a) {
+  return a.m == 1 && a.t_dtype == OFQ_F16 && a.bits == 4 && a.w_signed && a.symmetric
+         && a.group_dim == 0 && a.group_size % 16 == 0 && a.n % a.group_size == 0
+         && a.k % 256 == 0 && a.k <= 16384 && a.n >= 1 && a.n <= (1 << 24)
+         && (reinterpret_cast<uintptr_t>(a.scale) & 15u) == 0
+         && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0
+         && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0;
+}
+
+int launch_gemv_m1_gn(hipStream_t st, const LinearArgs& a) {
+  if (!gemv_m1_gn_supported(a)) return OFQ_ERR_UNSUPPORTED;
+#define OFQ_M1_GN(NW, H, XU) launch_m1_gn_inst<NW, H, XU>(st, a)
+  OFQ_M1_DISPATCH(a.k, OFQ_M1_GN);
+#undef OFQ_M1_GN
 }
 
 // Two weights of equal shape on one x (hidden, gate) + the gating, one launch.

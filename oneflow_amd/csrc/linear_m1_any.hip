@@ -36,6 +36,7 @@ int launch_any_inst(hipStream_t st, const LinearArgs& a) {
   sh.rows_per_block = (int)rpb;
   sh.gshift = log2_pow2(a.group_size);
   sh.G = (int)(a.k / a.group_size);
+  sh.gn = 1;
   gemv_m1_any<T, BITS, SIGNED, ZMODE, NW, H>
       <<<(int)grid, NW * 64, gemv_m1_any_lds_bytes<BITS>(H), st>>>(
           static_cast<const uint16_t*>(a.x), static_cast<const uint8_t*>(a.w),

@@ -37,6 +37,9 @@ bool gemv_m1_supported(const LinearArgs& a);
 int launch_gemv_m1(hipStream_t st, const LinearArgs& a);
 int launch_gemv_m1_grouped(hipStream_t st, const LinearArgs* problems, int count);
 int launch_gemv_m1_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g, void* y, int act);
+// the same for groups along N (scale [n / group_size, k]): the scale meets x, once per block
+bool gemv_m1_gn_supported(const LinearArgs& a);
+int launch_gemv_m1_gn(hipStream_t st, const LinearArgs& a);
 
 // m = 1, fp16 or bf16, 4- or 8-bit codes in either container, symmetric or with a zero point,
 // groups along K of a power-of-two size: the same row-per-wave structure with the reference's
