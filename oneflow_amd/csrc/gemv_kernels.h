@@ -523,9 +523,9 @@ __device__ __forceinline__ float glu_activation(float v, int act) {
 // chunk c of the 16 rows of the block's tile t is one contiguous KB in the order the lanes take
 // it, [k-slot 0..3][row 0..15][16 bytes], at ((block * tiles_per_block + t) * nchunks + c) * 1024.
 // A request of a wave is then 1 KB of consecutive bytes instead of 16 pieces of 64.
-// PH = 2: m * k is more than LDS holds at once (8 rows of 11008): the chunk pairs of a row are
-// walked in two halves, each with its own staging of x; the x of the second half is requested
-// while the first is worked on, and the sums of a (tile, wave) add up in `red`.
+// PH > 1: m * k is more than LDS holds at once (8 rows of 11008): the chunk pairs of a row are
+// walked in PH parts, each with its own staging of x; the x of the next part is requested while
+// the current one is worked on, and the sums of a (tile, wave) add up in `red`.
 template<int NWAVES, int kW4pDepth = 2, bool EXACT = false, bool SIGNED = true,
          int ZMODE = kZeroNone, bool GLU = false, bool TILED = false, int PH = 1>
 __device__ __forceinline__ void
@@ -535,16 +535,17 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
               int group_size, int cpg_shift, int rows_per_block, GluArgs glu = GluArgs()) {
   static_assert(EXACT || (SIGNED && ZMODE == kZeroNone), "the unrounded path has no zero term");
   static_assert(!(GLU && TILED), "the tile-major layout serves the plain linear only");
-  static_assert(PH == 1 || PH == 2, "one staging of x or two");
+  static_assert(PH >= 1 && PH <= 4, "one to four stagings of x");
   constexpr int NMAT = GLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   constexpr int NT = NWAVES * 64;
   const int nchunks = K >> 7;
   const int npairs_all = (nchunks + 1) >> 1;
   // the phase being worked on: its chunk pairs [., + npairs), its chunks [cbeg, cbeg + ncs)
-  int npairs = PH == 2 ? (npairs_all + 1) >> 1 : npairs_all;
+  const int pairs_per_phase = (npairs_all + PH - 1) / PH;
+  int npairs = pairs_per_phase;
   int cbeg = 0;
-  int ncs = PH == 2 ? 2 * npairs : nchunks;
+  int ncs = PH > 1 && 2 * pairs_per_phase < nchunks ? 2 * pairs_per_phase : nchunks;
   uint32_t inv_chunks = row_of_inv(ncs);
   const int G = K / group_size;
   const int tid = threadIdx.x;
@@ -778,16 +779,23 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     }
   };
   stage_x();
-  if constexpr (PH == 2) {
-    // the second half's x goes out now; it is staged when the first half has been walked
-    const int ncs2 = nchunks - ncs;
-    request_x(M * ncs2 * 8, ncs2, ncs, row_of_inv(ncs2 > 0 ? ncs2 : 1));
+  // chunks of phase ph (none when the row has fewer pairs than phases)
+  auto phase_chunks = [&](int ph) {
+    const int c0 = 2 * pairs_per_phase * ph;
+    int cs = nchunks - c0;
+    if (cs > 2 * pairs_per_phase) cs = 2 * pairs_per_phase;
+    return cs > 0 ? cs : 0;
+  };
+  if constexpr (PH > 1) {
+    // the next part's x goes out now; it is staged when this part has been walked
+    const int cs = phase_chunks(1);
+    request_x(M * cs * 8, cs, 2 * pairs_per_phase, row_of_inv(cs > 0 ? cs : 1));
   }
   __syncthreads();
 
   const uint8_t* xrec = has_x ? xs + (size_t)r * (ncs * 256 + 16) + kb * 64 : zrec;
   const int xrec_stride = has_x ? 256 : 0;
-  bool add_to_red = false;  // second phase: the (tile, wave) slots already hold the first's sums
+  bool add_to_red = false;  // later phases: the (tile, wave) slots already hold earlier sums
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
   f32x4 total1 = {0.f, 0.f, 0.f, 0.f};  // second accumulator of the exact path
   auto flush = [&](int t) {
@@ -797,7 +805,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
       if (m < M) {
         float* slot = red + ((t * NWAVES + wave) * M + m) * 16 + r;
         const float sum = total[v] + total1[v];
-        *slot = PH == 2 && add_to_red ? *slot + sum : sum;
+        *slot = PH > 1 && add_to_red ? *slot + sum : sum;
       }
     }
     total1 = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -916,20 +924,26 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
     }
   };
   walk();
-  if constexpr (PH == 2) {
-    // second half of the chunk pairs: its first items are requested before the barrier behind
-    // which the x records are replaced
-    cbeg = ncs;
-    npairs = npairs_all - npairs;
-    ncs = nchunks - ncs;
-    if (ncs > 0) {
+  if constexpr (PH > 1) {
+    // the further parts of the chunk pairs: a part's first items are requested before the
+    // barrier behind which the x records are replaced
+#pragma unroll 1
+    for (int ph = 1; ph < PH; ++ph) {
+      cbeg = 2 * pairs_per_phase * ph;
+      ncs = phase_chunks(ph);
+      if (ncs <= 0) break;  // uniform
+      npairs = (ncs + 1) >> 1;
       inv_chunks = row_of_inv(ncs);
       nunits = M * ncs * 8;
       add_to_red = true;
       total = f32x4{0.f, 0.f, 0.f, 0.f};
       first_items();
-      __syncthreads();  // every wave has read its last x record and correction of the first half
+      __syncthreads();  // every wave has read its last x record and correction of the part before
       stage_x();
+      if (ph + 1 < PH) {
+        const int cs = phase_chunks(ph + 1);
+        request_x(M * cs * 8, cs, 2 * pairs_per_phase * (ph + 1), row_of_inv(cs > 0 ? cs : 1));
+      }
       __syncthreads();
       xrec = has_x ? xs + (size_t)r * (ncs * 256 + 16) + kb * 64 : zrec;
       walk();
@@ -1041,11 +1055,12 @@ gemv_w4p_f16_glu(const f16* __restrict__ x, const uint8_t* __restrict__ w,
       glu);
 }
 
-// chunks of x a block holds at once: all of a row's, or (two stagings) the larger half of its
-// chunk pairs
+// chunks of x a block holds at once: all of a row's, or (several stagings) the largest part of
+// its chunk pairs
 inline int gemv_w4p_phase_chunks(int K, int phases) {
   const int nchunks = K >> 7;
-  return phases == 2 ? 2 * ((((nchunks + 1) >> 1) + 1) >> 1) : nchunks;
+  const int per_phase = 2 * ((((nchunks + 1) >> 1) + phases - 1) / phases);
+  return phases > 1 && per_phase < nchunks ? per_phase : nchunks;
 }
 
 inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,

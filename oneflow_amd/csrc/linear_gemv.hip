@@ -250,26 +250,31 @@ int launch_w4p(hipStream_t st, const LinearArgs& a, int cpg_shift, bool tiled) {
   size_t lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
                                   !a.symmetric);
   if (a.m * a.k / 16 > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) {
-    // m * k beyond one staging of x: two stagings, each of half the chunk pairs of a row (one
-    // block per CU only)
+    // m * k beyond one staging of x: two to four stagings, each of an equal part of the chunk
+    // pairs of a row (one block per CU only)
     if (nw != 16) return OFQ_ERR_UNSUPPORTED;
-    const int64_t half_units = a.m * gemv_w4p_phase_chunks((int)a.k, 2) * 8;
-    lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
-                             !a.symmetric, 1, 2);
-    if (half_units > (int64_t)kGemvMaxUnits * nw * 64 || lds > lds_cap) return OFQ_ERR_UNSUPPORTED;
-#define OFQ_W4P2(TL)                                                                         \
-  if (tiled == TL) {                                                                         \
+    int phases = 0;
+    for (int ph = 2; ph <= 4 && phases == 0; ++ph) {
+      const int64_t part_units = a.m * gemv_w4p_phase_chunks((int)a.k, ph) * 8;
+      lds = gemv_w4p_lds_bytes(nw, (int)a.m, (int)a.k, (int)a.group_size, rpb, exact,
+                               !a.symmetric, 1, ph);
+      if (part_units <= (int64_t)kGemvMaxUnits * nw * 64 && lds <= lds_cap) phases = ph;
+    }
+    if (phases == 0) return OFQ_ERR_UNSUPPORTED;
+#define OFQ_W4PN(TL, PHV)                                                                    \
+  if (tiled == TL && phases == PHV) {                                                        \
     if (!exact)                                                                              \
-      return launch_w4p_inst<16, false, true, kZeroNone, TL, 2>(st, a, (int)grid, rpb, lds,  \
-                                                                cpg_shift);                  \
+      return launch_w4p_inst<16, false, true, kZeroNone, TL, PHV>(st, a, (int)grid, rpb,     \
+                                                                  lds, cpg_shift);           \
     if (a.symmetric)                                                                         \
-      return launch_w4p_inst<16, true, false, kZeroSymU, TL, 2>(st, a, (int)grid, rpb, lds,  \
+      return launch_w4p_inst<16, true, false, kZeroSymU, TL, PHV>(st, a, (int)grid, rpb,     \
+                                                                  lds, cpg_shift);           \
+    return launch_w4p_inst<16, true, false, kZeroAsym, TL, PHV>(st, a, (int)grid, rpb, lds,  \
                                                                 cpg_shift);                  \
-    return launch_w4p_inst<16, true, false, kZeroAsym, TL, 2>(st, a, (int)grid, rpb, lds,    \
-                                                              cpg_shift);                    \
   }
-    OFQ_W4P2(false) OFQ_W4P2(true)
-#undef OFQ_W4P2
+    OFQ_W4PN(false, 2) OFQ_W4PN(true, 2) OFQ_W4PN(false, 3) OFQ_W4PN(true, 3)
+    OFQ_W4PN(false, 4) OFQ_W4PN(true, 4)
+#undef OFQ_W4PN
   }
 #define OFQ_W4P(NWV, TL)                                                                     \
   if (nw == NWV && tiled == TL) {                                                            \

@@ -170,12 +170,14 @@ def test_decode_w4a16_row_balanced_shapes(m, n, k, container):
 
 @pytest.mark.parametrize("m,n,k", [(16, 80, 8192), (8, 48, 11008), (13, 4096, 4096),
                                    (8, 100, 11136), (5, 300, 16512), (6, 4096, 11008),
-                                   (16, 5000, 8192), (8, 11008, 11008), (7, 33, 22016)])
+                                   (16, 5000, 8192), (8, 11008, 11008), (7, 33, 22016),
+                                   (16, 4096, 11008), (12, 300, 11136), (16, 11008, 11008),
+                                   (16, 64, 16384), (9, 1000, 19200)])
 @pytest.mark.parametrize("symmetric,qdt", VARIANTS)
 def test_decode_w4a16_large_x(m, n, k, symmetric, qdt):
     """m * k too large for x to be staged in LDS at once, for all three code variants: x staged
-    in two halves of a row's chunk pairs (symmetric int8 container; an odd number of chunks, one
-    and several tiles per block, two blocks per CU) or read from L2 per chunk."""
+    in two, three or four parts of a row's chunk pairs (an odd number of chunks, parts of unequal
+    size, one and several tiles per block, two blocks per CU) or read from L2 per chunk."""
     rng = np.random.Generator(np.random.PCG64(m * 131 + n))
     x = H.as_T(rng.standard_normal((m, k)).astype(np.float32), "f16")
     wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
