@@ -328,7 +328,19 @@ namespace {
 // K slices of the int8 GEMM when its 128-wide tiles alone would leave most CUs without a block:
 // as many as still fit one resident round (256x128 tiles: one block per CU; 128x128: two), each
 // at least 4 k-tiles of 128.
+// 64 < m <= 512 on rows of up to 6144 codes, with at least 128 tiles of 64 x 64: the 64 x 64
+// tiles alone fill the chip (256 x 4096 x 4096: 256 blocks), and one launch without partial sums
+// beats K slices over larger tiles (13.7 against 18.7 us; 128 rows 12.6 against 15.1, 512 rows
+// 18.7 against 24.5, 256 x 11008 x 4096 23.1 against 33.1).  A block's k loop costs about 0.43 us
+// per 128-byte k-tile whatever the tile size, so with long rows the slices win again
+// (256 x 4096 x 11008: 46.9 us against 27.8 us).
+bool mq_small_tiles(int64_t m, int64_t n, int64_t k) {
+  return m > kMatmulQuantRowsMaxM && m <= 512 && k % 128 == 0 && k <= 6144
+         && ((m + 63) / 64) * ((n + 63) / 64) >= 128;
+}
+
 int mq_splits(int64_t m, int64_t n, int64_t k) {
+  if (mq_small_tiles(m, n, k)) return 1;
   // long rows (k >= 8192) already pay for slices from 33 rows of a on: 4096 x 11008 at m = 64
   // streams in 33 us and runs in 22 us as slices
   if (m <= (k >= 8192 ? kMatmulQuantRowsMaxM / 2 : kMatmulQuantRowsMaxM) || k % 128 != 0) return 1;
@@ -486,6 +498,10 @@ extern "C" int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, c
     ep.b_scale = b_scale;                                                                      \
     ep.bias = static_cast<const TT<T>::storage*>(bias);                                        \
     ep.out = static_cast<TT<T>::storage*>(out);                                                \
+    if (mq_small_tiles(m, n, k)) {                                                             \
+      return launch_core2<MfmaI8, B2Copy<64, 256>, EP, 64, 64, 2, 2>(st, a, k, bp, ep, m, n,   \
+                                                                    k / 128);                  \
+    }                                                                                          \
     const int bn = m > 128 ? pick_tile_width(m, n, true) : 128;                                \
     if (bn == 384) {                                                                           \
       return launch_core2<MfmaI8, B2Copy<384, 512>, EP, 256, 384, 4, 2>(st, a, k, bp, ep, m,   \

@@ -297,6 +297,37 @@ def test_matmul_quant_few_rows_streaming(m, n, k, t):
 
 
 @pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(65, 8192, 256), (80, 4100, 1024), (256, 4096, 4096), (200, 3001, 640),
+                                   (512, 1100, 6144), (130, 2789, 1152)])
+def test_matmul_quant_64_row_tiles(m, n, k, t):
+    """64 < m <= 512 on rows of up to 6144 codes with at least 128 tiles of 64 x 64: one launch of
+    64 x 64 tiles, no workspace asked for; ragged last tiles in both directions; bit-identical to
+    the oracle's int64 sums and fp32 epilogue."""
+    import torch
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    rng = np.random.Generator(np.random.PCG64(m * 3 + n + k))
+    a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, size=(n, k)).astype(np.int8)
+    a_scale = np.array([0.0173], np.float32)
+    b_scale = rng.uniform(1e-3, 1e-2, size=n).astype(np.float32)
+    bias = H.as_T(rng.standard_normal(n).astype(np.float32), t)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[t]
+    tcode = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16}[t]
+    assert L.ofq_matmul_quant_workspace_bytes(m, n, k) == 0
+    at, bt, ast, bst, biast = map(H.to_torch, (a, b, a_scale, b_scale, bias))
+    out = torch.full((m, n), float("nan"), dtype=tdt, device="cuda")
+    rc = L.ofq_matmul_quant(torch.cuda.current_stream().cuda_stream, at.data_ptr(), bt.data_ptr(),
+                            ast.data_ptr(), bst.data_ptr(), biast.data_ptr(), out.data_ptr(), tcode,
+                            m, n, k)
+    assert rc == 0
+    view = np.uint32 if t == "f32" else np.uint16
+    ref = O.matmul_quant(a, b, a_scale, b_scale, bias,
+                         {"f32": np.float32, "f16": np.float16, "bf16": np.uint16}[t])
+    assert np.array_equal(H.to_numpy(out).view(view), ref.view(view))
+
+
+@pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("m,n,k", [(65, 256, 2048), (128, 1000, 4096), (200, 130, 1024), (512, 384, 1024),
                                    (300, 203, 1536), (40, 256, 8192)])
 def test_matmul_quant_k_slices(m, n, k, t):
