@@ -32,6 +32,9 @@ int pick_tile_width(int64_t m, int64_t n, bool allow_wide) {
   auto cost = [&](int64_t bn) { return ((m_tiles * ((n + bn - 1) / bn) + 255) / 256) * bn; };
   int best = 128;
   if (cost(192) <= cost(best)) best = 192;
+  // 256 x 256 (copy-fed operands only): one round of 256 blocks where 128-wide tiles take two
+  // (int8 4096 x 4096 x 4096: 101 -> 87 us, 3072 rows 85 -> 76 us)
+  if (allow_wide && cost(256) <= cost(best)) best = 256;
   if (allow_wide && cost(384) * 9 <= cost(best) * 10) best = 384;
   return best;
 }
@@ -53,6 +56,9 @@ int launch_plain(hipStream_t st, const LinearArgs& a, const void* wt) {
   switch (pick_tile_width(a.m, a.n, true)) {
     case 384:
       return launch_core2<MF, B2Copy<384, 512>, EP, 256, 384, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
+                                                                    a.n, a.k / 64);
+    case 256:
+      return launch_core2<MF, B2Copy<256, 512>, EP, 256, 256, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
                                                                     a.n, a.k / 64);
     case 192:
       return launch_core2<MF, B2Copy<192, 512>, EP, 256, 192, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
@@ -328,19 +334,29 @@ namespace {
 // K slices of the int8 GEMM when its 128-wide tiles alone would leave most CUs without a block:
 // as many as still fit one resident round (256x128 tiles: one block per CU; 128x128: two), each
 // at least 4 k-tiles of 128.
-// 64 < m <= 512 on rows of up to 6144 codes, with at least 128 tiles of 64 x 64: the 64 x 64
-// tiles alone fill the chip (256 x 4096 x 4096: 256 blocks), and one launch without partial sums
-// beats K slices over larger tiles (13.7 against 18.7 us; 128 rows 12.6 against 15.1, 512 rows
-// 18.7 against 24.5, 256 x 11008 x 4096 23.1 against 33.1).  A block's k loop costs about 0.43 us
-// per 128-byte k-tile whatever the tile size, so with long rows the slices win again
-// (256 x 4096 x 11008: 46.9 us against 27.8 us).
-bool mq_small_tiles(int64_t m, int64_t n, int64_t k) {
-  return m > kMatmulQuantRowsMaxM && m <= 512 && k % 128 == 0 && k <= 6144
-         && ((m + 63) / 64) * ((n + 63) / 64) >= 128;
+// Tiles below 256 rows, one launch, no K slices and no workspace, for the int8 GEMM on rows of up
+// to 6144 codes (a block's k loop costs about 0.4 us per 128-byte k-tile whatever the tile, so
+// on long rows K slices win again: 256 x 4096 x 11008 46.9 us against 27.8 us):
+//  - 64 x 64 tiles (4 waves) when there are 128 to 768 of them: they alone fill the chip
+//    (256 x 4096 x 4096: 256 blocks) and no partial sum leaves it -- 13.3 us against 18.7 us with
+//    slices; 128 rows 12.6 against 15.1, 512 rows 18.7 against 24.5, 768 rows 24.9 against 34.9,
+//    256 x 11008 x 4096 23.1 against 33.1;
+//  - 128 x 128 tiles on 8 waves when the 256-row tiles would leave a quarter of the CUs without
+//    a block and these give 192 to 512 blocks (1024 x 4096 x 4096: 28.7 against 36.3 us,
+//    512 x 11008 x 4096: 40.5 against 48.3 us).
+enum MqTile { kMqTileDefault = 0, kMqTile64 = 64, kMqTile128 = 128 };
+MqTile mq_tile(int64_t m, int64_t n, int64_t k) {
+  if (m <= kMatmulQuantRowsMaxM || k % 128 != 0 || k > 6144) return kMqTileDefault;
+  const int64_t t64 = ((m + 63) / 64) * ((n + 63) / 64);
+  if (m <= 768 && t64 >= 128 && t64 <= 768) return kMqTile64;
+  const int64_t b256 = ((m + 255) / 256) * ((n + 127) / 128);
+  const int64_t b128 = ((m + 127) / 128) * ((n + 127) / 128);
+  if (b256 < 192 && b128 >= 192 && b128 <= 512) return kMqTile128;
+  return kMqTileDefault;
 }
 
 int mq_splits(int64_t m, int64_t n, int64_t k) {
-  if (mq_small_tiles(m, n, k)) return 1;
+  if (mq_tile(m, n, k) != kMqTileDefault) return 1;
   // long rows (k >= 8192) already pay for slices from 33 rows of a on: 4096 x 11008 at m = 64
   // streams in 33 us and runs in 22 us as slices
   if (m <= (k >= 8192 ? kMatmulQuantRowsMaxM / 2 : kMatmulQuantRowsMaxM) || k % 128 != 0) return 1;
@@ -498,11 +514,20 @@ extern "C" int ofq_matmul_quant_ws(void* stream, const void* a, const void* b, c
     ep.b_scale = b_scale;                                                                      \
     ep.bias = static_cast<const TT<T>::storage*>(bias);                                        \
     ep.out = static_cast<TT<T>::storage*>(out);                                                \
-    if (mq_small_tiles(m, n, k)) {                                                             \
+    const MqTile tile = mq_tile(m, n, k);                                                      \
+    if (tile == kMqTile64) {                                                                   \
       return launch_core2<MfmaI8, B2Copy<64, 256>, EP, 64, 64, 2, 2>(st, a, k, bp, ep, m, n,   \
                                                                     k / 128);                  \
     }                                                                                          \
+    if (tile == kMqTile128) {                                                                  \
+      return launch_core2<MfmaI8, B2Copy<128, 512>, EP, 128, 128, 4, 2>(st, a, k, bp, ep, m,   \
+                                                                       n, k / 128);            \
+    }                                                                                          \
     const int bn = m > 128 ? pick_tile_width(m, n, true) : 128;                                \
+    if (bn == 256) {                                                                           \
+      return launch_core2<MfmaI8, B2Copy<256, 512>, EP, 256, 256, 4, 2>(st, a, k, bp, ep, m,   \
+                                                                        n, k / 128);           \
+    }                                                                                          \
     if (bn == 384) {                                                                           \
       return launch_core2<MfmaI8, B2Copy<384, 512>, EP, 256, 384, 4, 2>(st, a, k, bp, ep, m,   \
                                                                         n, k / 128);           \

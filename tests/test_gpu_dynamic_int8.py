@@ -298,11 +298,14 @@ def test_matmul_quant_few_rows_streaming(m, n, k, t):
 
 @pytest.mark.parametrize("t", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("m,n,k", [(65, 8192, 256), (80, 4100, 1024), (256, 4096, 4096), (200, 3001, 640),
-                                   (512, 1100, 6144), (130, 2789, 1152)])
-def test_matmul_quant_64_row_tiles(m, n, k, t):
-    """64 < m <= 512 on rows of up to 6144 codes with at least 128 tiles of 64 x 64: one launch of
-    64 x 64 tiles, no workspace asked for; ragged last tiles in both directions; bit-identical to
-    the oracle's int64 sums and fp32 epilogue."""
+                                   (512, 1100, 6144), (130, 2789, 1152), (768, 4096, 384),
+                                   (1024, 4096, 256), (600, 5000, 640), (2200, 4096, 256),
+                                   (3000, 4100, 128)])
+def test_matmul_quant_one_launch_tile_choices(m, n, k, t):
+    """Shapes for which one launch without K slices and without a workspace is the path: 64 x 64
+    tiles (128 to 768 of them, m <= 768), 128 x 128 tiles where 256-row tiles would leave CUs
+    idle, 256 x 256 tiles where they make one round of two; ragged last tiles in both
+    directions; bit-identical to the oracle's int64 sums and fp32 epilogue."""
     import torch
     from oneflow_amd import _lib
     L = _lib.lib()
