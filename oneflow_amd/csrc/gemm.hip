@@ -33,7 +33,8 @@ int pick_tile_width(int64_t m, int64_t n, bool allow_wide) {
   int best = 128;
   if (cost(192) <= cost(best)) best = 192;
   // 256 x 256 (copy-fed operands only): one round of 256 blocks where 128-wide tiles take two
-  // (int8 4096 x 4096 x 4096: 101 -> 87 us, 3072 rows 85 -> 76 us)
+  // (int8 4096 x 4096 x 4096: 101 -> 87 us; bf16 4096 x 4096 x 11008 behind the dequantised
+  // weight: 410 -> 331 us, 8192 rows 1050 -> 750 us)
   if (allow_wide && cost(256) <= cost(best)) best = 256;
   if (allow_wide && cost(384) * 9 <= cost(best) * 10) best = 384;
   return best;
@@ -53,6 +54,14 @@ int launch_plain(hipStream_t st, const LinearArgs& a, const void* wt) {
   typename EP::Params ep;
   ep.bias = static_cast<const S*>(a.bias);
   ep.out = static_cast<S*>(a.out);
+  // 256-row tiles that would leave a quarter of the CUs without a block, where 128 x 128 tiles
+  // give 192 to 512 blocks: those, on 8 waves (1024 x 4096 x 4096)
+  const int64_t b256 = ((a.m + 255) / 256) * ((a.n + 127) / 128);
+  const int64_t b128 = ((a.m + 127) / 128) * ((a.n + 127) / 128);
+  if (b256 < 192 && b128 >= 192 && b128 <= 512) {
+    return launch_core2<MF, B2Copy<128, 512>, EP, 128, 128, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,
+                                                                  a.n, a.k / 64);
+  }
   switch (pick_tile_width(a.m, a.n, true)) {
     case 384:
       return launch_core2<MF, B2Copy<384, 512>, EP, 256, 384, 4, 2>(st, a.x, a.k * 2, bp, ep, a.m,

@@ -528,12 +528,13 @@ def test_fp32_activations(m, n, k, g, num_bits):
 
 
 @pytest.mark.parametrize("t", ["bf16", "f16"])
-@pytest.mark.parametrize("m,n", [(700, 11012), (1030, 8300), (4000, 4096)])
+@pytest.mark.parametrize("m,n", [(700, 11012), (1030, 8300), (1100, 4100), (4000, 4096)])
 def test_prefill_192_wide_tiles(t, m, n):
     """m and n for which three or four 256-row tiles of x times the 128-wide weight tiles spill
     into a second, nearly empty round of blocks: the 192-wide tiles, in-tile (m < 1024) and
-    copy-fed behind the dequantised weight (m >= 1024, with the workspace); and 16 row tiles on
-    n = 4096, which the copy-fed path covers with one round of 256-wide tiles; sampled rows."""
+    copy-fed behind the dequantised weight (m >= 1024, with the workspace); and five row tiles on
+    n = 4100, which the copy-fed path covers with 128 x 128 tiles on 8 waves, and 16 on n = 4096,
+    which it covers with one round of 256-wide tiles; sampled rows."""
     import torch
     from oneflow_amd import _lib
     L = _lib.lib()
