@@ -118,7 +118,6 @@ gemv_m1_any(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
     }
   };
   issue(0, 0);
-  issue(1, 1);
 
   // ---- x -> LDS: piece t of lane l of KB h at ((h*XP + t)*64 + l)*16 ---------------------------
 #pragma unroll
@@ -132,6 +131,7 @@ gemv_m1_any(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
     }
   }
   __syncthreads();
+  issue(1, 1);  // behind the barrier: a smaller first burst streams a little better
 
   u32x4 xr[kXInRegs ? H : 1][XP];
   if (kXInRegs) {
