@@ -213,10 +213,14 @@ int launch_wave_rows_inst(hipStream_t st, const uint8_t* a, const uint8_t* b, co
                           const float* b_scale, const void* bias, void* out, int m, int64_t n,
                           int64_t k) {
   typedef typename TT<T>::storage S;
-  constexpr int NW = 16;
-  // one block per CU, two from 128 rows per block on; a wave then walks its rows two ahead
-  int64_t grid = 256;
-  if ((n + grid - 1) / grid >= 128) grid = 512;
+  // A lane holds 4 H MR registers of a and 8 H of b: 16 waves (128 registers each) while that
+  // fits, 8 waves (256 each) beyond, where the compiler would otherwise spill to scratch memory
+  // (8192 x 8192, 2 rows).
+  constexpr int NW = H * (4 * MR + 8) <= 100 ? 16 : 8;
+  // 16 waves per CU, twice as many blocks from 128 rows per block on; a wave then walks its rows
+  // two ahead
+  int64_t grid = 256 * (16 / NW);
+  if ((n + grid - 1) / grid >= 128) grid *= 2;
   int rpb = (int)((n + grid - 1) / grid);
   if (rpb < NW) rpb = NW;
   grid = (n + rpb - 1) / rpb;
@@ -226,7 +230,9 @@ int launch_wave_rows_inst(hipStream_t st, const uint8_t* a, const uint8_t* b, co
   return ofq_check_launch();
 }
 
-// m <= 4, 16 | k <= 8192 (the rows of a are held in registers: 4 H m of them)
+// m <= 2 with 16 | k <= 8192, m <= 4 with k <= 4096 (the rows of a are held in registers: 4 H m
+// of them).  Three and four rows of more than 4 KB run faster on the matrix-core kernel below
+// (4096 x 8192, 4 rows: 14.5 us here, 9.4 us there).
 template<typename T>
 int launch_wave_rows(hipStream_t st, const uint8_t* a, const uint8_t* b, const float* a_scale,
                      const float* b_scale, const void* bias, void* out, int m, int64_t n,
@@ -236,7 +242,11 @@ int launch_wave_rows(hipStream_t st, const uint8_t* a, const uint8_t* b, const f
   case HV:                                                                                     \
     if (m == 1) return launch_wave_rows_inst<T, HV, 1>(st, a, b, a_scale, b_scale, bias, out, m, n, k); \
     if (m == 2) return launch_wave_rows_inst<T, HV, 2>(st, a, b, a_scale, b_scale, bias, out, m, n, k); \
-    return launch_wave_rows_inst<T, HV, 4>(st, a, b, a_scale, b_scale, bias, out, m, n, k);
+    if constexpr (HV <= 4) {                                                                   \
+      return launch_wave_rows_inst<T, HV, 4>(st, a, b, a_scale, b_scale, bias, out, m, n, k);  \
+    } else {                                                                                   \
+      return OFQ_ERR_UNSUPPORTED;                                                              \
+    }
   switch (h) {
     OFQ_WR(1) OFQ_WR(2) OFQ_WR(3) OFQ_WR(4) OFQ_WR(5) OFQ_WR(6) OFQ_WR(7) OFQ_WR(8)
     default: return OFQ_ERR_UNSUPPORTED;

@@ -256,10 +256,12 @@ def test_matmul_quant_wide_tiles_full_output(t, m, n):
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (5, 1000, 192), (16, 37, 64), (17, 688, 1024),
                                    (33, 2049, 448), (64, 300, 11008), (200, 130, 192),
                                    (2, 11008, 4096), (3, 1000, 192), (4, 37, 8192), (1, 30000, 64),
-                                   (4, 4099, 1088), (2, 70000, 128), (1, 13, 7168), (4, 33, 11008)])
+                                   (4, 4099, 1088), (2, 70000, 128), (1, 13, 7168), (4, 33, 11008),
+                                   (2, 9000, 8192), (4, 9000, 5120), (3, 600, 7232)])
 def test_matmul_quant_few_rows_streaming(m, n, k, t):
     """m <= 64 (and any m when k is a multiple of 64 but not of 128) runs the streaming int8
-    kernels: up to 4 rows of a with k <= 8192 the one in which a wave owns whole rows of b (every
+    kernels: up to 2 rows of a with k <= 8192, up to 4 with k <= 4096, the one in which a wave owns
+    whole rows of b (every
     row length class incl. partial KBs, one and two blocks per CU, many rows per wave, fewer rows
     than waves), beyond that the MFMA kernel with 1, 2 and 4 tiles of a, ragged n, k from one
     chunk to many, several passes for m = 200.  Bit-exact: int32 sums are order-free and the
