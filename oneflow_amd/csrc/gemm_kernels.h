@@ -4,6 +4,7 @@
 #pragma once
 
 #include <atomic>
+#include <type_traits>
 #include "dequant_regs.h"
 #include "ofq_device.h"
 
@@ -258,8 +259,11 @@ struct B2Dequant {
   // would put a wait for the loads right behind their issue
   struct Regs {
     u32x4 v[kChunks];
-    typename TT<T>::storage s[kChunks];
-    typename TT<T>::storage z[kChunks];
+    // raw 16 bits each.  With a zero term or 8-bit codes they get registers of their own:
+    // 16-bit slots there ended up in scratch memory (a store and two loads per k-tile).
+    typedef typename std::conditional<BITS == 4 && ZMODE == 0, uint16_t, uint32_t>::type Slot;
+    Slot s[kChunks];
+    Slot z[kChunks];
   };
   static __device__ __forceinline__ void load(const Params& p, int n0, int kt, int, int, int tid,
                                               Regs& r, uint8_t*) {
@@ -274,8 +278,8 @@ struct B2Dequant {
                                                + (int64_t)kt * kCodeBytesPerRow + c * 16);
       const int k = kt * 64 + c * kElemsPerChunk;
       const int64_t si = (int64_t)row * p.G + k / p.group_size;
-      r.s[i] = p.scale[si];
-      if (ZMODE == 2) r.z[i] = p.zero[si];
+      r.s[i] = reinterpret_cast<const uint16_t*>(p.scale)[si];
+      if (ZMODE == 2) r.z[i] = reinterpret_cast<const uint16_t*>(p.zero)[si];
     }
   }
   // dequantise and store a quarter of the thread's chunks (all of them when there are fewer)
@@ -290,9 +294,9 @@ struct B2Dequant {
       const int c = q % kChunksPerRow;
       uint8_t* rowp = lds + row * kStageRow;
       const int sw = swizzle_key(row);
-      const float sc = TT<T>::load(&r.s[i]);
+      const float sc = raw16_to_float<T>((uint16_t)r.s[i]);
       float zc = 0.f;
-      if (ZMODE == 2) zc = TT<T>::load(&r.z[i]);
+      if (ZMODE == 2) zc = raw16_to_float<T>((uint16_t)r.z[i]);
       if (ZMODE == 1) zc = TT<T>::round(-(float)((1 << (BITS - 1)) - 1) * sc);
       if constexpr (BITS == 8) {
         u32x4 o0, o1;

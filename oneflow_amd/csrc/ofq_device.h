@@ -70,6 +70,17 @@ struct TT<bf16> {
   }
 };
 
+// raw bits of a 16-bit T -> float.  Registers that hold scales between their load and their use
+// keep them as uint16_t: arrays of f16 inside a struct can end up in scratch memory.
+template<typename T>
+__device__ __forceinline__ float raw16_to_float(uint16_t raw) {
+  if constexpr (TT<T>::dtype == OFQ_BF16) {
+    return __builtin_bit_cast(float, (uint32_t)raw << 16);
+  } else {
+    return (float)__builtin_bit_cast(f16, raw);
+  }
+}
+
 // ---- wave64 reductions through DPP-free cross-lane shuffles (ds_bpermute / permlane) ----
 template<typename V, typename Op>
 __device__ __forceinline__ V wave_reduce(V v, Op op) {
