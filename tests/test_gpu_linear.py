@@ -98,7 +98,9 @@ def test_decode_m1_row_per_wave_shapes(n, k, g, with_bias):
     (5, 300, 5120, 128, True), (6, 2048, 8192, 1024, True), (7, 64, 11008, 128, True),
     (8, 4096, 4096, 128, True), (8, 129, 7936, 128, False), (4, 77, 13824, 128, True),
     (3, 33, 16384, 128, True), (2, 50, 14336, 256, False), (8, 20000, 256, 128, True),
-    (8, 64, 11008, 128, True), (5, 64, 16384, 128, True),
+    (8, 64, 11008, 128, True), (5, 64, 16384, 128, True), (4, 11008, 4096, 128, True),
+    (2, 33000, 512, 128, False), (3, 20000, 1280, 256, True), (8, 11008, 4096, 128, True),
+    (6, 1001, 3840, 128, True), (7, 4096, 2304, 256, False), (5, 6, 256, 128, True),
 ])
 def test_decode_few_rows_of_x_long_and_ragged_rows(m, n, k, g, with_bias):
     """2 .. 8 rows of x, fp16, symmetric int4 in an int8 container: every row length up to 16384
