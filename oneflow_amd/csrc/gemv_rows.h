@@ -311,15 +311,33 @@ gemv_rows_grouped(GemvGroup g, int M, int K, int group_size, int gs_shift, int r
 
 // ---------------------------------------------------------------------------------------------
 // 16 < m <= 64: the same row split with MT = 2 or 4 sixteen-row tiles of x per MFMA group.  A
-// weight tile is expanded once per chunk and meets all MT tiles of x, which come straight from
-// L2 (x is far too large for LDS here: m * k * 2 bytes per block); a wave walks chunks
+// weight tile is expanded once per chunk and meets all MT tiles of x, which come from L2 chunk
+// by chunk (x is far too large for LDS here: m * k * 2 bytes per block); a wave walks chunks
 // c = wave, wave + NWAVES, ... and, per chunk, every 16-row weight tile of the block, with the
 // codes of the next (tile, chunk) requested before the current ones are used.  Sums stay in
 // registers (kRowsMaxTiles * MT accumulators) and are folded through LDS one weight tile at a
 // time.  No barrier inside the k loop, unlike the tiled GEMM, whose per-k-tile cost does not
 // shrink with m.
 // ---------------------------------------------------------------------------------------------
-template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, int MT>
+// XLDS: a lane's operand of x is 16 bytes out of a 64-byte run of one of 16 rows, so a
+// wave-level request straight from global memory touches 64 cache lines for 1 KB of data and the
+// vector cache's tag rate bounds the kernel (4096 x 11008 at 64 rows of x: 6 us per chunk and
+// wave).  With XLDS a wave requests the chunk's MT * 16 rows x 2 CK bytes of x with neighbouring
+// lanes on neighbouring bytes (8 cache lines per request), one chunk ahead, parks them in a
+// buffer of its own in LDS (rows padded by 16 bytes) and reads its operands from there.  The
+// buffers share their memory with the reduction area, which is used only after the k loop.
+template<int BITS, int MT>
+struct RowsMtX {
+  static constexpr int CK = BITS == 4 ? 128 : 64;
+  static constexpr int kRowBytes = CK * 2;           // of x per row and chunk
+  static constexpr int kPitch = kRowBytes + 16;      // in LDS
+  static constexpr int kLanesPerRow = kRowBytes / 16;
+  static constexpr int kRowsPerReq = 64 / kLanesPerRow;
+  static constexpr int kReqs = MT * 16 / kRowsPerReq;
+  static constexpr int kWaveBytes = MT * 16 * kPitch;
+};
+
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, int MT, bool XLDS = false>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_rows_mt(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
              const uint16_t* __restrict__ scale, const uint16_t* __restrict__ zero,
@@ -346,11 +364,17 @@ gemv_rows_mt(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
   if (rows_blk <= 0) return;
   const int ntiles = (rows_blk + 15) >> 4;
 
-  // LDS: [red NWAVES*MT*256 f32][scales rows_per_block*G, padded to 16 B][zeros (asymmetric)]
+  // LDS: [red NWAVES*MT*256 f32 | the waves' x buffers (XLDS)][scales rows_per_block*G, padded
+  //      to 16 B][zeros (asymmetric)]
+  typedef RowsMtX<BITS, MT> XB;
   float* red = reinterpret_cast<float*>(smem);
   const int tile_bytes = (rows_per_block * G * 2 + 15) & ~15;
-  uint16_t* sl = reinterpret_cast<uint16_t*>(smem + (size_t)NWAVES * MT * 256 * 4);
+  constexpr size_t kRedBytes = (size_t)NWAVES * MT * 256 * 4;
+  constexpr size_t kFront = XLDS && (size_t)NWAVES * XB::kWaveBytes > kRedBytes
+                                ? (size_t)NWAVES * XB::kWaveBytes : kRedBytes;
+  uint16_t* sl = reinterpret_cast<uint16_t*>(smem + kFront);
   uint16_t* zl = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
+  uint8_t* xbuf = smem + (size_t)wave * XB::kWaveBytes;
 
   const uint8_t* wbase = w + (int64_t)row0 * row_bytes + kb * 16;
   auto issue = [&](int tile, int c, bool live) {
@@ -380,6 +404,24 @@ gemv_rows_mt(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
     const int row = mt * 16 + r;
     xrow[mt] = reinterpret_cast<const uint8_t*>(x) + ((size_t)(row < M ? row : 0) * K + kb * LK) * 2;
   }
+  // XLDS: request i of a chunk covers rows kRowsPerReq * i + lane / kLanesPerRow, 16 bytes per lane
+  const uint8_t* xreq[XLDS ? XB::kReqs : 1];
+  u32x4 xg[XLDS ? XB::kReqs : 1];
+  if (XLDS) {
+#pragma unroll
+    for (int i = 0; i < XB::kReqs; ++i) {
+      const int row = i * XB::kRowsPerReq + lane / XB::kLanesPerRow;
+      xreq[i] = reinterpret_cast<const uint8_t*>(x) + (size_t)(row < M ? row : 0) * K * 2
+                + (lane % XB::kLanesPerRow) * 16;
+    }
+  }
+  auto request_x = [&](int chunk) {  // (a chunk past the end re-reads chunk 0)
+#pragma unroll
+    for (int i = 0; i < XB::kReqs; ++i) {
+      xg[i] = *reinterpret_cast<const u32x4*>(xreq[i] + (size_t)chunk * XB::kRowBytes);
+    }
+  };
+  if (XLDS) request_x(c < nchunks ? c : 0);
   f32x4 acc[kRowsMaxTiles][MT];
 #pragma unroll
   for (int t = 0; t < kRowsMaxTiles; ++t)
@@ -388,11 +430,30 @@ gemv_rows_mt(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
 
   while (c < nchunks) {
     u32x4 xa[MT][XV];
+    if (XLDS) {
+      // the wave's own buffer: its LDS operations retire in order, so these stores cannot pass
+      // the operand reads of the chunk before
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const u32x4* xp = reinterpret_cast<const u32x4*>(xrow[mt] + (size_t)c * (CK * 2));
+      for (int i = 0; i < XB::kReqs; ++i) {
+        const int row = i * XB::kRowsPerReq + lane / XB::kLanesPerRow;
+        *reinterpret_cast<u32x4*>(xbuf + row * XB::kPitch + (lane % XB::kLanesPerRow) * 16) = xg[i];
+      }
+      request_x(c + NWAVES < nchunks ? c + NWAVES : 0);
 #pragma unroll
-      for (int j = 0; j < XV; ++j) xa[mt][j] = xp[j];
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int j = 0; j < XV; ++j) {
+          xa[mt][j] = *reinterpret_cast<const u32x4*>(xbuf + (mt * 16 + r) * XB::kPitch
+                                                      + kb * (LK * 2) + j * 16);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const u32x4* xp = reinterpret_cast<const u32x4*>(xrow[mt] + (size_t)c * (CK * 2));
+#pragma unroll
+        for (int j = 0; j < XV; ++j) xa[mt][j] = xp[j];
+      }
     }
     const int k0 = c * CK + kb * LK;
     const int grp = gs_shift >= 0 ? (k0 >> gs_shift) : (k0 / group_size);
@@ -433,6 +494,7 @@ gemv_rows_mt(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
   }
 
   // fold, one weight tile at a time: red[wave][m (MT*16)][n (16)]
+  if (XLDS) __syncthreads();  // the reduction area overlays the x buffers of other waves
 #pragma unroll
   for (int t = 0; t < kRowsMaxTiles; ++t) {
     if (t < ntiles) {
@@ -612,10 +674,13 @@ inline size_t gemv_rows_f32_lds_bytes(int nwaves, int K, int group_size, int row
 }
 
 inline size_t gemv_rows_mt_lds_bytes(int nwaves, int mt, int K, int group_size,
-                                     int rows_per_block, bool asym) {
+                                     int rows_per_block, bool asym, int bits = 4,
+                                     bool xlds = false) {
   const int G = K / group_size;
-  return (size_t)nwaves * mt * 256 * 4
-         + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15);
+  size_t front = (size_t)nwaves * mt * 256 * 4;
+  const size_t xb = (size_t)nwaves * mt * 16 * ((bits == 4 ? 256 : 128) + 16);
+  if (xlds && xb > front) front = xb;
+  return front + (size_t)(asym ? 2 : 1) * ((rows_per_block * G * 2 + 15) & ~15);
 }
 
 inline size_t gemv_rows_lds_bytes(int nwaves, int M, int K, int group_size, int rows_per_block,

@@ -440,10 +440,10 @@ int launch_gemv_variant(hipStream_t st, const LinearArgs& a) {
 }
 
 // ---- 16 < m <= 128: several tiles of x per weight tile ----------------------------------------
-template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT>
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT, bool XLDS>
 int launch_rows_mt_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m,
                         int grid, int rows_per_block, size_t lds) {
-  auto kern = gemv_rows_mt<T, BITS, SIGNED, ZMODE, NW, MT>;
+  auto kern = gemv_rows_mt<T, BITS, SIGNED, ZMODE, NW, MT, XLDS>;
   static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
   if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(
@@ -454,13 +454,13 @@ int launch_rows_mt_inst(hipStream_t st, const LinearArgs& a, const void* x, void
   return ofq_check_launch();
 }
 
-template<typename T, int NW, int MT>
+template<typename T, int NW, int MT, bool XLDS>
 int launch_rows_mt_t(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m,
                      int grid, int rpb, size_t lds) {
   const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
 #define OFQ_R(B, SG, ZM)                                              \
   if (a.bits == B && a.w_signed == SG && zmode == ZM)                 \
-    return launch_rows_mt_inst<T, B, SG, ZM, NW, MT>(st, a, x, out, m, grid, rpb, lds);
+    return launch_rows_mt_inst<T, B, SG, ZM, NW, MT, XLDS>(st, a, x, out, m, grid, rpb, lds);
   OFQ_R(4, true, kZeroNone)
   OFQ_R(4, false, kZeroSymU)
   OFQ_R(4, false, kZeroAsym)
@@ -481,19 +481,38 @@ int launch_rows_mt_part(hipStream_t st, const LinearArgs& a, int64_t m0, int m) 
   if (rpb < 16) rpb = 16;
   grid = (a.n + rpb - 1) / rpb;
   const int mt = (m + 15) / 16;  // 2, 3 or 4 tiles of x
+  const size_t esz = 2;
+  const void* x = static_cast<const char*>(a.x) + (size_t)m0 * a.k * esz;
+  void* out = static_cast<char*>(a.out) + (size_t)m0 * a.n * esz;
+  // x through per-wave buffers in LDS (coalesced requests, one chunk ahead): 12 waves for two
+  // tiles of x, 8 for three and four (the buffers and the registers of the chunk in flight)
+  {
+    const int nw = mt == 2 ? 12 : 8;
+    const size_t lds = gemv_rows_mt_lds_bytes(nw, mt, (int)a.k, (int)a.group_size, rpb,
+                                              !a.symmetric, a.bits, true);
+    if (lds <= 160u * 1024u) {
+#define OFQ_MTX(TT_)                                                                            \
+  switch (mt) {                                                                                 \
+    case 2: return launch_rows_mt_t<TT_, 12, 2, true>(st, a, x, out, m, (int)grid, rpb, lds);   \
+    case 3: return launch_rows_mt_t<TT_, 8, 3, true>(st, a, x, out, m, (int)grid, rpb, lds);    \
+    default: return launch_rows_mt_t<TT_, 8, 4, true>(st, a, x, out, m, (int)grid, rpb, lds);   \
+  }
+      if (a.t_dtype == OFQ_BF16) { OFQ_MTX(bf16) }
+      OFQ_MTX(f16)
+#undef OFQ_MTX
+    }
+  }
+  // x straight from L2 (the scales of a long-rowed block leave no room for the buffers):
   // 16 waves while the registers allow four waves per SIMD, 12 beyond
   const int nw = mt == 2 ? 16 : 12;
   const size_t lds =
       gemv_rows_mt_lds_bytes(nw, mt, (int)a.k, (int)a.group_size, rpb, !a.symmetric);
   if (lds > 160u * 1024u) return OFQ_ERR_UNSUPPORTED;
-  const size_t esz = 2;
-  const void* x = static_cast<const char*>(a.x) + (size_t)m0 * a.k * esz;
-  void* out = static_cast<char*>(a.out) + (size_t)m0 * a.n * esz;
-#define OFQ_MT(TT_)                                                                        \
-  switch (mt) {                                                                            \
-    case 2: return launch_rows_mt_t<TT_, 16, 2>(st, a, x, out, m, (int)grid, rpb, lds);    \
-    case 3: return launch_rows_mt_t<TT_, 12, 3>(st, a, x, out, m, (int)grid, rpb, lds);    \
-    default: return launch_rows_mt_t<TT_, 12, 4>(st, a, x, out, m, (int)grid, rpb, lds);   \
+#define OFQ_MT(TT_)                                                                               \
+  switch (mt) {                                                                                   \
+    case 2: return launch_rows_mt_t<TT_, 16, 2, false>(st, a, x, out, m, (int)grid, rpb, lds);    \
+    case 3: return launch_rows_mt_t<TT_, 12, 3, false>(st, a, x, out, m, (int)grid, rpb, lds);    \
+    default: return launch_rows_mt_t<TT_, 12, 4, false>(st, a, x, out, m, (int)grid, rpb, lds);   \
   }
   if (a.t_dtype == OFQ_BF16) { OFQ_MT(bf16) }
   OFQ_MT(f16)

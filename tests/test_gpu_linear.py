@@ -417,6 +417,25 @@ def test_small_batch_multi_tile_kernel(m, n, k, g, num_bits, t):
         assert r < (3e-3 if t == "bf16" else 1e-4)
 
 
+@pytest.mark.parametrize("m,n,k,g,symmetric,qdt", [
+    (33, 11008, 4096, 128, True, np.int8), (64, 4096, 11008, 128, False, np.uint8),
+    (17, 16400, 11008, 32, False, np.uint8)])
+def test_small_batch_multi_tile_kernel_model_shapes(m, n, k, g, symmetric, qdt):
+    """16 < m <= 64 on the shapes of a model: many chunks per wave (the x of a chunk goes through
+    the wave's buffer in LDS while the next chunk's is in flight), three and four weight tiles
+    per block; the last case leaves no room for the buffers beside the block's scales and zeros
+    (64 rows x 344 groups) and takes x straight from L2."""
+    rng = np.random.Generator(np.random.PCG64(m * 7 + n))
+    x = H.as_T((rng.standard_normal((m, k)) / 4).astype(np.float32), "f16")
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    b = H.as_T((rng.standard_normal(n) * 0.01).astype(np.float32), "f16")
+    w, scale, zero = H.quantize_groupwise(wf, 4, symmetric, 1, g, qdt, "f16")
+    ref = O.fused_linear(x, w, scale, zero, b, 4, symmetric, 1, g)
+    got = _run(x, w, scale, zero, b, 4, symmetric, 1, g)
+    r, e = H.assert_linear_parity(got, ref, "f16", f"m={m} n={n} k={k}")
+    assert r < 1e-4
+
+
 @pytest.mark.parametrize("m,n,k", [(65, 300, 1024), (128, 1000, 4096), (130, 520, 2048),
                                    (300, 384, 1024), (257, 203, 1536)])
 @pytest.mark.parametrize("num_bits", [4, 8])
