@@ -103,10 +103,10 @@ def main():
                 w = torch.randint(-128, 128, (n, k // 2), dtype=torch.int8, device=dev)
                 scale = torch.empty((n, k // 128), dtype=torch.float16, device=dev).uniform_(1e-3, 1e-2)
                 bias = (torch.randn(n, device=dev) * 0.01).to(torch.float16)
-                out = torch.empty((max(M, 8), n), dtype=torch.float16, device=dev)
+                out = torch.empty((max(M, 64), n), dtype=torch.float16, device=dev)
                 mats.append((name, n, k, w, scale, bias, out))
         layers.append(mats)
-    x_by_k = {k: torch.randn((max(M, 8), k), device=dev).to(torch.float16) for k in (4096, 11008)}
+    x_by_k = {k: torch.randn((max(M, 64), k), device=dev).to(torch.float16) for k in (4096, 11008)}
 
     def launch(mat, m=M):
         name, n, k, w, scale, bias, out = mat
@@ -129,7 +129,7 @@ def main():
 
     # the same step with the block's neighbouring ops fused: q/k/v as one grouped launch,
     # o, gate|up with the SiLU gating as one launch, down: 4 launches per layer, not 7 (+ gating)
-    glu_y = torch.empty((max(M, 8), 11008), dtype=torch.float16, device=dev)
+    glu_y = torch.empty((max(M, 64), 11008), dtype=torch.float16, device=dev)
     vp = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
     i64 = lambda v: (ctypes.c_int64 * len(v))(*v)
 
@@ -319,7 +319,8 @@ def main():
                 "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
                              "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4)}}
         del tiled
-        # per shape: the GEMV alone over all layers for 1, 4 and 8 rows of x, and beside it a
+        # per shape: the GEMV alone over all layers for 1, 4 and 8 rows of x (and 32 and 64, the
+        # batch sizes of a serving loop, which run the multi-tile streaming kernel), and beside it a
         # kernel that only reads the codes of the same weight tensors (ofq_probe_read; 97% of the
         # bytes the GEMV reads, in one launch per tensor) in the same graph-replay harness: what
         # reading those bytes once takes on this box
@@ -331,7 +332,7 @@ def main():
                 st = L.ofq_probe_read(stream, mat[3].data_ptr(), mat[3].numel(), sink.data_ptr())
                 if st != 0:
                     raise RuntimeError(f"ofq_probe_read status {st}")
-        for m in sorted({M, 1, 4, 8}):
+        for m in sorted({M, 1, 4, 8, 32, 64}):
             by_shape = {}
             for name, n, k, cnt in LLAMA7B_LAYER:
                 mats_s = [mat for mats in layers for mat in mats if mat[0] == name]
