@@ -19,7 +19,9 @@
 namespace ofq {
 namespace {
 
-template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, int MT>
+// XLDS: x through per-wave buffers in LDS, requested with neighbouring lanes on neighbouring
+// bytes one chunk ahead (see gemv_rows_mt); the buffers share their memory with `red`.
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NWAVES, int MT, bool XLDS = false>
 __global__ void __launch_bounds__(NWAVES * 64)
 gemv_rows_gn(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
              const uint16_t* __restrict__ scale, const uint16_t* __restrict__ zero,
@@ -47,10 +49,16 @@ gemv_rows_gn(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
   const int g_first = row0 / group_size;
   const int ng = (row0 + rows_blk - 1) / group_size - g_first + 1;
 
-  // LDS: [red NWAVES*MT*256 f32][scale rows of the block's groups, ng x K][zero rows (asymmetric)]
+  // LDS: [red NWAVES*MT*256 f32 | the waves' x buffers (XLDS)][scale rows of the block's groups,
+  //      ng x K][zero rows (asymmetric)]
+  typedef RowsMtX<BITS, MT> XB;
   float* red = reinterpret_cast<float*>(smem);
-  uint16_t* sl = reinterpret_cast<uint16_t*>(smem + (size_t)NWAVES * MT * 256 * 4);
+  constexpr size_t kRedBytes = (size_t)NWAVES * MT * 256 * 4;
+  constexpr size_t kFront = XLDS && (size_t)NWAVES * XB::kWaveBytes > kRedBytes
+                                ? (size_t)NWAVES * XB::kWaveBytes : kRedBytes;
+  uint16_t* sl = reinterpret_cast<uint16_t*>(smem + kFront);
   uint16_t* zl = sl + (size_t)ng * K;
+  uint8_t* xbuf = smem + (size_t)wave * XB::kWaveBytes;
 
   const uint8_t* wbase = w + (int64_t)row0 * row_bytes + kb * 16;
   auto issue = [&](int tile, int c, bool live) {
@@ -89,6 +97,24 @@ gemv_rows_gn(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
     const int row = mt * 16 + r;
     xrow[mt] = reinterpret_cast<const uint8_t*>(x) + ((size_t)(row < M ? row : 0) * K + kb * LK) * 2;
   }
+  // XLDS: request i of a chunk covers rows kRowsPerReq * i + lane / kLanesPerRow, 16 bytes per lane
+  const uint8_t* xreq[XLDS ? XB::kReqs : 1];
+  u32x4 xg[XLDS ? XB::kReqs : 1];
+  if (XLDS) {
+#pragma unroll
+    for (int i = 0; i < XB::kReqs; ++i) {
+      const int row = i * XB::kRowsPerReq + lane / XB::kLanesPerRow;
+      xreq[i] = reinterpret_cast<const uint8_t*>(x) + (size_t)(row < M ? row : 0) * K * 2
+                + (lane % XB::kLanesPerRow) * 16;
+    }
+  }
+  auto request_x = [&](int chunk) {  // (a chunk past the end re-reads chunk 0)
+#pragma unroll
+    for (int i = 0; i < XB::kReqs; ++i) {
+      xg[i] = *reinterpret_cast<const u32x4*>(xreq[i] + (size_t)chunk * XB::kRowBytes);
+    }
+  };
+  if (XLDS) request_x(c < nchunks ? c : 0);
   f32x4 acc[kRowsMaxTiles][MT];
 #pragma unroll
   for (int t = 0; t < kRowsMaxTiles; ++t)
@@ -97,11 +123,30 @@ gemv_rows_gn(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
 
   while (c < nchunks) {
     u32x4 xa[MT][XV];
+    if (XLDS) {
+      // the wave's own buffer: its LDS operations retire in order, so these stores cannot pass
+      // the operand reads of the chunk before
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const u32x4* xp = reinterpret_cast<const u32x4*>(xrow[mt] + (size_t)c * (CK * 2));
+      for (int i = 0; i < XB::kReqs; ++i) {
+        const int row = i * XB::kRowsPerReq + lane / XB::kLanesPerRow;
+        *reinterpret_cast<u32x4*>(xbuf + row * XB::kPitch + (lane % XB::kLanesPerRow) * 16) = xg[i];
+      }
+      request_x(c + NWAVES < nchunks ? c + NWAVES : 0);
 #pragma unroll
-      for (int j = 0; j < XV; ++j) xa[mt][j] = xp[j];
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int j = 0; j < XV; ++j) {
+          xa[mt][j] = *reinterpret_cast<const u32x4*>(xbuf + (mt * 16 + r) * XB::kPitch
+                                                      + kb * (LK * 2) + j * 16);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const u32x4* xp = reinterpret_cast<const u32x4*>(xrow[mt] + (size_t)c * (CK * 2));
+#pragma unroll
+        for (int j = 0; j < XV; ++j) xa[mt][j] = xp[j];
+      }
     }
 #pragma unroll
     for (int t = 0; t < kRowsMaxTiles; ++t) {
@@ -138,6 +183,7 @@ gemv_rows_gn(const uint16_t* __restrict__ x, const uint8_t* __restrict__ w,
   }
 
   // fold, one weight tile at a time: red[wave][m (MT*16)][n (16)]
+  if (XLDS) __syncthreads();  // the reduction area overlays the x buffers of other waves
 #pragma unroll
   for (int t = 0; t < kRowsMaxTiles; ++t) {
     if (t < ntiles) {
@@ -317,9 +363,11 @@ inline int gemv_rows_gn_groups(int rows_per_block, int group_size) {
 }
 
 inline size_t gemv_rows_gn_lds_bytes(int nwaves, int mt, int K, int group_size, int rows_per_block,
-                                     bool asym) {
-  return (size_t)nwaves * mt * 256 * 4
-         + (size_t)(asym ? 2 : 1) * gemv_rows_gn_groups(rows_per_block, group_size) * K * 2;
+                                     bool asym, int bits = 4, bool xlds = false) {
+  size_t front = (size_t)nwaves * mt * 256 * 4;
+  const size_t xb = (size_t)nwaves * mt * 16 * ((bits == 4 ? 256 : 128) + 16);
+  if (xlds && xb > front) front = xb;
+  return front + (size_t)(asym ? 2 : 1) * gemv_rows_gn_groups(rows_per_block, group_size) * K * 2;
 }
 
 inline size_t gemv_rows_f32_gn_lds_bytes(int nwaves, int K, int group_size, int rows_per_block,

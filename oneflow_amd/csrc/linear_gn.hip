@@ -10,10 +10,10 @@
 namespace ofq {
 namespace {
 
-template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT>
+template<typename T, int BITS, bool SIGNED, int ZMODE, int NW, int MT, bool XLDS>
 int launch_gn_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m, int grid,
                    int rows_per_block, size_t lds) {
-  auto kern = gemv_rows_gn<T, BITS, SIGNED, ZMODE, NW, MT>;
+  auto kern = gemv_rows_gn<T, BITS, SIGNED, ZMODE, NW, MT, XLDS>;
   static std::atomic<uint64_t> lds_allowed{0};  // devices on which the kernel's LDS limit is raised
   if (!ofq_allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, lds_allowed)) return OFQ_ERR_LAUNCH;
   kern<<<grid, NW * 64, lds, st>>>(
@@ -24,13 +24,13 @@ int launch_gn_inst(hipStream_t st, const LinearArgs& a, const void* x, void* out
   return ofq_check_launch();
 }
 
-template<typename T, int NW, int MT>
+template<typename T, int NW, int MT, bool XLDS>
 int launch_gn_t(hipStream_t st, const LinearArgs& a, const void* x, void* out, int m, int grid,
                 int rpb, size_t lds) {
   const int zmode = !a.symmetric ? kZeroAsym : (a.w_signed ? kZeroNone : kZeroSymU);
 #define OFQ_R(B, SG, ZM)                              \
   if (a.bits == B && a.w_signed == SG && zmode == ZM) \
-    return launch_gn_inst<T, B, SG, ZM, NW, MT>(st, a, x, out, m, grid, rpb, lds);
+    return launch_gn_inst<T, B, SG, ZM, NW, MT, XLDS>(st, a, x, out, m, grid, rpb, lds);
   OFQ_R(4, true, kZeroNone)
   OFQ_R(4, false, kZeroSymU)
   OFQ_R(4, false, kZeroAsym)
@@ -65,17 +65,36 @@ int launch_gn_part(hipStream_t st, const LinearArgs& a, int64_t m0, int m) {
   const int mt = gn_mt(m);
   const int nw = gn_waves(mt);
   const int rpb = gn_rows_per_block(a, mt);
-  const size_t lds =
-      gemv_rows_gn_lds_bytes(nw, mt, (int)a.k, (int)a.group_size, rpb, !a.symmetric);
-  if (lds > 160u * 1024u) return OFQ_ERR_UNSUPPORTED;
   const int grid = (int)((a.n + rpb - 1) / rpb);
   const void* x = static_cast<const char*>(a.x) + (size_t)m0 * a.k * 2;
   void* out = static_cast<char*>(a.out) + (size_t)m0 * a.n * 2;
-#define OFQ_MT(TT_)                                                                   \
-  switch (mt) {                                                                       \
-    case 1: return launch_gn_t<TT_, 16, 1>(st, a, x, out, m, grid, rpb, lds);         \
-    case 2: return launch_gn_t<TT_, 16, 2>(st, a, x, out, m, grid, rpb, lds);         \
-    default: return launch_gn_t<TT_, 12, 4>(st, a, x, out, m, grid, rpb, lds);        \
+  // More than 16 rows of x: x through per-wave buffers in LDS when they fit beside the block's
+  // scale rows (12 / 8 waves for two / four tiles of x).  Up to 16 rows the direct requests
+  // touch few enough cache lines (11008 x 4096, fp16 with a zero point, 2 rows: 10.8 us direct,
+  // 12.1 us through the buffers; 32 rows: 19.5 against 15.0).
+  if (mt > 1) {
+    const int nwx = mt == 2 ? 12 : 8;
+    const size_t ldsx = gemv_rows_gn_lds_bytes(nwx, mt, (int)a.k, (int)a.group_size, rpb,
+                                               !a.symmetric, a.bits, true);
+    if (ldsx <= 160u * 1024u) {
+#define OFQ_MTX(TT_)                                                                       \
+  switch (mt) {                                                                            \
+    case 2: return launch_gn_t<TT_, 12, 2, true>(st, a, x, out, m, grid, rpb, ldsx);       \
+    default: return launch_gn_t<TT_, 8, 4, true>(st, a, x, out, m, grid, rpb, ldsx);       \
+  }
+      if (a.t_dtype == OFQ_BF16) { OFQ_MTX(bf16) }
+      OFQ_MTX(f16)
+#undef OFQ_MTX
+    }
+  }
+  const size_t lds =
+      gemv_rows_gn_lds_bytes(nw, mt, (int)a.k, (int)a.group_size, rpb, !a.symmetric);
+  if (lds > 160u * 1024u) return OFQ_ERR_UNSUPPORTED;
+#define OFQ_MT(TT_)                                                                          \
+  switch (mt) {                                                                              \
+    case 1: return launch_gn_t<TT_, 16, 1, false>(st, a, x, out, m, grid, rpb, lds);         \
+    case 2: return launch_gn_t<TT_, 16, 2, false>(st, a, x, out, m, grid, rpb, lds);         \
+    default: return launch_gn_t<TT_, 12, 4, false>(st, a, x, out, m, grid, rpb, lds);        \
   }
   if (a.t_dtype == OFQ_BF16) { OFQ_MT(bf16) }
   OFQ_MT(f16)
