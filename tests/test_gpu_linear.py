@@ -622,10 +622,12 @@ def test_decode_vocabulary_sized_n(t, m):
 @pytest.mark.parametrize("m,n,k,g", [(1, 512, 256, 512), (1, 4096, 1024, 128), (8, 1000, 512, 200),
                                      (16, 688, 256, 16), (17, 96, 128, 48), (40, 2048, 384, 64),
                                      (64, 320, 256, 32), (3, 11008, 128, 128), (1, 11008, 4096, 128),
-                                     (1, 1040, 11008, 16), (1, 4112, 5120, 2056)])
+                                     (1, 1040, 11008, 16), (1, 4112, 5120, 2056), (40, 256, 11008, 128),
+                                     (24, 4096, 1024, 128)])
 def test_groups_along_n_streaming(t, num_bits, m, n, k, g):
     """group_dim = 0 (scale / zero [n / g, k], one value per k): the streaming kernel that applies
-    a scale per element, through every container, 1, 2 and 4 tiles of x, groups from one 16-row
+    a scale per element, through every container, 1, 2 and 4 tiles of x (x through the waves'
+    LDS buffers beyond 16 rows; 40 rows of 11008 in two passes), groups from one 16-row
     tile to the whole weight, and n with a ragged last block; one row of x on fp16 / 4-bit /
     int8-container weights takes the kernel in which a wave owns whole rows and the scale meets x
     (rows of 128 bytes to 5.4 KB, groups of one block's rows and of many)."""
