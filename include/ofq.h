@@ -101,7 +101,10 @@ int ofq_groupwise_dequantize(void* stream, const void* in, const void* scale, co
  *   q*scale is never rounded to fp16; the result is closer to exact arithmetic and differs from
  *   the composition above by ~3e-4 rel-L2 (contract: 1e-3).  The same codes with groups along
  *   N (16 | group_size, 256 | k) at m = 1 take a kernel of that family in which the scale meets
- *   x instead (x*scale is rounded to fp16 once per k, q*scale never): the same ~3e-4.  Every
+ *   x instead (x*scale is rounded to fp16 once per k, q*scale never): the same ~3e-4.  Neither
+ *   kernel rescales x by a constant: x meets the codes as stored, and x*scale is brought to a
+ *   common power of two per 32 k before its rounding, so the bound holds for any magnitude of x
+ *   and of the scales whose outputs are normal halves (tested from 1e-3 to hundreds).  Every
  *   other combination (uint8 container, a zero term, 8 bit, bf16, fp32, m > 16, groups along N
  *   otherwise) forms w~ with the two roundings of groupwise_dequantize.  The same weights in the two containers can therefore
  *   differ in the last bits of the output.

@@ -173,14 +173,15 @@ gemv_f16_mfma(const f16* __restrict__ x, const uint8_t* __restrict__ w,
 //      flight, and kept in LDS; the waves then fetch ready-made operands with ds_read_b128
 //      (only the lanes of rows m < M read at all).  When M*K is too large for LDS (STAGED =
 //      false) each lane loads and permutes the x of its own k-slot instead.
-//  (2) The codes are never converted to their integer value.  The halves 0x6400|nibble are
-//      1024+u (low nibbles) and 1024+16u (high nibbles), u = q+8 after the xor that turns two's
-//      complement into offset binary (the xor is folded into the mask-and-merge, one v_bitop3).
-//      The x that meets high nibbles is pre-divided by 16 (exact in fp16 unless subnormal), so
-//      one MFMA accumulator collects
+//  (2) The codes are never converted to their integer value.  With u = q+8 (the xor that turns
+//      two's complement into offset binary is folded into the mask-and-merge, one v_bitop3) the
+//      half 0x6400|u is 1024+u for a low nibble (one ulp of [1024,2048) is 1) and the half
+//      0x5400|(u<<4) is 64+u for a high nibble left where it is (one ulp of [64,128) is 1/16, so
+//      mantissa bits 4..7 count in units of 1).  One MFMA accumulator collects
 //        acc = sum_k x q + 1032 * sum_lo x + 72 * sum_hi x
 //      and the constant part `corr` depends on (m, chunk) only: it is computed once per block
 //      when x is staged (or with two MFMAs against constant operands when x is not staged).
+//      x itself is used as stored (no rescaling, so no range of x is special).
 //      All products are exact in fp32; the cancellation is done per chunk of 128 k, where the
 //      partial sums are ~1e4 and fp32 resolves 1e-3 of a code unit.  The group scale multiplies
 //      the chunk result once (fp32), i.e. w~ = q*s is not rounded to fp16 first: the result is
@@ -207,7 +208,7 @@ __device__ __forceinline__ int row_of(int v, uint32_t inv) {
 }
 
 // x of one 16-k unit (two 128-bit words, natural order) -> low-nibble operand and high-nibble
-// operand, the latter divided by 16
+// operand
 __device__ __forceinline__ void permute_unit(const u32x4 a, const u32x4 b, u32x4& lo, u32x4& hi) {
   lo[0] = __builtin_amdgcn_perm(a[2], a[0], 0x07060302u);  // (x1, x5)
   lo[1] = __builtin_amdgcn_perm(a[3], a[1], 0x07060302u);  // (x3, x7)
@@ -217,9 +218,6 @@ __device__ __forceinline__ void permute_unit(const u32x4 a, const u32x4 b, u32x4
   hi[1] = __builtin_amdgcn_perm(a[3], a[1], 0x05040100u);  // (x2, x6)
   hi[2] = __builtin_amdgcn_perm(b[2], b[0], 0x05040100u);  // (x8, x12)
   hi[3] = __builtin_amdgcn_perm(b[3], b[1], 0x05040100u);  // (x10, x14)
-  const f16x2 sixteenth = {(f16)0.0625f, (f16)0.0625f};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) hi[i] = as_u32(as_h2(hi[i]) * sixteenth);
 }
 
 // 1032 * (sum of the low-nibble x) + 72 * (sum of the high-nibble x) of one permuted unit
@@ -231,7 +229,7 @@ __device__ __forceinline__ float unit_corr(const u32x4 lo, const u32x4 hi) {
     sl += (float)l[0] + (float)l[1];
     sh += (float)h[0] + (float)h[1];
   }
-  return 1032.0f * sl + 1152.0f * sh;  // hi carries x/16: 72 * 16 = 1152
+  return 1032.0f * sl + 72.0f * sh;
 }
 
 __device__ __forceinline__ float unit_corr_of(const u32x4 a, const u32x4 b) {
@@ -370,9 +368,9 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const int xrec_stride = has_x ? 256 : 0;
   const f16* xrow = x + (int64_t)(has_x ? r : 0) * K + kb * 32;
   const f16* slr = sl + r * G;
-  const f16 c_lo = (f16)1032.0f, c_hi = (f16)1152.0f;
+  const f16 c_lo = (f16)1032.0f, c_hi = (f16)72.0f;
   const f16x8 k1032 = {c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo};
-  const f16x8 k1152 = {c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi};
+  const f16x8 k72 = {c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi};
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
 
@@ -421,10 +419,10 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
           blo[1] = (w0s & 0x000F000Fu) ^ 0x64086408u;
           blo[2] = (w1 & 0x000F000Fu) ^ 0x64086408u;
           blo[3] = (w1s & 0x000F000Fu) ^ 0x64086408u;
-          bhi[0] = (w0 & 0x00F000F0u) ^ 0x64806480u;
-          bhi[1] = (w0s & 0x00F000F0u) ^ 0x64806480u;
-          bhi[2] = (w1 & 0x00F000F0u) ^ 0x64806480u;
-          bhi[3] = (w1s & 0x00F000F0u) ^ 0x64806480u;
+          bhi[0] = (w0 & 0x00F000F0u) ^ 0x54805480u;
+          bhi[1] = (w0s & 0x00F000F0u) ^ 0x54805480u;
+          bhi[2] = (w1 & 0x00F000F0u) ^ 0x54805480u;
+          bhi[3] = (w1s & 0x00F000F0u) ^ 0x54805480u;
           const f16x8 a_lo = __builtin_bit_cast(f16x8, xa[2 * h]);
           const f16x8 a_hi = __builtin_bit_cast(f16x8, xa[2 * h + 1]);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, __builtin_bit_cast(f16x8, blo), acc,
@@ -433,7 +431,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
                                                        0, 0, 0);
           if (!STAGED) {
             corr = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, k1032, corr, 0, 0, 0);
-            corr = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, k1152, corr, 0, 0, 0);
+            corr = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, k72, corr, 0, 0, 0);
           }
         }
 #pragma unroll
@@ -865,10 +863,10 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
           blo[1] = (w0s & 0x000F000Fu) ^ 0x64086408u;
           blo[2] = (w1 & 0x000F000Fu) ^ 0x64086408u;
           blo[3] = (w1s & 0x000F000Fu) ^ 0x64086408u;
-          bhi[0] = (w0 & 0x00F000F0u) ^ 0x64806480u;
-          bhi[1] = (w0s & 0x00F000F0u) ^ 0x64806480u;
-          bhi[2] = (w1 & 0x00F000F0u) ^ 0x64806480u;
-          bhi[3] = (w1s & 0x00F000F0u) ^ 0x64806480u;
+          bhi[0] = (w0 & 0x00F000F0u) ^ 0x54805480u;
+          bhi[1] = (w0s & 0x00F000F0u) ^ 0x54805480u;
+          bhi[2] = (w1 & 0x00F000F0u) ^ 0x54805480u;
+          bhi[3] = (w1s & 0x00F000F0u) ^ 0x54805480u;
           acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h]),
                                                        __builtin_bit_cast(f16x8, blo), acc, 0, 0, 0);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h + 1]),

@@ -22,8 +22,8 @@
 //   - x is permuted into the order the nibble masks deliver the codes ONCE per block, into LDS,
 //     laid out lane-major, and every wave copies it to registers while the weights are in
 //     flight.
-// Arithmetic as in gemv_kernels.h: 0x6400|nibble is the half 1032+q (low nibbles) or 1152+16q
-// (high nibbles, met by x/16); the constant part per lane, 1032*sum_lo(x) + 72*sum_hi(x), is
+// Arithmetic as in gemv_kernels.h: the half 0x6400|nibble is 1032+q (low nibbles), the half
+// 0x5400|nibble<<4 is 72+q (high nibbles); the constant part per lane, 1032*sum_lo(x) + 72*sum_hi(x), is
 // computed at staging and seeds the accumulator negated; products are exact in fp32, the group
 // scale multiplies the lane's fp32 sum (w~ = q*s is not rounded to fp16).
 #pragma once
@@ -41,8 +41,8 @@ struct M1Shape {
   int gn;      // groups along N (GN kernels): rows per group, a multiple of rows_per_block
 };
 
-// LDS: [x operands H x 4 pieces x 64 lanes x 16 B] [corr H x 64 f32]
-inline size_t gemv_m1_lds_bytes(int H) { return (size_t)H * 4096 + (size_t)H * 256; }
+// LDS: [x operands H x 4 pieces x 64 lanes x 16 B] [corr H x 64 f32] [GN: power of two H x 64 f32]
+inline size_t gemv_m1_lds_bytes(int H) { return (size_t)H * 4096 + (size_t)H * 512; }
 
 template<int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
@@ -75,10 +75,10 @@ __device__ __forceinline__ float m1_dot32(const u32x4 wq, const u32x4 (&xa)[4], 
     blo[1] = (w0s & 0x000F000Fu) ^ 0x64086408u;
     blo[2] = (w1 & 0x000F000Fu) ^ 0x64086408u;
     blo[3] = (w1s & 0x000F000Fu) ^ 0x64086408u;
-    bhi[0] = (w0 & 0x00F000F0u) ^ 0x64806480u;
-    bhi[1] = (w0s & 0x00F000F0u) ^ 0x64806480u;
-    bhi[2] = (w1 & 0x00F000F0u) ^ 0x64806480u;
-    bhi[3] = (w1s & 0x00F000F0u) ^ 0x64806480u;
+    bhi[0] = (w0 & 0x00F000F0u) ^ 0x54805480u;
+    bhi[1] = (w0s & 0x00F000F0u) ^ 0x54805480u;
+    bhi[2] = (w1 & 0x00F000F0u) ^ 0x54805480u;
+    bhi[3] = (w1s & 0x00F000F0u) ^ 0x54805480u;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       acc = __builtin_amdgcn_fdot2(as_h2(blo[e]), as_h2(xa[2 * h][e]), acc, false);
@@ -105,8 +105,9 @@ struct M1Glu {
 // thread at staging; NM = 1, or 2 for the GLU (hidden and gate).
 // GN: groups run along N (scale [N / gn, K], one value per k, shared by the gn rows of a group;
 // a block's rows lie in one group).  The scale then meets x instead of the codes: the block
-// stages x * s (one fp16 rounding per k, where the reference rounds q * s per element) and the
-// rows need no scale of their own.
+// stages x * s (one fp16 rounding per k, where the reference rounds q * s per element; a power of
+// two per lane piece keeps the rounded value a normal half) and the rows need no scale of their
+// own.
 template<int NW, int RPW, int H, int XU, int NM, bool GN = false>
 __device__ __forceinline__ void
 m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
@@ -198,15 +199,40 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
     if (wave * 64 + i * NTH >= nunits) break;  // wave-uniform
     const int u = tid + i * NTH;
     const bool ok = u < nunits;
+    float unscale = 1.f;
     if (GN) {
+      // x * s is exact in fp32.  The 32 products of a lane's piece (this unit and its
+      // neighbour's) are brought to a common power of two that puts the largest in [2^12, 2^13)
+      // before the one rounding to fp16, so that no product of ordinary size lands among the
+      // subnormal halves whatever the magnitudes of x and s; the inverse power multiplies the
+      // lane's fp32 sum.
+      float v[2][8];
+      float amax = 0.f;
 #pragma unroll
       for (int p2 = 0; p2 < 2; ++p2) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           // (each word through a scalar of its own, see dequant8_b4_v)
-          const uint32_t xw = xu[i][p2][e];
-          const uint32_t sw = su[GN ? i : 0][p2][e];
-          xu[i][p2][e] = as_u32(as_h2(xw) * as_h2(sw));
+          const uint32_t xw_u = xu[i][p2][e];
+          const uint32_t sw_u = su[GN ? i : 0][p2][e];
+          const f16x2 xw = as_h2(xw_u);
+          const f16x2 sw = as_h2(sw_u);
+          v[p2][2 * e] = (float)xw[0] * (float)sw[0];
+          v[p2][2 * e + 1] = (float)xw[1] * (float)sw[1];
+          amax = fmaxf(amax, fmaxf(fabsf(v[p2][2 * e]), fabsf(v[p2][2 * e + 1])));
+        }
+      }
+      amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+      const int eb = (__builtin_bit_cast(int, amax) >> 23) & 0xFF;  // 0 (zero), or 79 .. 159
+      const bool live = eb >= 64 && eb < 192;
+      const float up = live ? __builtin_bit_cast(float, (266 - eb) << 23) : 1.f;    // 2^(12 - e)
+      unscale = live ? __builtin_bit_cast(float, (eb - 12) << 23) : 1.f;            // 2^(e - 12)
+#pragma unroll
+      for (int p2 = 0; p2 < 2; ++p2) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const f16x2 r = {(f16)(v[p2][2 * e] * up), (f16)(v[p2][2 * e + 1] * up)};
+          xu[i][p2][e] = as_u32(r);
         }
       }
     }
@@ -219,7 +245,10 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
     }
     float cpart = ok ? unit_corr(lo, hi) : 0.f;
     cpart += __shfl_xor(cpart, 1, 64);
-    if (ok && p == 0) corr_l[h * 64 + l] = -cpart;
+    if (ok && p == 0) {
+      corr_l[h * 64 + l] = -cpart;
+      if (GN) corr_l[(H + h) * 64 + l] = unscale;
+    }
   }
   __syncthreads();
 
@@ -243,7 +272,7 @@ m1_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
 #pragma unroll
       for (int i = 0; i < RPW; ++i) {
         const float acc = m1_dot32(wq[q][i][h], xa, cr);
-        const float term = GN ? acc : acc * (float)sc[q][i][h];
+        const float term = acc * (GN ? corr_l[(H + h) * 64 + lane] : (float)sc[q][i][h]);
         tot[q][i] += valid[h] ? term : 0.f;
       }
     }

@@ -118,6 +118,39 @@ def test_decode_few_rows_of_x_long_and_ragged_rows(m, n, k, g, with_bias):
     assert r < 5e-4
 
 
+@pytest.mark.parametrize("x_std,s_lo,s_hi", [
+    (1e-2, 1e-3, 1e-2), (1e-3, 1e-3, 1e-2), (1e-2, 1e-4, 1e-3), (1.0, 1e-4, 1e-3),
+    (3e-3, 1e-4, 1e-3), (100.0, 1e-4, 2e-4), (30.0, 1e-4, 1e-3),
+])
+@pytest.mark.parametrize("m,group_dim,n,k,g", [
+    (1, 1, 4096, 4096, 128), (1, 1, 1024, 11008, 128), (1, 1, 11008, 2048, 256),
+    (1, 0, 4096, 4096, 128), (1, 0, 1024, 11008, 64), (1, 0, 512, 512, 16),
+    (4, 1, 4096, 4096, 128), (8, 1, 1024, 11008, 128), (2, 1, 11008, 1024, 128),
+    (16, 1, 300, 4096, 128), (4, 0, 1024, 4096, 128),
+])
+def test_decode_does_not_depend_on_the_magnitude_of_x_or_of_the_scales(x_std, s_lo, s_hi, m,
+                                                                       group_dim, n, k, g):
+    """The contract holds for any magnitude of x and of the scales the output type can carry
+    (the reference's arithmetic does not depend on it): activations of 1e-3, scales of 1e-4,
+    activations of hundreds (with scales that keep the outputs near 10, where the absolute bound
+    of 2e-2 still is the tighter of the two).  fp16, symmetric int4 in an int8 container, both group directions;
+    no bias, so that the bound is on the product itself.  A tenth of every row of x is another
+    hundred times smaller, so that large and small values meet inside one group."""
+    rng = np.random.default_rng(int(x_std * 1e6) + int(s_lo * 1e7) + m * 7 + group_dim + n + k)
+    xf = rng.standard_normal((m, k)).astype(np.float32) * x_std
+    xf[:, rng.random(k) < 0.1] *= 0.01
+    x = H.as_T(xf, "f16")
+    codes = rng.integers(-8, 8, size=(n, k)).astype(np.int8)
+    w = H.pack_int4(codes)
+    sshape = (n, k // g) if group_dim == 1 else (n // g, k)
+    scale = H.as_T(rng.uniform(s_lo, s_hi, size=sshape).astype(np.float32), "f16")
+    ref = O.fused_linear(x, w, scale, None, None, 4, True, group_dim, g)
+    assert np.abs(O.to_f32(ref)).mean() > 6.2e-5, "outputs must be normal halves for the bound to mean something"
+    got = _run(x, w, scale, None, None, 4, True, group_dim, g)
+    r, e = H.assert_linear_parity(got, ref, "f16", f"x~{x_std} s~{s_lo} m={m} dim={group_dim} {n}x{k}")
+    assert r < 5e-4
+
+
 @pytest.mark.parametrize("m", [1, 8])
 def test_same_weights_in_both_containers_differ_by_rounding_of_w_only(m):
     """The same symmetric 4-bit weights stored as int8 codes q and as uint8 codes q + 7: the int8
