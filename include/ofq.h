@@ -63,6 +63,14 @@ typedef enum { OFQ_FORMULA_GOOGLE = 0, OFQ_FORMULA_CAMBRICON = 1 } ofq_formula;
  *   OFQ_ZP_UINT8     rounded to uint8 first (the rule of the CPU kernels,
  *                    oneflow/user/kernels/quantization_kernel.cpp:41-43). */
 typedef enum { OFQ_ZP_FLOAT = 0, OFQ_ZP_UINT8 = 1 } ofq_zp_mode;
+/* how LayerNorm takes the mean and the variance of a row:
+ *   OFQ_LN_STATS_FP32  accumulated in fp32 (the reference's precision,
+ *                      oneflow/core/cuda/layer_norm.cuh:212-233; the last bit of mean / inv then
+ *                      depends on the order of summation, there as here)
+ *   OFQ_LN_STATS_FP64  accumulated in fp64 and rounded once: the correctly rounded fp32 mean and
+ *                      inv of the row, whatever the order -- y, scale and the codes made from them
+ *                      are then reproducible bit for bit by any implementation of the same rule */
+typedef enum { OFQ_LN_STATS_FP32 = 0, OFQ_LN_STATS_FP64 = 1 } ofq_ln_statistics;
 
 const char* ofq_status_string(int status);
 /* library ABI version; bumped on any signature change */
@@ -226,6 +234,18 @@ int ofq_fused_skip_layer_norm_min_max_observer(void* stream, const void* x, cons
                                                float* zero_point, int t_dtype, int64_t rows,
                                                int64_t cols, double epsilon, int quantization_bit,
                                                void* workspace, size_t workspace_bytes);
+
+/*
+ * The two ops above with the precision of the row statistics as an attribute (ofq_ln_statistics).
+ * No reference interface (the ops themselves are absent there).  with_skip = 0: the plain op
+ * (bias, skip, alpha ignored); with_skip != 0: the skip_layer_norm input.  OFQ_LN_STATS_FP32 runs
+ * the same kernels as the entry points above.
+ */
+int ofq_fused_layer_norm_min_max_observer_stats(
+    void* stream, const void* x, const void* bias, const void* skip, double alpha, int with_skip,
+    const void* gamma, const void* beta, void* y, float* scale, float* zero_point, int t_dtype,
+    int64_t rows, int64_t cols, double epsilon, int quantization_bit, int statistics,
+    void* workspace, size_t workspace_bytes);
 
 /*
  * groupwise_quantize: the producer of the weight format of the two ops above.

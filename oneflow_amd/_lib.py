@@ -15,6 +15,7 @@ F32, F16, BF16, F64, I8, U8 = 0, 1, 2, 3, 4, 5
 SCHEME = {"symmetric": 0, "affine": 1}
 FORMULA = {"google": 0, "cambricon": 1}
 ZP_MODE = {"float": 0, "uint8": 1}
+LN_STATS_FP32, LN_STATS_FP64 = 0, 1
 
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -44,6 +45,9 @@ SIGNATURES = {
     "ofq_fused_skip_layer_norm_min_max_observer": (_i, [_vp, _vp, _vp, _vp, ctypes.c_double, _vp,
                                                         _vp, _vp, _vp, _vp, _i, _i64, _i64,
                                                         ctypes.c_double, _i, _vp, _sz]),
+    "ofq_fused_layer_norm_min_max_observer_stats": (_i, [_vp, _vp, _vp, _vp, ctypes.c_double, _i,
+                                                         _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64,
+                                                         ctypes.c_double, _i, _i, _vp, _sz]),
     "ofq_grouped_linear_gq": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _i64]),
     "ofq_fused_glu_gq": (_i, [_vp] * 13 + [_i, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64]),

@@ -73,26 +73,52 @@ struct SkipArgs {
   float alpha;
 };
 
+// T((x - mean) * inv) as the reference forms it: the fp32 product, rounded to fp32, is narrowed
+// to T (layer_norm.cuh stores through static_cast).  The empty asm keeps the two roundings
+// apart: fused into v_fma_mixlo_f16 the product would be rounded to fp16 once, which differs in
+// about one element of 30000.
+template<typename T>
+__device__ __forceinline__ float normalised(float d, float inv) {
+  float p = d * inv;
+  if constexpr (TT<T>::dtype == OFQ_F16) asm volatile("" : "+v"(p));
+  return TT<T>::round(p);
+}
+
 template<typename T>
 __device__ __forceinline__ float skip_sum(float x, float b, float s, float alpha) {
   return TT<T>::round(TT<T>::round(x + b) + TT<T>::round(s * alpha));
 }
 
+// EXACT statistics: the row sum and the squared deviations from the unrounded mean are taken in
+// fp64 (a sum of fp16 / bf16 values of ordinary range is exact there in any order, the squares
+// carry errors of 1e-16), and mean and inv are each rounded once to the fp32 values the
+// normalisation uses -- the correctly rounded statistics of the row, independent of the order of
+// summation.  The fp32 statistics (the default) depend on that order in the last bit, as the
+// reference's own do.  The cost is three fp64 operations per element and pass.
+__device__ __forceinline__ float exact_inv(double m2, double n, double eps) {
+  double var = m2 / n;
+  if (var < 0.0) var = 0.0;
+  return (float)(1.0 / __builtin_sqrt(var + eps));
+}
+
 // NP = packs of 8 elements each lane caches; cols <= kLnBlock * 8 * NP and 8 | cols.
-template<typename T, int NP, bool SKIP>
+template<typename T, int NP, bool SKIP, bool EXACT>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
                  const typename TT<T>::storage* __restrict__ gamma,
                  const typename TT<T>::storage* __restrict__ beta,
                  typename TT<T>::storage* __restrict__ y, float* __restrict__ row_absmax,
-                 int64_t cols, float eps, SkipArgs<T> sk) {
+                 int64_t cols, double eps64, SkipArgs<T> sk) {
   __shared__ float smem[kLnBlock / kWave];
+  __shared__ double smem64[EXACT ? kLnBlock / kWave : 1];
+  const float eps = (float)eps64;
   const int64_t row = blockIdx.x;
   const typename TT<T>::storage* xr = x + row * cols;
   typename TT<T>::storage* yr = y + row * cols;
   const int npacks = (int)(cols / 8);
   float v[NP][8];
   float sum = 0.0f;
+  double sum64 = 0.0;
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
     const int p = threadIdx.x + i * kLnBlock;
@@ -107,26 +133,50 @@ ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
         for (int e = 0; e < 8; ++e) v[i][e] = skip_sum<T>(v[i][e], bb[e], ss[e], sk.alpha);
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sum += v[i][e];
-    }
-  }
-  sum = block_reduce(sum, OpSum(), smem);
-  const float mean = sum / (float)cols;
-  float m2 = 0.0f;
-#pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    const int p = threadIdx.x + i * kLnBlock;
-    if (p < npacks) {
-#pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float d = v[i][e] - mean;
-        m2 = __builtin_fmaf(d, d, m2);
+        if constexpr (EXACT) sum64 += (double)v[i][e];
+        else sum += v[i][e];
       }
     }
   }
-  m2 = block_reduce(m2, OpSum(), smem);
-  const float var = fmaxf(m2 / (float)cols, 0.0f);
-  const float inv = 1.0f / __builtin_sqrtf(var + eps);
+  float mean, inv;
+  if constexpr (EXACT) {
+    sum64 = block_reduce(sum64, OpSum(), smem64);
+    const double mean64 = sum64 / (double)cols;
+    double q = 0.0;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = threadIdx.x + i * kLnBlock;
+      if (p < npacks) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const double d = (double)v[i][e] - mean64;
+          q = __builtin_fma(d, d, q);
+        }
+      }
+    }
+    q = block_reduce(q, OpSum(), smem64);
+    mean = (float)mean64;
+    inv = exact_inv(q, (double)cols, eps64);
+  } else {
+    sum = block_reduce(sum, OpSum(), smem);
+    mean = sum / (float)cols;
+    float m2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = threadIdx.x + i * kLnBlock;
+      if (p < npacks) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = v[i][e] - mean;
+          m2 = __builtin_fmaf(d, d, m2);
+        }
+      }
+    }
+    m2 = block_reduce(m2, OpSum(), smem);
+    const float var = fmaxf(m2 / (float)cols, 0.0f);
+    inv = 1.0f / __builtin_sqrtf(var + eps);
+  }
   float amax = 0.0f;
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
@@ -137,7 +187,7 @@ ln_observer_rows(const typename TT<T>::storage* __restrict__ x,
       if (beta) load8<T>(beta + (int64_t)p * 8, b);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float t = TT<T>::round((v[i][e] - mean) * inv);
+        float t = normalised<T>(v[i][e] - mean, inv);
         if (gamma) t = TT<T>::round(t * g[e]);
         if (beta) t = TT<T>::round(t + b[e]);
         else if (gamma) t = t + 0.0f;  // the reference adds its default beta 0: -0 becomes +0
@@ -211,13 +261,14 @@ __device__ __forceinline__ RawPack<T> narrow(const float* f) {
 // x, gamma and beta are all requested before anything is waited for and stay in registers in
 // storage format (half the registers of fp32 for the 16-bit types), so the row's critical path
 // holds one memory round trip, not two.
-template<typename T, int NP, bool SKIP>
+template<typename T, int NP, bool SKIP, bool EXACT>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
                       const typename TT<T>::storage* __restrict__ gamma,
                       const typename TT<T>::storage* __restrict__ beta,
                       typename TT<T>::storage* __restrict__ y, float* __restrict__ wave_absmax,
-                      int64_t rows, int64_t cols, float eps, SkipArgs<T> sk) {
+                      int64_t rows, int64_t cols, double eps64, SkipArgs<T> sk) {
+  const float eps = (float)eps64;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t gw = (int64_t)blockIdx.x * (kLnBlock / kWave) + (threadIdx.x >> 6);
   const int64_t nwaves = (int64_t)gridDim.x * (kLnBlock / kWave);
@@ -272,38 +323,72 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
       }
       first = false;
     }
-    float sum = 0.0f;
+    float mean, inv;
+    if constexpr (EXACT) {
+      double sum64 = 0.0;
 #pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int p = lane + i * kWave;
-      if (p < npacks) {
-        // (plain widen-and-add: a chain of v_dot2_f32_f16 on one accumulator came out of the
-        // compiler with the same source register in every link)
-        float f[8];
-        widen<T>(v[i], f);
+      for (int i = 0; i < NP; ++i) {
+        const int p = lane + i * kWave;
+        if (p < npacks) {
+          float f[8];
+          widen<T>(v[i], f);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sum += f[e];
-      }
-    }
-    sum = wave_reduce(sum, OpSum());
-    const float mean = sum / (float)cols;
-    float m2 = 0.0f;
-#pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int p = lane + i * kWave;
-      if (p < npacks) {
-        float f[8];
-        widen<T>(v[i], f);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float d = f[e] - mean;
-          m2 = __builtin_fmaf(d, d, m2);
+          for (int e = 0; e < 8; ++e) sum64 += (double)f[e];
         }
       }
+      sum64 = wave_reduce(sum64, OpSum());
+      const double mean64 = sum64 / (double)cols;
+      double q = 0.0;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const int p = lane + i * kWave;
+        if (p < npacks) {
+          float f[8];
+          widen<T>(v[i], f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const double d = (double)f[e] - mean64;
+            q = __builtin_fma(d, d, q);
+          }
+        }
+      }
+      q = wave_reduce(q, OpSum());
+      mean = (float)mean64;
+      inv = exact_inv(q, (double)cols, eps64);
+    } else {
+      float sum = 0.0f;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const int p = lane + i * kWave;
+        if (p < npacks) {
+          // (plain widen-and-add: a chain of v_dot2_f32_f16 on one accumulator came out of the
+          // compiler with the same source register in every link)
+          float f[8];
+          widen<T>(v[i], f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) sum += f[e];
+        }
+      }
+      sum = wave_reduce(sum, OpSum());
+      mean = sum / (float)cols;
+      float m2 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const int p = lane + i * kWave;
+        if (p < npacks) {
+          float f[8];
+          widen<T>(v[i], f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float d = f[e] - mean;
+            m2 = __builtin_fmaf(d, d, m2);
+          }
+        }
+      }
+      m2 = wave_reduce(m2, OpSum());
+      const float var = fmaxf(m2 / (float)cols, 0.0f);
+      inv = 1.0f / __builtin_sqrtf(var + eps);
     }
-    m2 = wave_reduce(m2, OpSum());
-    const float var = fmaxf(m2 / (float)cols, 0.0f);
-    const float inv = 1.0f / __builtin_sqrtf(var + eps);
     f16x8 amax8 = {(f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f};
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
@@ -329,7 +414,7 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
           if (beta) widen<T>(br[i], b);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            float t = TT<T>::round((f[e] - mean) * inv);
+            float t = normalised<T>(f[e] - mean, inv);
             if (gamma) t = TT<T>::round(t * g[e]);
             if (beta) t = TT<T>::round(t + b[e]);
             else if (gamma) t = t + 0.0f;  // default beta 0 of the reference: -0 -> +0
@@ -359,13 +444,14 @@ ln_observer_wave_rows(const typename TT<T>::storage* __restrict__ x,
 // SKIP: the normalised row is (x + bias[c]) + skip * T(alpha) (see the top of the file), formed
 // as the row arrives and kept in storage format in place of x; the next row is then not
 // requested ahead (LOOP must be false), the registers hold the residual inputs instead.
-template<typename T, int NP, bool LOOP, bool SKIP = false>
+template<typename T, int NP, bool LOOP, bool SKIP, bool EXACT>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
                       const typename TT<T>::storage* __restrict__ gamma,
                       const typename TT<T>::storage* __restrict__ beta,
                       typename TT<T>::storage* __restrict__ y, float* __restrict__ wave_absmax,
-                      int64_t rows, float eps, SkipArgs<T> sk = SkipArgs<T>()) {
+                      int64_t rows, double eps64, SkipArgs<T> sk) {
+  const float eps = (float)eps64;
   static_assert(sizeof(typename TT<T>::storage) == 2, "16-bit types only");
   static_assert(!(SKIP && LOOP), "the residual variant does not prefetch");
   constexpr int kCols = NP * 512;
@@ -446,12 +532,16 @@ ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
     }
     float f[NP][8];
     float sum = 0.0f;
+    double sum64 = 0.0;
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
       RawPack<T> rp;
       rp.q[0] = cur[i];
       widen<T>(rp, f[i]);
-      if constexpr (TT<T>::dtype == OFQ_F16) {
+      if constexpr (EXACT) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum64 += (double)f[i][e];
+      } else if constexpr (TT<T>::dtype == OFQ_F16) {
         // (1, 1) held in a register: with the constant as a literal operand the compiler emits
         // the four dot products of a pack with one and the same source register
         uint32_t ones_bits = 0x3c003c00u;
@@ -469,20 +559,39 @@ ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
         for (int e = 0; e < 8; ++e) sum += f[i][e];
       }
     }
-    sum = wave_reduce(sum, OpSum());
-    const float mean = sum / (float)kCols;
-    float m2 = 0.0f;
+    float mean, inv;
+    if constexpr (EXACT) {
+      sum64 = wave_reduce(sum64, OpSum());
+      const double mean64 = sum64 / (double)kCols;
+      mean = (float)mean64;
+      double q = 0.0;
 #pragma unroll
-    for (int i = 0; i < NP; ++i) {
+      for (int i = 0; i < NP; ++i) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        f[i][e] = f[i][e] - mean;
-        m2 = __builtin_fmaf(f[i][e], f[i][e], m2);
+        for (int e = 0; e < 8; ++e) {
+          const double d = (double)f[i][e] - mean64;
+          q = __builtin_fma(d, d, q);
+          f[i][e] = f[i][e] - mean;
+        }
       }
+      q = wave_reduce(q, OpSum());
+      inv = exact_inv(q, (double)kCols, eps64);
+    } else {
+      sum = wave_reduce(sum, OpSum());
+      mean = sum / (float)kCols;
+      float m2 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          f[i][e] = f[i][e] - mean;
+          m2 = __builtin_fmaf(f[i][e], f[i][e], m2);
+        }
+      }
+      m2 = wave_reduce(m2, OpSum());
+      const float var = fmaxf(m2 / (float)kCols, 0.0f);
+      inv = 1.0f / __builtin_sqrtf(var + eps);
     }
-    m2 = wave_reduce(m2, OpSum());
-    const float var = fmaxf(m2 / (float)kCols, 0.0f);
-    const float inv = 1.0f / __builtin_sqrtf(var + eps);
     typename TT<T>::storage* yr = y + row * kCols + lane * 8;
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
@@ -508,7 +617,7 @@ ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
         widen<T>(bp, b);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          float t = TT<T>::round(f[i][e] * inv);
+          float t = normalised<T>(f[i][e], inv);
           t = TT<T>::round(t * g[e]);
           t = TT<T>::round(t + b[e]);
           o[e] = t;
@@ -534,14 +643,16 @@ ln_observer_wave_full(const typename TT<T>::storage* __restrict__ x,
 
 // any cols: three passes over the row through L2 (the row was just read, so only the first
 // pass touches HBM), scalar accesses.
-template<typename T, bool SKIP>
+template<typename T, bool SKIP, bool EXACT>
 __global__ void __launch_bounds__(kLnBlock)
 ln_observer_rows_generic(const typename TT<T>::storage* __restrict__ x,
                          const typename TT<T>::storage* __restrict__ gamma,
                          const typename TT<T>::storage* __restrict__ beta,
                          typename TT<T>::storage* __restrict__ y, float* __restrict__ row_absmax,
-                         int64_t cols, float eps, SkipArgs<T> sk) {
+                         int64_t cols, double eps64, SkipArgs<T> sk) {
   __shared__ float smem[kLnBlock / kWave];
+  __shared__ double smem64[EXACT ? kLnBlock / kWave : 1];
+  const float eps = (float)eps64;
   const int64_t row = blockIdx.x;
   const typename TT<T>::storage* xr = x + row * cols;
   typename TT<T>::storage* yr = y + row * cols;
@@ -552,21 +663,37 @@ ln_observer_rows_generic(const typename TT<T>::storage* __restrict__ x,
     const float sv = sk.skip ? TT<T>::load(sk.skip + row * cols + c) : 0.f;
     return skip_sum<T>(xv, bv, sv, sk.alpha);
   };
-  float sum = 0.0f;
-  for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) sum += input(c);
-  sum = block_reduce(sum, OpSum(), smem);
-  const float mean = sum / (float)cols;
-  float m2 = 0.0f;
-  for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
-    const float d = input(c) - mean;
-    m2 = __builtin_fmaf(d, d, m2);
+  float mean, inv;
+  if constexpr (EXACT) {
+    double sum64 = 0.0;
+    for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) sum64 += (double)input(c);
+    sum64 = block_reduce(sum64, OpSum(), smem64);
+    const double mean64 = sum64 / (double)cols;
+    double q = 0.0;
+    for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
+      const double d = (double)input(c) - mean64;
+      q = __builtin_fma(d, d, q);
+    }
+    q = block_reduce(q, OpSum(), smem64);
+    mean = (float)mean64;
+    inv = exact_inv(q, (double)cols, eps64);
+  } else {
+    float sum = 0.0f;
+    for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) sum += input(c);
+    sum = block_reduce(sum, OpSum(), smem);
+    mean = sum / (float)cols;
+    float m2 = 0.0f;
+    for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
+      const float d = input(c) - mean;
+      m2 = __builtin_fmaf(d, d, m2);
+    }
+    m2 = block_reduce(m2, OpSum(), smem);
+    const float var = fmaxf(m2 / (float)cols, 0.0f);
+    inv = 1.0f / __builtin_sqrtf(var + eps);
   }
-  m2 = block_reduce(m2, OpSum(), smem);
-  const float var = fmaxf(m2 / (float)cols, 0.0f);
-  const float inv = 1.0f / __builtin_sqrtf(var + eps);
   float amax = 0.0f;
   for (int64_t c = threadIdx.x; c < cols; c += kLnBlock) {
-    float t = TT<T>::round((input(c) - mean) * inv);
+    float t = normalised<T>(input(c) - mean, inv);
     if (gamma) t = TT<T>::round(t * TT<T>::load(gamma + c));
     if (beta) t = TT<T>::round(t + TT<T>::load(beta + c));
     else if (gamma) t = t + 0.0f;  // default beta 0 of the reference: -0 -> +0
@@ -613,9 +740,9 @@ float round_to_T_host(float v) {
   return v;
 }
 
-template<typename T, bool SKIP>
+template<typename T, bool SKIP, bool EXACT>
 int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, void* y,
-           float* scale, float* zero_point, int64_t rows, int64_t cols, float eps, int bits,
+           float* scale, float* zero_point, int64_t rows, int64_t cols, double eps, int bits,
            float* ws, const void* bias, const void* skip, double alpha) {
   typedef typename TT<T>::storage S;
   const S* xs = static_cast<const S*>(x);
@@ -648,13 +775,14 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
       nparts = waves;
 #define OFQ_LN_FULL(NPV)                                                                        \
   if (SKIP) {                                                                                    \
-    ln_observer_wave_full<T, NPV, false, SKIP><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws,    \
-                                                                          rows, eps, sk);        \
+    ln_observer_wave_full<T, NPV, false, SKIP, EXACT><<<grid, kLnBlock, 0, st>>>(                \
+        xs, gs, bs, ys, ws, rows, eps, sk);                                                      \
   } else if (loop) {                                                                             \
-    ln_observer_wave_full<T, NPV, true><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, eps); \
+    ln_observer_wave_full<T, NPV, true, false, EXACT><<<grid, kLnBlock, 0, st>>>(                \
+        xs, gs, bs, ys, ws, rows, eps, sk);                                                      \
   } else {                                                                                       \
-    ln_observer_wave_full<T, NPV, false><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows,    \
-                                                                    eps);                        \
+    ln_observer_wave_full<T, NPV, false, false, EXACT><<<grid, kLnBlock, 0, st>>>(               \
+        xs, gs, bs, ys, ws, rows, eps, sk);                                                      \
   }
       switch (np) {
         case 1: OFQ_LN_FULL(1) break;
@@ -679,8 +807,8 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
     const int grid = (int)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
     nparts = (int64_t)grid * kWavesPerBlock < rows ? (int64_t)grid * kWavesPerBlock : rows;
 #define OFQ_LN_WAVE(NPV)                                                                       \
-  ln_observer_wave_rows<T, NPV, SKIP><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, cols, \
-                                                                 eps, sk)
+  ln_observer_wave_rows<T, NPV, SKIP, EXACT><<<grid, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, rows, \
+                                                                        cols, eps, sk)
     if (npacks <= kWave) {
       OFQ_LN_WAVE(1);
     } else if (npacks <= 2 * kWave) {
@@ -692,15 +820,15 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
     }
 #undef OFQ_LN_WAVE
   } else if (vec_ok && npacks <= kLnBlock) {
-    ln_observer_rows<T, 1, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
+    ln_observer_rows<T, 1, SKIP, EXACT><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else if (vec_ok && npacks <= 2 * kLnBlock) {
-    ln_observer_rows<T, 2, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
+    ln_observer_rows<T, 2, SKIP, EXACT><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else if (vec_ok && npacks <= 4 * kLnBlock) {
-    ln_observer_rows<T, 4, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
+    ln_observer_rows<T, 4, SKIP, EXACT><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else if (vec_ok && npacks <= 8 * kLnBlock) {
-    ln_observer_rows<T, 8, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
+    ln_observer_rows<T, 8, SKIP, EXACT><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols, eps, sk);
   } else {
-    ln_observer_rows_generic<T, SKIP><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols,
+    ln_observer_rows_generic<T, SKIP, EXACT><<<(int)rows, kLnBlock, 0, st>>>(xs, gs, bs, ys, ws, cols,
                                                                       eps, sk);
   }
   ln_observer_finalize<<<1, kWave, 0, st>>>(ws, nparts, bits, scale, zero_point);
@@ -710,8 +838,10 @@ int launch(hipStream_t st, const void* x, const void* gamma, const void* beta, v
 int run(void* stream, const void* x, const void* bias, const void* skip, double alpha,
         bool with_skip, const void* gamma, const void* beta, void* y, float* scale,
         float* zero_point, int t_dtype, int64_t rows, int64_t cols, double epsilon,
-        int quantization_bit, void* workspace, size_t workspace_bytes) {
+        int quantization_bit, int statistics, void* workspace, size_t workspace_bytes) {
   OFQ_RETURN_IF(quantization_bit <= 1 || quantization_bit > 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(statistics != OFQ_LN_STATS_FP32 && statistics != OFQ_LN_STATS_FP64,
+                OFQ_ERR_BAD_ATTR);
   OFQ_RETURN_IF(t_dtype != OFQ_F16 && t_dtype != OFQ_BF16 && t_dtype != OFQ_F32,
                 OFQ_ERR_BAD_DTYPE);
   OFQ_RETURN_IF(rows < 1 || cols < 1 || rows > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
@@ -721,18 +851,22 @@ int run(void* stream, const void* x, const void* bias, const void* skip, double 
                 OFQ_ERR_WORKSPACE);
   hipStream_t st = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
-  const float eps = (float)epsilon;
-#define OFQ_LN_RUN(T)                                                                          \
-  return with_skip ? launch<T, true>(st, x, gamma, beta, y, scale, zero_point, rows, cols, eps, \
-                                     quantization_bit, ws, bias, skip, alpha)                  \
-                   : launch<T, false>(st, x, gamma, beta, y, scale, zero_point, rows, cols,    \
-                                      eps, quantization_bit, ws, nullptr, nullptr, 0.0)
+  const double eps = epsilon;  // (the fp32 statistics round it to fp32 in the kernel)
+#define OFQ_LN_RUN2(T, EX)                                                                     \
+  return with_skip ? launch<T, true, EX>(st, x, gamma, beta, y, scale, zero_point, rows, cols, \
+                                         eps, quantization_bit, ws, bias, skip, alpha)         \
+                   : launch<T, false, EX>(st, x, gamma, beta, y, scale, zero_point, rows,      \
+                                          cols, eps, quantization_bit, ws, nullptr, nullptr, 0.0)
+#define OFQ_LN_RUN(T)                                    \
+  if (statistics == OFQ_LN_STATS_FP64) OFQ_LN_RUN2(T, true); \
+  OFQ_LN_RUN2(T, false)
   switch (t_dtype) {
     case OFQ_F16: OFQ_LN_RUN(f16);
     case OFQ_BF16: OFQ_LN_RUN(bf16);
     default: OFQ_LN_RUN(float);
   }
 #undef OFQ_LN_RUN
+#undef OFQ_LN_RUN2
 }
 
 // device address of `scratch` on the current device, looked up once per device
@@ -771,7 +905,7 @@ extern "C" int ofq_fused_layer_norm_min_max_observer_static(void* stream, const 
   // every partial the finalize kernel reads is written by the row kernel of the same call, so
   // nothing has to be cleared between calls
   return ofq::run(stream, x, nullptr, nullptr, 0.0, false, gamma, beta, y, scale, zero_point,
-                  t_dtype, rows, cols, epsilon, quantization_bit, ws,
+                  t_dtype, rows, cols, epsilon, quantization_bit, OFQ_LN_STATS_FP32, ws,
                   (size_t)OFQ_LN_STATIC_MAX_ROWS * sizeof(float));
 }
 
@@ -787,7 +921,8 @@ extern "C" int ofq_fused_layer_norm_min_max_observer(void* stream, const void* x
                                                      int quantization_bit, void* workspace,
                                                      size_t workspace_bytes) {
   return ofq::run(stream, x, nullptr, nullptr, 0.0, false, gamma, beta, y, scale, zero_point,
-                  t_dtype, rows, cols, epsilon, quantization_bit, workspace, workspace_bytes);
+                  t_dtype, rows, cols, epsilon, quantization_bit, OFQ_LN_STATS_FP32, workspace,
+                  workspace_bytes);
 }
 
 extern "C" int ofq_fused_skip_layer_norm_min_max_observer(
@@ -796,5 +931,17 @@ extern "C" int ofq_fused_skip_layer_norm_min_max_observer(
     int64_t rows, int64_t cols, double epsilon, int quantization_bit, void* workspace,
     size_t workspace_bytes) {
   return ofq::run(stream, x, bias, skip, alpha, true, gamma, beta, y, scale, zero_point, t_dtype,
-                  rows, cols, epsilon, quantization_bit, workspace, workspace_bytes);
+                  rows, cols, epsilon, quantization_bit, OFQ_LN_STATS_FP32, workspace,
+                  workspace_bytes);
+}
+
+extern "C" int ofq_fused_layer_norm_min_max_observer_stats(
+    void* stream, const void* x, const void* bias, const void* skip, double alpha, int with_skip,
+    const void* gamma, const void* beta, void* y, float* scale, float* zero_point, int t_dtype,
+    int64_t rows, int64_t cols, double epsilon, int quantization_bit, int statistics,
+    void* workspace, size_t workspace_bytes) {
+  return ofq::run(stream, x, with_skip ? bias : nullptr, with_skip ? skip : nullptr,
+                  with_skip ? alpha : 0.0, with_skip != 0, gamma, beta, y, scale, zero_point,
+                  t_dtype, rows, cols, epsilon, quantization_bit, statistics, workspace,
+                  workspace_bytes);
 }

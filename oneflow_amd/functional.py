@@ -510,9 +510,13 @@ def _fake_quantization_forward(in_, scale, zero_point, quantization_formula, qua
 # --------------------------------------------------------------------------------------------
 # Ops named by the task but absent from the reference tree
 # --------------------------------------------------------------------------------------------
-def fused_layer_norm_min_max_observer(x, gamma=None, beta=None, epsilon=1e-5, quantization_bit=8):
+def fused_layer_norm_min_max_observer(x, gamma=None, beta=None, epsilon=1e-5, quantization_bit=8,
+                                      *, exact_statistics=False):
     """LayerNorm over the last axis + per-tensor symmetric observer of the result.
-    Returns ``(y, scale, zero_point)`` with fp32 ``scale`` / ``zero_point`` of shape ``[1]``."""
+    Returns ``(y, scale, zero_point)`` with fp32 ``scale`` / ``zero_point`` of shape ``[1]``.
+    ``exact_statistics``: mean and variance of a row accumulated in fp64 and rounded once (the
+    correctly rounded fp32 statistics, independent of the order of summation) instead of
+    accumulated in fp32."""
     _check(1 < quantization_bit <= 8, "quantization_bit should be in range (1, 8].")
     _check(x.dtype in (torch.float16, torch.bfloat16, torch.float32),
            f"no fused_layer_norm_min_max_observer kernel for dtype {x.dtype}")
@@ -530,15 +534,22 @@ def fused_layer_norm_min_max_observer(x, gamma=None, beta=None, epsilon=1e-5, qu
     L = _lib.lib()
     ws_bytes = L.ofq_fused_layer_norm_min_max_observer_workspace_bytes(_dt(x), rows, cols)
     ws = _workspace(ws_bytes, x.device)
-    st = L.ofq_fused_layer_norm_min_max_observer(
-        _stream(x), _ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(scale), _ptr(zero_point),
-        _dt(x), rows, cols, float(epsilon), quantization_bit, _ptr(ws), ws_bytes)
+    if exact_statistics:
+        st = L.ofq_fused_layer_norm_min_max_observer_stats(
+            _stream(x), _ptr(x), None, None, 0.0, 0, _ptr(gamma), _ptr(beta), _ptr(y),
+            _ptr(scale), _ptr(zero_point), _dt(x), rows, cols, float(epsilon), quantization_bit,
+            _lib.LN_STATS_FP64, _ptr(ws), ws_bytes)
+    else:
+        st = L.ofq_fused_layer_norm_min_max_observer(
+            _stream(x), _ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(scale), _ptr(zero_point),
+            _dt(x), rows, cols, float(epsilon), quantization_bit, _ptr(ws), ws_bytes)
     _lib.check("ofq_fused_layer_norm_min_max_observer", st)
     return y, scale, zero_point
 
 
 def fused_skip_layer_norm_min_max_observer(x, gamma=None, beta=None, bias=None, skip=None,
-                                           epsilon=1e-5, alpha=1e1, quantization_bit=8):
+                                           epsilon=1e-5, alpha=1e1, quantization_bit=8,
+                                           *, exact_statistics=False):
     """``skip_layer_norm`` (same arguments and defaults as the reference functional,
     functional_api.yaml:1545-1546: the row normalised is ``(x + bias) + skip * alpha`` in the
     dtype of x) + per-tensor symmetric observer of the result.  Returns
@@ -564,10 +575,16 @@ def fused_skip_layer_norm_min_max_observer(x, gamma=None, beta=None, bias=None, 
     L = _lib.lib()
     ws_bytes = L.ofq_fused_layer_norm_min_max_observer_workspace_bytes(_dt(x), rows, cols)
     ws = _workspace(ws_bytes, x.device)
-    st = L.ofq_fused_skip_layer_norm_min_max_observer(
-        _stream(x), _ptr(x), _ptr(bias), _ptr(skip), float(alpha), _ptr(gamma), _ptr(beta),
-        _ptr(y), _ptr(scale), _ptr(zero_point), _dt(x), rows, cols, float(epsilon),
-        quantization_bit, _ptr(ws), ws_bytes)
+    if exact_statistics:
+        st = L.ofq_fused_layer_norm_min_max_observer_stats(
+            _stream(x), _ptr(x), _ptr(bias), _ptr(skip), float(alpha), 1, _ptr(gamma),
+            _ptr(beta), _ptr(y), _ptr(scale), _ptr(zero_point), _dt(x), rows, cols,
+            float(epsilon), quantization_bit, _lib.LN_STATS_FP64, _ptr(ws), ws_bytes)
+    else:
+        st = L.ofq_fused_skip_layer_norm_min_max_observer(
+            _stream(x), _ptr(x), _ptr(bias), _ptr(skip), float(alpha), _ptr(gamma), _ptr(beta),
+            _ptr(y), _ptr(scale), _ptr(zero_point), _dt(x), rows, cols, float(epsilon),
+            quantization_bit, _ptr(ws), ws_bytes)
     _lib.check("ofq_fused_skip_layer_norm_min_max_observer", st)
     return y, scale, zero_point
 
