@@ -248,6 +248,14 @@ def test_dynamic_quantize_and_matmul_quant():
     assert np.array_equal(got.view(np.uint16), expect.view(np.uint16))
     ref = O.matmul_quant(a_np[rows], w[cols], H.to_numpy(s), w_scale[cols], None, np.float16)
     assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+    # every one of the 22.5 M outputs: the integer sums are exact in an fp64 matmul on all host
+    # cores (|acc| < 2^27), the epilogue is one int -> fp32 conversion, one fp32 product and one
+    # rounding to fp16; this composition is pinned by the oracle on the sample above
+    acc_all = (torch.from_numpy(a_np).double() @ torch.from_numpy(w).double().t())
+    sc_all = torch.from_numpy((H.to_numpy(s)[0] * w_scale).astype(np.float32))
+    expect_all = (acc_all.to(torch.int32).to(torch.float32) * sc_all[None, :]).to(torch.float16).numpy()
+    assert np.array_equal(expect_all[np.ix_(rows, cols)].view(np.uint16), ref.view(np.uint16))
+    assert np.array_equal(out.view(np.uint16), expect_all.view(np.uint16))
 
 
 @pytest.mark.parametrize("m,n,k,t", [(1, 16, 128, "f32"), (100, 200, 256, "f16"), (130, 33, 384, "bf16")])

@@ -371,6 +371,64 @@ def test_prefill_w8a16_sampled(t):
     assert np.array_equal(O.to_f32(got2), O.to_f32(got) * 2.0)
 
 
+def _composition_on_all_cores(x, w, scale, zero, g, t):
+    """The dequantize -> matmul composition at full size as torch CPU tensor operations on every
+    host core: w~ = T(T(q) * s) + z with one rounding per operation (a bf16 / fp16 tensor product
+    or sum rounds once, from the exact fp32 value), then an fp32 matmul, rounded to T."""
+    import torch
+    td = {"bf16": torch.bfloat16, "f16": torch.float16}[t]
+    n, k = w.shape
+    q = torch.from_numpy(w.astype(np.float32)).to(td).view(n, k // g, g)
+    s = H.to_torch(scale, "cpu").view(n, k // g, 1)
+    z = H.to_torch(zero, "cpu").view(n, k // g, 1)
+    wt = ((q * s) + z).view(n, k).float()
+    out = H.to_torch(x, "cpu").float() @ wt.t()
+    return H.to_numpy(out.to(td))
+
+
+@pytest.mark.parametrize("t", ["bf16", "f16"])
+def test_prefill_w8a16_full_shape_every_output_both_paths(t):
+    """Config 4 at full size (x [2048,4096], W uint8 asymmetric [11008,4096], g = 64) through the
+    C ABI twice: with the op's tmp_buffer (weight dequantised once, copy-fed GEMM) and with
+    workspace = NULL (weight tiles dequantised inside the GEMM).  EVERY output of both is held to
+    the contract against the composition computed on all host cores, which is itself checked
+    against the scalar oracle on sampled rows and columns; the two paths differ from each other
+    by fp32 summation order only."""
+    import torch
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    tcode = {"bf16": _lib.BF16, "f16": _lib.F16}[t]
+    m, n, k, g = 2048, 11008, 4096, 64
+    x = H.as_T(H.rng_for(4, 0).standard_normal((m, k)).astype(np.float32), t)
+    w = H.rng_for(4, 1).integers(0, 256, size=(n, k), dtype=np.uint8)
+    scale = H.as_T(H.rng_for(4, 2).uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float32), t)
+    zero = H.as_T(H.rng_for(4, 3).uniform(120, 136, size=(n, k // g)).astype(np.float32), t)
+    xt, wt, st, zt = map(H.to_torch, (x, w, scale, zero))
+    need = L.ofq_fused_linear_gq_workspace_bytes(_lib.U8, tcode, 8, 0, 1, g, m, n, k)
+    assert need == n * k * 2
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    outs = []
+    for wptr, wbytes in ((ws.data_ptr(), need), (None, 0)):
+        out = torch.empty((m, n), dtype=xt.dtype, device="cuda")
+        rc = L.ofq_fused_linear_gq(torch.cuda.current_stream().cuda_stream, xt.data_ptr(),
+                                   wt.data_ptr(), st.data_ptr(), zt.data_ptr(), None,
+                                   out.data_ptr(), _lib.U8, tcode, 8, 0, 1, g, m, n, k, wptr, wbytes)
+        assert rc == 0
+        torch.cuda.synchronize()
+        outs.append(H.to_numpy(out))
+    full = _composition_on_all_cores(x, w, scale, zero, g, t)
+    rows = np.array([0, 1, 127, 128, 255, 256, 1000, 1023, 1024, 2047])
+    cols = np.concatenate([np.arange(0, 40), np.arange(5000, 5040), np.arange(n - 40, n)])
+    ref = O.fused_linear(x[rows], w[cols], scale[cols], zero[cols], None, 8, False, 1, g)
+    # the all-cores composition against the oracle: same w~, same fp32 products, only the order
+    # of the fp32 sum differs (one ulp of T where the sum falls next to a rounding boundary)
+    assert H.rel_l2(O.to_f32(full[np.ix_(rows, cols)]), O.to_f32(ref)) < 2e-4
+    for name, got in (("tmp_buffer", outs[0]), ("workspace NULL", outs[1])):
+        H.assert_linear_parity(got[np.ix_(rows, cols)], ref, t, f"prefill {t} {name} vs oracle")
+        H.assert_linear_parity(got, full, t, f"prefill {t} {name}, all 22.5 M outputs")
+    assert H.rel_l2(O.to_f32(outs[1]), O.to_f32(outs[0])) < 1e-3
+
+
 @pytest.mark.parametrize("m", [17, 100, 130])
 @pytest.mark.parametrize("num_bits,symmetric,qdt", [(4, True, np.int8), (4, False, np.uint8),
                                                     (8, True, np.uint8)])
