@@ -152,8 +152,16 @@ __device__ __forceinline__ float div_of_half_value(float a, float b, float y) {
     if (cond) return (status);      \
   } while (0)
 
+// The runtime's record of a failed launch is read (and thereby cleared) here; it is kept for the
+// caller's own asynchronous-error query (ofq_hip_get_async_error, hip_shim.hip).
+namespace ofq {
+void note_launch_error(int hip_error);
+}
 static inline int ofq_check_launch() {
-  return hipGetLastError() == hipSuccess ? OFQ_OK : OFQ_ERR_LAUNCH;
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return OFQ_OK;
+  ofq::note_launch_error((int)e);
+  return OFQ_ERR_LAUNCH;
 }
 static inline bool ofq_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -27,6 +27,7 @@
 #include "oneflow/core/kernel/cuda_graph_support.h"
 
 #include "ofq.h"
+#include "ofq_hip_shim.h"
 
 namespace oneflow {
 
@@ -34,8 +35,9 @@ namespace {
 
 // OneFlow hands out the raw device stream through ep::CudaStream::cuda_stream()
 // (oneflow/core/ep/cuda/cuda_stream.h:91, the call of groupwise_quantization_kernels.cu:531); on
-// a ROCm build of the EP layer that handle IS the hipStream_t.  The standalone build carries the
-// same two headers with the same spelling, so this source is one text for both builds.
+// this device that handle IS the hipStream_t: ep_hip/oneflow/core/ep/cuda/cuda_stream.{h,cpp} is
+// ep::CudaStream over a HIP stream, under the reference's include path and spelling, so this
+// source is one text for a OneFlow tree and for the stand-alone build.
 inline void* RawStream(user_op::KernelComputeContext* ctx) {
   return ctx->stream()->As<ep::CudaStream>()->cuda_stream();
 }
@@ -52,8 +54,12 @@ inline int ToOfq(DataType dt) {
   }
 }
 
+// Argument errors end the process like the CHECKs of the kernels these replace.  A failed launch
+// does not: the reference's kernels do not test their launches either, the runtime asks the
+// stream after Compute (CHECK_JUST(stream->GetAsyncError()), stateful_opkernel.cpp:1007), and the
+// library keeps the device runtime's error for that query.
 inline void CheckOk(int status, const char* what) {
-  if (status != OFQ_OK) {
+  if (status != OFQ_OK && status != OFQ_ERR_LAUNCH) {
     std::cerr << what << ": " << ofq_status_string(status) << "\n";
     CHECK_EQ(status, OFQ_OK);
   }
@@ -587,7 +593,96 @@ const user_op::KernelRegistration* Lookup(const std::string& op, const user_op::
   }
   return best;
 }
+
+int CurrentDevice() {
+  int dev = 0;
+  if (ofq_hip_get_device(&dev) != 0) dev = 0;
+  return dev;
+}
+
+// the message of the last failed GetAsyncError of a hook, for ofq_plugin_last_async_error
+thread_local std::string g_last_async_error;
+
+// What the runtime does around a kernel (stateful_opkernel.cpp:1006-1007): Compute, then ask the
+// stream for an asynchronous error.  The runtime aborts on one (CHECK_JUST); the hooks return -2
+// and keep the message so that a test can look at it.
+int ComputeLikeTheRuntime(const user_op::OpKernel& kernel, user_op::KernelComputeContext* ctx) {
+  kernel.Compute(ctx, nullptr, nullptr);
+  const Maybe<void> err = ctx->stream()->GetAsyncError();
+  if (err.IsOk()) return 0;
+  g_last_async_error = err.error_message();
+  return -2;
+}
+
+int CopyOut(const std::string& text, char* msg, int cap) {
+  if (msg != nullptr && cap > 0) {
+    int j = 0;
+    for (; j < (int)text.size() && j < cap - 1; ++j) msg[j] = text[j];
+    msg[j] = 0;
+  }
+  return (int)text.size();
+}
 }  // namespace
+
+extern "C" int ofq_plugin_last_async_error(char* msg, int cap) {
+  return CopyOut(g_last_async_error, msg, cap);
+}
+
+// ---- ep::CudaStream / ep::CudaEvent through C hooks ---------------------------------------------
+extern "C" void* ofq_plugin_stream_new(int device) { return new ep::CudaStream(device); }
+extern "C" void* ofq_plugin_stream_view(int device, void* raw) {
+  return new ep::CudaStream(device, raw);
+}
+extern "C" void ofq_plugin_stream_delete(void* s) { delete static_cast<ep::CudaStream*>(s); }
+extern "C" void* ofq_plugin_stream_raw(void* s) {
+  // the way a kernel reaches it: through the base class and As<>
+  ep::Stream* base = static_cast<ep::CudaStream*>(s);
+  return base->As<ep::CudaStream>()->cuda_stream();
+}
+extern "C" int ofq_plugin_stream_device_type(void* s) {
+  return (int)static_cast<ep::Stream*>(static_cast<ep::CudaStream*>(s))->device_type();
+}
+extern "C" int ofq_plugin_stream_sync(void* s, char* msg, int cap) {
+  const Maybe<void> r = static_cast<ep::Stream*>(static_cast<ep::CudaStream*>(s))->Sync();
+  if (r.IsOk()) return 0;
+  CopyOut(r.error_message(), msg, cap);
+  return -1;
+}
+extern "C" int ofq_plugin_stream_get_async_error(void* s, char* msg, int cap) {
+  const Maybe<void> r = static_cast<ep::Stream*>(static_cast<ep::CudaStream*>(s))->GetAsyncError();
+  if (r.IsOk()) return 0;
+  CopyOut(r.error_message(), msg, cap);
+  return -1;
+}
+extern "C" int ofq_plugin_stream_on_execution_context_setup(void* s) {
+  ep::Stream* base = static_cast<ep::CudaStream*>(s);
+  return base->OnExecutionContextSetup().IsOk() && base->OnExecutionContextTeardown().IsOk() ? 0 : -1;
+}
+extern "C" int ofq_plugin_stream_cu_count(void* s) {
+  return static_cast<ep::CudaStream*>(s)->multi_processor_count();
+}
+extern "C" unsigned ofq_plugin_stream_grid_with_waves(void* s, size_t elem_cnt, size_t block_size,
+                                                      size_t max_waves) {
+  ep::CudaLaunchConfig config;
+  static_cast<ep::CudaStream*>(s)->InitLaunchConfigWithWaves(&config, elem_cnt, block_size, max_waves);
+  return config.grid_dim;
+}
+extern "C" void* ofq_plugin_event_new() { return new ep::CudaEvent(0); }
+extern "C" void ofq_plugin_event_delete(void* e) { delete static_cast<ep::CudaEvent*>(e); }
+extern "C" void ofq_plugin_stream_record_event(void* s, void* e) {
+  static_cast<ep::Stream*>(static_cast<ep::CudaStream*>(s))->RecordEvent(static_cast<ep::CudaEvent*>(e));
+}
+extern "C" void ofq_plugin_stream_wait_event(void* s, void* e) {
+  static_cast<ep::Stream*>(static_cast<ep::CudaStream*>(s))->WaitEvent(static_cast<ep::CudaEvent*>(e));
+}
+// 1 done, 0 pending, -1 error
+extern "C" int ofq_plugin_event_query_done(void* e) {
+  const Maybe<bool> r = static_cast<ep::Event*>(static_cast<ep::CudaEvent*>(e))->QueryDone();
+  return r.IsOk() ? (r.value() ? 1 : 0) : -1;
+}
+extern "C" int ofq_plugin_event_sync(void* e) {
+  return static_cast<ep::Event*>(static_cast<ep::CudaEvent*>(e))->Sync().IsOk() ? 0 : -1;
+}
 
 extern "C" int ofq_plugin_registration_count() { return (int)user_op::KernelRegistry().size(); }
 
@@ -659,7 +754,7 @@ extern "C" int ofq_plugin_run_fused_linear(void* stream, void* x, void* w, void*
   c.arg_dtypes["out"] = (DataType)t_dtype;
   const auto* r = Lookup("fused_linear_with_groupwise_quantized_weight", c);
   if (r == nullptr) return -1;
-  ep::CudaStream st(stream);
+  ep::CudaStream st(CurrentDevice(), stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   const DataType T = (DataType)t_dtype;
@@ -680,8 +775,7 @@ extern "C" int ofq_plugin_run_fused_linear(void* stream, void* x, void* w, void*
   ctx.attrs["group_dim"].i = group_dim;
   ctx.attrs["group_size"].i = group_size;
   auto kernel = r->create();
-  kernel->Compute(&ctx, nullptr, nullptr);
-  return 0;
+  return ComputeLikeTheRuntime(*kernel, &ctx);
 }
 // Runs the registered dynamic-int8 front end (LayerNorm + observer, with the optional residual
 // inputs) through a KernelComputeContext.
@@ -695,7 +789,7 @@ extern "C" int ofq_plugin_run_layer_norm_observer(void* stream, void* x, void* g
   c.arg_dtypes["y"] = (DataType)t_dtype;
   const auto* r = Lookup("fused_layer_norm_min_max_observer", c);
   if (r == nullptr) return -1;
-  ep::CudaStream st(stream);
+  ep::CudaStream st(CurrentDevice(), stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   const DataType T = (DataType)t_dtype;
@@ -712,8 +806,7 @@ extern "C" int ofq_plugin_run_layer_norm_observer(void* stream, void* x, void* g
   ctx.attrs["alpha"].f = alpha;
   ctx.attrs["quantization_bit"].i = bits;
   auto kernel = r->create();
-  kernel->Compute(&ctx, nullptr, nullptr);
-  return 0;
+  return ComputeLikeTheRuntime(*kernel, &ctx);
 }
 
 extern "C" int ofq_plugin_run_matmul_quant(void* stream, void* a, void* b, void* a_scale,
@@ -724,7 +817,7 @@ extern "C" int ofq_plugin_run_matmul_quant(void* stream, void* a, void* b, void*
   c.arg_dtypes["out"] = (DataType)out_dtype;
   const auto* r = Lookup("matmul_quant", c);
   if (r == nullptr) return -1;
-  ep::CudaStream st(stream);
+  ep::CudaStream st(CurrentDevice(), stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   ctx.AddTensor("a", {m, k}, DataType::kInt8, a);
@@ -734,8 +827,7 @@ extern "C" int ofq_plugin_run_matmul_quant(void* stream, void* a, void* b, void*
   if (bias) ctx.AddTensor("bias", {n}, (DataType)out_dtype, bias);
   ctx.AddTensor("out", {m, n}, (DataType)out_dtype, out);
   auto kernel = r->create();
-  kernel->Compute(&ctx, nullptr, nullptr);
-  return 0;
+  return ComputeLikeTheRuntime(*kernel, &ctx);
 }
 
 // q/k/v-style grouped call: `count` problems sharing x ([m,k]) with weights [ns[i], k*bits/8]
@@ -749,7 +841,7 @@ extern "C" int ofq_plugin_run_grouped_linear(void* stream, int count, void* x, v
   c.arg_dtypes["ys"] = (DataType)t_dtype;
   const auto* r = Lookup("grouped_linear_with_groupwise_quantized_weight", c);
   if (r == nullptr) return -1;
-  ep::CudaStream st(stream);
+  ep::CudaStream st(CurrentDevice(), stream);
   user_op::KernelComputeContext ctx;
   ctx.stream_ = &st;
   const DataType T = (DataType)t_dtype;
@@ -764,7 +856,6 @@ extern "C" int ofq_plugin_run_grouped_linear(void* stream, int count, void* x, v
   ctx.attrs["group_dim"].i = 1;
   ctx.attrs["group_size"].i = group_size;
   auto kernel = r->create();
-  kernel->Compute(&ctx, nullptr, nullptr);
-  return 0;
+  return ComputeLikeTheRuntime(*kernel, &ctx);
 }
 #endif  // OFQ_PLUGIN_STANDALONE

@@ -6,6 +6,9 @@
 //   oneflow/core/framework/user_op_kernel_registry.h:60-107, user_op_registry_manager.h:107-110
 //   oneflow/core/framework/user_op_hob.h:43-73           (HobDeviceType, HobDataType)
 //   oneflow/core/ep/include/stream.h:30-57               (ep::Stream)
+//   oneflow/core/ep/include/event.h:26-35                (ep::Event)
+//   oneflow/core/common/maybe.h, error.h                 (Maybe<void>, Maybe<bool>, Error: what
+//                                                         the stream layer constructs and tests)
 // When building against a real OneFlow tree this directory is simply left off the include path.
 #pragma once
 
@@ -15,6 +18,7 @@
 #include <iostream>
 #include <map>
 #include <memory>
+#include <sstream>
 #include <string>
 #include <utility>
 #include <vector>
@@ -56,10 +60,81 @@ class ShapeView {
   std::vector<int64_t> dims_;
 };
 
+// Error::RuntimeError() << "text" converts to a failed Maybe, Maybe<T>::Ok() / a value to a good
+// one; IsOk() is what callers test (CHECK_JUST aborts with the message otherwise).
+class Error {
+ public:
+  static Error RuntimeError() { return Error(); }
+  template<typename V>
+  Error&& operator<<(const V& v) && {
+    std::ostringstream os;
+    os << v;
+    msg_ += os.str();
+    return std::move(*this);
+  }
+  const std::string& msg() const { return msg_; }
+
+ private:
+  std::string msg_;
+};
+template<typename T>
+class Maybe;
+template<>
+class Maybe<void> {
+ public:
+  static Maybe Ok() { return Maybe(); }
+  Maybe(Error&& e) : ok_(false), msg_(e.msg()) {}  // NOLINT
+  bool IsOk() const { return ok_; }
+  const std::string& error_message() const { return msg_; }
+
+ private:
+  Maybe() : ok_(true) {}
+  bool ok_;
+  std::string msg_;
+};
+template<>
+class Maybe<bool> {
+ public:
+  Maybe(bool v) : ok_(true), value_(v) {}             // NOLINT
+  Maybe(Error&& e) : ok_(false), value_(false), msg_(e.msg()) {}  // NOLINT
+  bool IsOk() const { return ok_; }
+  bool value() const { return value_; }
+  const std::string& error_message() const { return msg_; }
+
+ private:
+  bool ok_;
+  bool value_;
+  std::string msg_;
+};
+#define CHECK_JUST(expr)                                                       \
+  do {                                                                         \
+    auto ofq_maybe_ = (expr);                                                  \
+    if (!ofq_maybe_.IsOk()) {                                                  \
+      std::cerr << "CHECK_JUST failed: " << ofq_maybe_.error_message() << "\n"; \
+      std::abort();                                                            \
+    }                                                                          \
+  } while (0)
+
 namespace ep {
+class Event {
+ public:
+  Event() = default;
+  virtual ~Event() = default;
+  virtual Maybe<bool> QueryDone() = 0;
+  virtual Maybe<void> Sync() = 0;
+};
+
 class Stream {
  public:
+  Stream() = default;
   virtual ~Stream() = default;
+  virtual DeviceType device_type() const = 0;
+  virtual Maybe<void> Sync() = 0;
+  virtual void RecordEvent(Event* event) = 0;
+  virtual void WaitEvent(Event*) { UNIMPLEMENTED(); }
+  virtual Maybe<void> GetAsyncError() { return Maybe<void>::Ok(); }
+  virtual Maybe<void> OnExecutionContextSetup() { return Maybe<void>::Ok(); }
+  virtual Maybe<void> OnExecutionContextTeardown() { return Maybe<void>::Ok(); }
   // oneflow/core/ep/include/stream.h:53-56: the device-specific stream is reached by a cast
   template<typename T>
   T* As() {

@@ -36,6 +36,19 @@ def test_header_symbols_are_exported_and_prototyped(lib):
     assert b"unknown" in lib.ofq_status_string(99)
 
 
+def test_stream_layer_symbols_are_exported(lib):
+    """include/ofq_hip_shim.h: the device / stream / event calls behind ep::CudaStream."""
+    text = open(os.path.join(ROOT, "include", "ofq_hip_shim.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(ofq_hip_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) == 16
+    raw = ctypes.CDLL(lib._name)
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in ofq_hip_shim.h but not exported"
+    raw.ofq_hip_error_string.restype = ctypes.c_char_p
+    assert raw.ofq_hip_error_string(0) == b"no error"
+
+
 # a fake, suitably aligned, never dereferenced device address
 P = ctypes.c_void_p(0x10000)
 U = ctypes.c_void_p(0x10008)  # not 16-byte aligned

@@ -175,3 +175,134 @@ def test_grouped_linear_through_the_adapter(plugin):
     torch.cuda.synchronize()
     for o, w in zip(outs, want):
         assert torch.equal(o, w)
+
+
+def _bind_stream_hooks(plugin):
+    vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    protos = {
+        "ofq_plugin_stream_new": (vp, [ci]), "ofq_plugin_stream_view": (vp, [ci, vp]),
+        "ofq_plugin_stream_delete": (None, [vp]), "ofq_plugin_stream_raw": (vp, [vp]),
+        "ofq_plugin_stream_device_type": (ci, [vp]),
+        "ofq_plugin_stream_sync": (ci, [vp, ctypes.c_char_p, ci]),
+        "ofq_plugin_stream_get_async_error": (ci, [vp, ctypes.c_char_p, ci]),
+        "ofq_plugin_stream_on_execution_context_setup": (ci, [vp]),
+        "ofq_plugin_stream_cu_count": (ci, [vp]),
+        "ofq_plugin_stream_grid_with_waves": (ctypes.c_uint, [vp, sz, sz, sz]),
+        "ofq_plugin_event_new": (vp, []), "ofq_plugin_event_delete": (None, [vp]),
+        "ofq_plugin_stream_record_event": (None, [vp, vp]),
+        "ofq_plugin_stream_wait_event": (None, [vp, vp]),
+        "ofq_plugin_event_query_done": (ci, [vp]), "ofq_plugin_event_sync": (ci, [vp]),
+        "ofq_plugin_last_async_error": (ci, [ctypes.c_char_p, ci]),
+    }
+    for name, (res, args) in protos.items():
+        f = getattr(plugin, name)
+        f.restype, f.argtypes = res, args
+
+
+def test_stream_hooks_are_exported(plugin):
+    _bind_stream_hooks(plugin)
+
+
+@pytest.mark.gpu
+def test_hip_stream_behind_ep_cuda_stream(plugin):
+    """ep::CudaStream / ep::CudaEvent over HIP (oneflow_amd/plugin/ep_hip): a stream of its own,
+    a registered kernel run on it through a KernelComputeContext, RecordEvent / QueryDone / Sync,
+    WaitEvent from a second stream, the CU count and the launch-size helper built on it, and
+    OnExecutionContextSetup."""
+    import torch
+    import helpers as H
+    import oneflow_amd as flow
+    _bind_stream_hooks(plugin)
+    dev = torch.cuda.current_device()
+    rng = np.random.default_rng(21)
+    m, n, k, g = 1, 2048, 4096, 128
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    w = H.pack_int4(rng.integers(-7, 8, size=(n, k)).astype(np.int8))
+    scale = rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float16)
+    xt, wt, st = map(H.to_torch, (x, w, scale))
+    direct = flow._C.fused_linear_with_groupwise_quantized_weight(
+        xt, wt, st, num_bits=4, symmetric=True, group_dim=1, group_size=g)
+    torch.cuda.synchronize()
+    s1 = plugin.ofq_plugin_stream_new(dev)
+    s2 = plugin.ofq_plugin_stream_new(dev)
+    ev = plugin.ofq_plugin_event_new()
+    try:
+        assert plugin.ofq_plugin_stream_device_type(s1) == K_CUDA
+        assert plugin.ofq_plugin_stream_on_execution_context_setup(s1) == 0
+        raw1 = plugin.ofq_plugin_stream_raw(s1)
+        assert raw1 and raw1 != plugin.ofq_plugin_stream_raw(s2)
+        cus = plugin.ofq_plugin_stream_cu_count(s1)
+        assert cus == torch.cuda.get_device_properties(dev).multi_processor_count == 256
+        # InitLaunchConfigWithWaves (cuda_stream.h:116-124): min(waves * CUs * threads/CU / block,
+        # blocks needed)
+        tpc = torch.cuda.get_device_properties(dev).max_threads_per_multi_processor
+        assert plugin.ofq_plugin_stream_grid_with_waves(s1, 1 << 30, 256, 32) == 32 * cus * (tpc // 256)
+        assert plugin.ofq_plugin_stream_grid_with_waves(s1, 1000, 256, 32) == 4
+        out = torch.empty_like(direct)
+        vp, ll = ctypes.c_void_p, ctypes.c_longlong
+        run = plugin.ofq_plugin_run_fused_linear
+        run.argtypes = [vp] * 7 + [ctypes.c_int] * 2 + [ll] * 3 + [ctypes.c_int] * 2 + [ll] * 2
+        assert run(raw1, xt.data_ptr(), wt.data_ptr(), st.data_ptr(), None, None, out.data_ptr(),
+                   K_FLOAT16, K_INT8, m, n, k, 4, 1, 1, g) == 0
+        plugin.ofq_plugin_stream_record_event(s1, ev)
+        # the second stream waits for the event, then runs the same kernel into a second buffer
+        plugin.ofq_plugin_stream_wait_event(s2, ev)
+        out2 = torch.empty_like(direct)
+        assert run(plugin.ofq_plugin_stream_raw(s2), xt.data_ptr(), wt.data_ptr(), st.data_ptr(),
+                   None, None, out2.data_ptr(), K_FLOAT16, K_INT8, m, n, k, 4, 1, 1, g) == 0
+        assert plugin.ofq_plugin_event_sync(ev) == 0
+        assert plugin.ofq_plugin_event_query_done(ev) == 1
+        assert torch.equal(out, direct)   # the event has completed, so the first kernel has
+        buf = ctypes.create_string_buffer(256)
+        assert plugin.ofq_plugin_stream_sync(s2, buf, 256) == 0
+        assert torch.equal(out2, direct)
+        assert plugin.ofq_plugin_stream_get_async_error(s1, buf, 256) == 0
+    finally:
+        plugin.ofq_plugin_event_delete(ev)
+        plugin.ofq_plugin_stream_delete(s1)   # synchronises and destroys its stream
+        plugin.ofq_plugin_stream_delete(s2)
+
+
+@pytest.mark.gpu
+def test_errors_of_the_device_runtime_surface_through_get_async_error(plugin):
+    """CudaStream::GetAsyncError is the device runtime's last error, cleared by the query
+    (cuda_stream.cpp:240-247).  The error is made on the host (a device ordinal that does not
+    exist): nothing faulty reaches the GPU.  Two routes: the stream is asked directly; and a
+    kernel of the library runs in between -- its launch check reads the runtime's record, the
+    C ABI reports OFQ_ERR_LAUNCH, and the runtime's query after Compute
+    (stateful_opkernel.cpp:1007) still gets the error."""
+    import torch
+    import helpers as H
+    from oneflow_amd import _lib
+    _bind_stream_hooks(plugin)
+    L = ctypes.CDLL(_lib.lib()._name)
+    dev = torch.cuda.current_device()
+    view = plugin.ofq_plugin_stream_view(dev, torch.cuda.current_stream().cuda_stream)
+    buf = ctypes.create_string_buffer(256)
+    try:
+        assert plugin.ofq_plugin_stream_get_async_error(view, buf, 256) == 0
+        assert L.ofq_hip_set_device(9999) != 0
+        assert plugin.ofq_plugin_stream_get_async_error(view, buf, 256) == -1
+        assert b"invalid device" in buf.value.lower()
+        assert plugin.ofq_plugin_stream_get_async_error(view, buf, 256) == 0   # cleared by the query
+
+        rng = np.random.default_rng(22)
+        m, n, k, g = 1, 256, 512, 128
+        xt = H.to_torch(rng.standard_normal((m, k)).astype(np.float16))
+        wt = H.to_torch(H.pack_int4(rng.integers(-7, 8, size=(n, k)).astype(np.int8)))
+        st = H.to_torch(rng.uniform(1e-3, 1e-2, size=(n, k // g)).astype(np.float16))
+        out = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        vp, ll = ctypes.c_void_p, ctypes.c_longlong
+        run = plugin.ofq_plugin_run_fused_linear
+        run.argtypes = [vp] * 7 + [ctypes.c_int] * 2 + [ll] * 3 + [ctypes.c_int] * 2 + [ll] * 2
+        args = (torch.cuda.current_stream().cuda_stream, xt.data_ptr(), wt.data_ptr(), st.data_ptr(),
+                None, None, out.data_ptr(), K_FLOAT16, K_INT8, m, n, k, 4, 1, 1, g)
+        assert L.ofq_hip_set_device(9999) != 0
+        assert run(*args) == -2                       # Compute, then GetAsyncError: the error
+        assert plugin.ofq_plugin_last_async_error(buf, 256) > 0
+        assert b"invalid device" in buf.value.lower()
+        assert run(*args) == 0                        # nothing is left behind
+        torch.cuda.synchronize()
+        assert L.ofq_hip_get_async_error() == 0
+    finally:
+        plugin.ofq_plugin_stream_delete(view)
