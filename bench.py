@@ -86,6 +86,7 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     L = _lib.lib()
+    P = load_probes()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     torch.manual_seed(1234)
@@ -321,7 +322,7 @@ def main():
         del tiled
         # per shape: the GEMV alone over all layers for 1, 4 and 8 rows of x (and 32 and 64, the
         # batch sizes of a serving loop, which run the multi-tile streaming kernel), and beside it a
-        # kernel that only reads the codes of the same weight tensors (ofq_probe_read; 97% of the
+        # kernel that only reads the codes of the same weight tensors (ofq_bench_probe_read; 97% of the
         # bytes the GEMV reads, in one launch per tensor) in the same graph-replay harness: what
         # reading those bytes once takes on this box
         sink = torch.zeros(1, dtype=torch.int32, device=dev)
@@ -329,9 +330,9 @@ def main():
         def read_only(mats):
             stream = torch.cuda.current_stream().cuda_stream
             for mat in mats:
-                st = L.ofq_probe_read(stream, mat[3].data_ptr(), mat[3].numel(), sink.data_ptr())
+                st = P.ofq_bench_probe_read(stream, mat[3].data_ptr(), mat[3].numel(), sink.data_ptr())
                 if st != 0:
-                    raise RuntimeError(f"ofq_probe_read status {st}")
+                    raise RuntimeError(f"ofq_bench_probe_read status {st}")
         for m in sorted({M, 1, 4, 8, 32, 64}):
             by_shape = {}
             for name, n, k, cnt in LLAMA7B_LAYER:
@@ -347,6 +348,39 @@ def main():
                     ev_r, _ = time_region(run_r, 10, 2)
                     by_shape[f"{n}x{k}"]["read_floor_us"] = round(ev_r * 1e3 / (10 * len(mats_s)), 2)
             other[f"decode_w4a16_m{m}_by_shape"] = by_shape
+        # the headline step replayed for at least a second (the timed region of the headline is
+        # `--steps` replays, some 20 ms): what the path sustains
+        n_sus = max(args.steps, int(1.05e3 / ms_per_step) + 1)
+        ev_sus, wall_sus = time_region(run_all, n_sus, 1)
+        gb_sus = bytes_step / (wall_sus / n_sus * 1e-3) / 1e9
+        other[f"decode_w4a16_m{M}_sustained"] = {
+            "replays": n_sus, "seconds": round(wall_sus * 1e-3, 3),
+            "ms_per_step": round(wall_sus / n_sus, 4), "gbps": round(gb_sus, 1),
+            "roofline": {"bound": "hbm", "achieved": round(gb_sus, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(gb_sus / HBM_PEAK_GBPS, 4)}}
+        # the ceilings the lines above are read against, in the same graph-replay harness: the
+        # fixed cost of a launch (a kernel that does nothing) and a plain copy kernel
+        stream_now = lambda: torch.cuda.current_stream().cuda_stream
+        run_e = make_runner(lambda: [P.ofq_bench_empty_launch(stream_now(), sink.data_ptr())
+                                     for _ in range(224)])
+        ev_e, _ = time_region(run_e, 10, 2)
+        ceilings = {"empty_kernel_us_per_launch": round(ev_e * 1e3 / (10 * 224), 3), "copy_kernel": {}}
+        for mb in (16, 32, 128):
+            nbytes = mb << 20
+            srcs = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(max(2, 1024 // mb))]
+            dsts = [torch.empty_like(t) for t in srcs]
+
+            def copies():
+                for a, b in zip(srcs, dsts):
+                    if P.ofq_bench_copy(stream_now(), b.data_ptr(), a.data_ptr(), nbytes) != 0:
+                        raise RuntimeError("ofq_bench_copy failed")
+            run_c = make_runner(copies)
+            ev_c, _ = time_region(run_c, 10, 2)
+            us_c = ev_c * 1e3 / (10 * len(srcs))
+            ceilings["copy_kernel"][f"{mb}MiB"] = {"us": round(us_c, 2),
+                                                  "gbps_read_plus_write": round(2 * nbytes / (us_c * 1e-6) / 1e9, 1)}
+            del srcs, dsts
+        other["ceilings_of_this_box"] = ceilings
         del layers
         torch.cuda.empty_cache()
         result["secondary"] = {**other, **secondary(L, _lib, torch, dev, args)}
@@ -355,6 +389,20 @@ def main():
                                    "unit": "TFLOP/s", "pct_mfma_peak": round(100 * pf["roofline"]["frac"], 2),
                                    "us": pf["us"]}
     print(json.dumps(result))
+
+
+def load_probes():
+    """The measurement probes (a kernel that only reads, an empty kernel, a plain copy): a
+    library of their own next to the product library, outside the ABI of include/ofq.h."""
+    path = os.path.join(ROOT, "oneflow_amd", "csrc", "libofq_bench_probes.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with __graft_entry__.build()")
+    P = ctypes.CDLL(path)
+    vp, sz = ctypes.c_void_p, ctypes.c_size_t
+    P.ofq_bench_probe_read.argtypes, P.ofq_bench_probe_read.restype = [vp, vp, sz, vp], ctypes.c_int
+    P.ofq_bench_empty_launch.argtypes, P.ofq_bench_empty_launch.restype = [vp, vp], ctypes.c_int
+    P.ofq_bench_copy.argtypes, P.ofq_bench_copy.restype = [vp, vp, vp, sz], ctypes.c_int
+    return P
 
 
 def cpu_baseline(M):

@@ -364,15 +364,6 @@ int ofq_fused_linear_gq_tiled(void* stream, const void* x, const void* w_tiled,
                               int w_dtype, int t_dtype, int num_bits, int symmetric,
                               int group_dim, int64_t group_size, int64_t m, int64_t n, int64_t k);
 
-/*
- * Measurement aid, no counterpart in the reference: a kernel that reads `bytes` (rounded down to
- * 16) from buf once, one 16-byte request per lane, and computes nothing.  What it takes is the
- * time below which no kernel that reads those bytes once can finish on this device; a benchmark
- * reports it beside the decode kernels.  buf 16-byte aligned; sink: 4 writable bytes (left
- * untouched in practice).
- */
-int ofq_probe_read(void* stream, const void* buf, size_t bytes, void* sink);
-
 #ifdef __cplusplus
 }
 #endif

@@ -55,7 +55,6 @@ SIGNATURES = {
     "ofq_matmul_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64]),
     "ofq_matmul_quant_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "ofq_matmul_quant_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _vp, _sz]),
-    "ofq_probe_read": (_i, [_vp, _vp, _sz, _vp]),
     "ofq_groupwise_repack_bytes": (_sz, [_i, _i64, _i64]),
     "ofq_groupwise_repack": (_i, [_vp, _vp, _vp, _i, _i64, _i64]),
     "ofq_fused_linear_gq_tiled": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64,

@@ -928,7 +928,7 @@ extern "C" size_t ofq_fused_linear_gq_workspace_bytes(int w_dtype, int t_dtype, 
   a.m = m;
   a.n = n;
   a.k = k;
-  if (gemv_wq_supported(a) || gemv_mt_supported(a)) return 0;
+  if (gemv_wq_supported(a) || gemv_m1_any_supported(a) || gemv_mt_supported(a)) return 0;
   if (group_dim == 0) return gemm_gn_workspace_bytes(a);
   return gemm_wq_workspace_bytes(a);  // 0 for every path but the two-pass GEMM at large m
 }
@@ -979,7 +979,9 @@ extern "C" int ofq_fused_linear_gq(void* stream, const void* x, const void* w,
   a.n = n;
   a.k = k;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (gemv_wq_supported(a)) {
+  // (the row-per-wave kernel for one row of x covers rows and groups off the chunk grid of the
+  // MFMA kernels: k a multiple of 32 / 16 elements, groups from 32 / 16)
+  if (gemv_wq_supported(a) || gemv_m1_any_supported(a)) {
     const int rc = launch_gemv_wq(st, a);
     if (rc != OFQ_ERR_UNSUPPORTED) return rc;  // e.g. bf16 with an x too large to stage
   }

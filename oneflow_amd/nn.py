@@ -107,6 +107,11 @@ class QuantizedLinear(torch.nn.Module):
             (out_features, groups), dtype=dtype, device=device))
         self.register_buffer("bias", torch.zeros(out_features, dtype=dtype, device=device)
                              if bias else None)
+        # the optional tile-major copy of `weight` (make_decode_copy): a buffer, so that it moves
+        # with the module, but not part of state_dict; `_tiled_from` names the weight tensor and
+        # the version of its contents the copy was made from
+        self.register_buffer("weight_tiled", None, persistent=False)
+        self._tiled_from = None
 
     @classmethod
     def from_float(cls, linear, num_bits=4, symmetric=True, group_size=128,
@@ -131,11 +136,37 @@ class QuantizedLinear(torch.nn.Module):
         """Extension: keeps a tile-major copy of the 4-bit weight beside the row-major one
         (``_C.groupwise_repack``; not part of ``state_dict``).  ``forward`` then reads it for 2 to
         16 rows of fp16 ``x`` and the row-major weight for everything else."""
-        self.weight_tiled = _C.groupwise_repack(self.weight, self.num_bits)
+        self._set_decode_copy(_C.groupwise_repack(self.weight, self.num_bits))
         return self
 
+    def _set_decode_copy(self, tiled):
+        self.weight_tiled = tiled
+        self._tiled_from = (self.weight.data_ptr(), self.weight._version)
+
+    def _decode_copy(self):
+        """The tile-major copy if it still belongs to ``weight``; a copy made from a weight that
+        has since been reassigned or written to (``load_state_dict``, ``copy_``) is dropped, so
+        that every batch size reads the same weights."""
+        if self.weight_tiled is None:
+            return None
+        if self._tiled_from != (self.weight.data_ptr(), self.weight._version):
+            self.weight_tiled, self._tiled_from = None, None
+        return self.weight_tiled
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .cuda() move weight and its copy together: the copy stays valid if it was
+        valid = self._decode_copy() is not None
+        super()._apply(fn, *args, **kwargs)
+        if valid and self.weight_tiled is not None:
+            self._tiled_from = (self.weight.data_ptr(), self.weight._version)
+        return self
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        self.weight_tiled, self._tiled_from = None, None
+
     def forward(self, x):
-        tiled = getattr(self, "weight_tiled", None)
+        tiled = self._decode_copy()
         if tiled is not None and x.dtype == torch.float16 and self.group_size % 128 == 0:
             m = x.numel() // x.shape[-1]
             if 2 <= m <= 16:

@@ -137,3 +137,30 @@ def test_glu_grouped_and_skip_layer_norm_checks():
         sln(x, bias=torch.zeros((1, 64), dtype=torch.float16))
     with pytest.raises(CheckFailedError, match=r"quantization_bit should be in range \(1, 8\]."):
         sln(x, quantization_bit=9)
+
+
+def test_quantized_linear_drops_a_stale_decode_copy():
+    """The tile-major copy made by make_decode_copy belongs to one weight tensor and one version
+    of its contents: loading a state dict, writing to the weight in place or assigning a new weight
+    drops it (otherwise 2..16 rows of x would read the old weights and every other batch size the
+    new ones); moving the module keeps it."""
+    import torch
+    from oneflow_amd.nn import QuantizedLinear
+    mod = QuantizedLinear(256, 64, bias=True, num_bits=4, group_size=128, device="cpu")
+    assert mod._decode_copy() is None and "weight_tiled" not in mod.state_dict()
+    fake = torch.zeros(64 * 128, dtype=torch.int8)
+    mod._set_decode_copy(fake)
+    assert mod._decode_copy() is fake
+    assert "weight_tiled" not in mod.state_dict()
+    mod.to(torch.device("cpu"))          # a move: still the same weights
+    mod.float()                          # only floating-point buffers are converted
+    assert mod._decode_copy() is not None
+    sd = {k: v.clone() for k, v in mod.state_dict().items()}
+    mod.load_state_dict(sd)
+    assert mod._decode_copy() is None
+    mod._set_decode_copy(fake)
+    mod.weight.add_(1)                   # written in place
+    assert mod._decode_copy() is None
+    mod._set_decode_copy(fake)
+    mod.weight = torch.ones_like(mod.weight)   # reassigned
+    assert mod._decode_copy() is None

@@ -11,7 +11,7 @@ import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-def _call(static, x, gamma, beta, eps, bits):
+def _call(static, x, gamma, beta, eps, bits, sync=True):
     from oneflow_amd import _lib
     L = _lib.lib()
     rows, cols = x.shape
@@ -30,7 +30,8 @@ def _call(static, x, gamma, beta, eps, bits):
         st = L.ofq_fused_layer_norm_min_max_observer(
             stream, x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), y.data_ptr(), scale.data_ptr(),
             zp.data_ptr(), dt, rows, cols, eps, bits, ws.data_ptr(), nbytes)
-    torch.cuda.synchronize()
+    if sync:
+        torch.cuda.synchronize()
     return st, y, scale, zp
 
 
@@ -49,6 +50,45 @@ def test_static_scratch_entry_matches_workspace_entry(dtype):
         assert torch.equal(y_a.view(torch.uint8), y_b.view(torch.uint8))
         assert torch.equal(s_a.view(torch.int32), s_b.view(torch.int32)) and s_b.item() > 0
         assert z_b.item() == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cols", [512, 1024, 2048, 4096])
+def test_static_scratch_entry_when_a_wave_walks_several_rows(dtype, cols):
+    """More than 4096 rows of 512 * {1, 2, 4, 8} elements: 2048 waves walk the rows with the next
+    row requested ahead and leave one partial maximum each; then a small call whose values are
+    smaller (its scale must not see the 2048 partials the large call left)."""
+    gen = torch.Generator(device="cpu").manual_seed(cols)
+    for rows, amp in ((4097 + cols // 8, 2.0), (40, 0.125)):
+        x = (torch.randn(rows, cols, generator=gen) * amp).to(dtype).cuda()
+        gamma = (1 + 0.1 * torch.randn(cols, generator=gen)).to(dtype).cuda()
+        beta = (0.1 * torch.randn(cols, generator=gen)).to(dtype).cuda()
+        st_a, y_a, s_a, z_a = _call(False, x, gamma, beta, 1e-5, 8)
+        st_b, y_b, s_b, z_b = _call(True, x, gamma, beta, 1e-5, 8)
+        assert st_a == 0 and st_b == 0
+        assert torch.equal(y_a.view(torch.uint8), y_b.view(torch.uint8))
+        assert torch.equal(s_a.view(torch.int32), s_b.view(torch.int32)) and s_b.item() > 0
+
+
+def test_static_scratch_entry_back_to_back_on_one_stream_without_a_host_wait():
+    """Two calls queued on one stream with nothing between them (the documented use): the second
+    call's kernels run behind the first call's finalize, so each sees its own partials.  Large
+    amplitudes first, then a smaller input with small ones; both against the workspace entry."""
+    gen = torch.Generator(device="cpu").manual_seed(99)
+    cases = []
+    for rows, cols, amp in ((3000, 2048, 4.0), (64, 2048, 0.1), (6000, 512, 2.0), (7, 8200, 0.5)):
+        x = (torch.randn(rows, cols, generator=gen) * amp).to(torch.float16).cuda()
+        gamma = (1 + 0.1 * torch.randn(cols, generator=gen)).to(torch.float16).cuda()
+        beta = (0.1 * torch.randn(cols, generator=gen)).to(torch.float16).cuda()
+        cases.append((x, gamma, beta))
+    want = [_call(False, x, g, b, 1e-5, 8) for x, g, b in cases]
+    torch.cuda.synchronize()
+    got = [_call(True, x, g, b, 1e-5, 8, sync=False) for x, g, b in cases]   # queued, not waited for
+    torch.cuda.synchronize()
+    for (st_a, y_a, s_a, z_a), (st_b, y_b, s_b, z_b) in zip(want, got):
+        assert st_a == 0 and st_b == 0
+        assert torch.equal(y_a.view(torch.uint8), y_b.view(torch.uint8))
+        assert torch.equal(s_a.view(torch.int32), s_b.view(torch.int32)) and s_b.item() > 0
 
 
 def test_static_scratch_entry_rejects_more_rows_than_its_capacity():
