@@ -14,7 +14,7 @@ inline int log2_exact(int64_t v) {
   return s;
 }
 
-template<int NW, int H, int XU>
+template<int NW, int H, int XU, int D = H>
 int launch_m1_inst(hipStream_t st, const LinearArgs& a) {
   M1Shape sh;
   sh.N = (int)a.n;
@@ -24,7 +24,7 @@ int launch_m1_inst(hipStream_t st, const LinearArgs& a) {
   sh.G = (int)(a.k / a.group_size);
   sh.gn = 1;
   const int grid = (int)((a.n + NW - 1) / NW);
-  gemv_w4_m1<NW, 1, H, XU><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
+  gemv_w4_m1<NW, 1, H, XU, D><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
       static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
       static_cast<const f16*>(a.scale), static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
       sh);
@@ -143,16 +143,29 @@ bool gemv_m1_supported(const LinearArgs& a) {
          && a.n <= (1 << 24);
 }
 
-// Blocks of 16 waves when a row is at most 2 KB of codes (k <= 4096), of 8 waves beyond: with
-// longer rows two small blocks per CU, each with its own barrier, run ahead of one large one
-// (4096 x 11008: 6.3 against 6.7 us), with short rows the second staging of x costs more than
-// that gains (4096 x 4096: 3.55 against 3.8 us).
+// Blocks of 16 waves when a row is at most 2 KB of codes (k <= 4096): with short rows a second
+// staging of x costs more than two small blocks gain (4096 x 4096: 3.55 against 3.8 us).  Longer
+// rows: 16 waves with 3 KB of the row requested ahead when the blocks fill the chip (n >= 3072),
+// otherwise blocks of 8 waves with the whole row requested up front (2048 x 11008: 4.5 against
+// 4.85 us; with everything requested up front two small blocks per CU, each with its own
+// barrier, run ahead of one large one, 4096 x 11008: 6.3 against 6.7 us).
 // One row per wave while one resident round of blocks covers n (n <= 4096); beyond that, for rows
 // of at most 2 KB of codes, the streaming kernel (11008 x 4096: 6.2 against 6.4 us; 128256 x
 // 4096: 41.5 against 50 us, 6.5 TB/s).
 int launch_gemv_m1(hipStream_t st, const LinearArgs& a) {
   if (a.n > 4096 && a.k <= 4096) {
     return a.k <= 2048 ? launch_m1_stream_inst<1>(st, a) : launch_m1_stream_inst<2>(st, a);
+  }
+  if (a.k > 4096 && a.n >= 3072) {
+    switch ((int)((a.k / 2 + 1023) / 1024)) {
+      case 3: return launch_m1_inst<16, 3, 1, 2>(st, a);
+      case 4: return launch_m1_inst<16, 4, 1, 3>(st, a);
+      case 5: return launch_m1_inst<16, 5, 1, 3>(st, a);
+      case 6: return launch_m1_inst<16, 6, 1, 3>(st, a);
+      case 7: return launch_m1_inst<16, 7, 1, 3>(st, a);
+      case 8: return launch_m1_inst<16, 8, 1, 3>(st, a);
+      default: return OFQ_ERR_UNSUPPORTED;
+    }
   }
 #define OFQ_M1_PLAIN(NW, H, XU) launch_m1_inst<NW, H, XU>(st, a)
   OFQ_M1_DISPATCH(a.k, OFQ_M1_PLAIN);
