@@ -449,6 +449,161 @@ gemv_w4_m1_stream(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   }
 }
 
+// Many rows per wave for the fused GLU and for several problems in one launch (rows of at most
+// 2 KB of codes): a block of the grid owns rows_per_block consecutive rows of ONE problem, stages
+// that problem's x once, and each wave walks its rows wave, wave + NW, .. as one sequence of KB
+// chunks with H chunks (one row) requested ahead of the arithmetic -- about 2 KB per wave and
+// 32 KB per CU in flight, which is what a CU sustains; more only queues (two rows ahead, the
+// plain streaming kernel's depth, was slower for these).  GLU: the sequence alternates between
+// the row of the first weight and the same row of the gate weight, so a trip of the loop (two
+// rows) is one (hidden, gate) pair and the wave that owns it forms y = hidden * act(gate).
+// One resident round of blocks replaces the one-and-a-half rounds of one-row-per-wave blocks
+// (2 x 11008 x 4096: 12.5 -> 9.7 us, three 4096 x 4096 problems: 7.8 -> 6.5 us).
+template<int NW, int H, int XU, bool GLU>
+__device__ __forceinline__ void
+m1_walk_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ w,
+             const f16* __restrict__ scale, const f16* __restrict__ bias, f16* __restrict__ out,
+             int N, const M1Shape& sh, const M1Glu& glu) {
+  static_assert(H == 1 || H == 2, "x operands stay in registers");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int NTH = NW * 64;
+  constexpr int RING = 2 * H;  // two rows
+  constexpr int D = H;         // one row ahead
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int K = sh.K;
+  const int row_bytes = K >> 1;
+  const int row0 = block * sh.rows_per_block;
+  int rows_blk = N - row0;
+  if (rows_blk > sh.rows_per_block) rows_blk = sh.rows_per_block;
+  const int nr = rows_blk > wave ? (rows_blk - wave + NW - 1) / NW : 0;  // rows (GLU: pairs)
+  const int nseq = GLU ? 2 * nr : nr;  // rows of the sequence
+  const int nchunks = nseq * H;
+
+  const int nunits = K >> 4;
+  const bool stage_wave = wave * 64 < nunits;  // wave-uniform
+  u32x4 xu[XU][2];
+  if (stage_wave) {
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+      int u = tid + i * NTH;
+      u = u < nunits ? u : nunits - 1;
+      const u32x4* src = reinterpret_cast<const u32x4*>(x) + (size_t)u * 2;
+      xu[i][0] = src[0];
+      xu[i][1] = src[1];
+    }
+  }
+  bool valid[H];
+  uint32_t voff[H];
+  int goff[H];
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+    valid[h] = h * 1024 + lane * 16 < row_bytes;
+    voff[h] = valid[h] ? (uint32_t)(h * 1024 + lane * 16) : 0u;
+    goff[h] = valid[h] ? (h * 2048 + lane * 32) >> sh.gshift : 0;
+  }
+  u32x4 wq[RING];
+  f16 sc[RING];
+  uint16_t braw[2];
+  // chunk c of the sequence: row c / H of the sequence (GLU: pair c / 2H, weight (c / H) & 1),
+  // KB h of that row; slot c % RING.  Every request is unconditional so that the wait counts
+  // stay exact: past the wave's last chunk all lanes read one and the same 16 bytes.
+  auto issue = [&](int c, int slot, int h, int which) {
+    const bool live = c < nchunks;  // wave-uniform
+    const int i = live ? (GLU ? c / (2 * H) : c / H) : 0;
+    const int row_l = live ? wave + i * NW : 0;
+    const uint8_t* wb = (GLU && which) ? glu.w2 : w;
+    const f16* sb = (GLU && which) ? glu.scale2 : scale;
+    const f16* bb = (GLU && which) ? glu.bias2 : bias;
+    const uint8_t* rowp = wb + (int64_t)(row0 + row_l) * row_bytes;
+    wq[slot] = __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4*>(rowp + (live ? voff[h] : 0u)));
+    sc[slot] = sb[(int64_t)(row0 + row_l) * sh.G + (live ? goff[h] : 0)];
+    if (h == 0) {
+      braw[(slot / H) & 1] =
+          bb != nullptr ? reinterpret_cast<const uint16_t*>(bb)[row0 + row_l] : (uint16_t)0;
+    }
+  };
+#pragma unroll
+  for (int c = 0; c < D; ++c) issue(c, c % RING, c % H, (c / H) & 1);
+
+  float* corr_l = reinterpret_cast<float*>(smem + (size_t)H * 4096);
+#pragma unroll
+  for (int i = 0; i < XU; ++i) {
+    if (wave * 64 + i * NTH >= nunits) break;  // wave-uniform
+    const int u = tid + i * NTH;
+    const bool ok = u < nunits;
+    u32x4 lo, hi;
+    permute_unit(xu[i][0], xu[i][1], lo, hi);
+    const int h = u >> 7, l = (u >> 1) & 63, p = u & 1;
+    if (ok) {
+      *reinterpret_cast<u32x4*>(smem + (size_t)(((h * 4 + 2 * p) * 64 + l) * 16)) = lo;
+      *reinterpret_cast<u32x4*>(smem + (size_t)(((h * 4 + 2 * p + 1) * 64 + l) * 16)) = hi;
+    }
+    float cpart = ok ? unit_corr(lo, hi) : 0.f;
+    cpart += __shfl_xor(cpart, 1, 64);
+    if (ok && p == 0) corr_l[h * 64 + l] = -cpart;
+  }
+  __syncthreads();
+  u32x4 xr[H][4];
+  float crr[H];
+#pragma unroll
+  for (int h = 0; h < H; ++h) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      xr[h][t] = *reinterpret_cast<const u32x4*>(smem + (size_t)(((h * 4 + t) * 64 + lane) * 16));
+    }
+    crr[h] = corr_l[h * 64 + lane];
+  }
+  for (int c0 = 0; c0 < nchunks; c0 += RING) {
+    float tot = 0.f;
+    float first = 0.f;  // the first row of the trip (GLU: hidden), bias added, rounded to T
+#pragma unroll
+    for (int j = 0; j < RING; ++j) {
+      const int h = j % H;
+      issue(c0 + j + D, (j + D) % RING, (j + D) % H, ((j + D) / H) & 1);
+      const float term = m1_dot32(wq[j], xr[h], crr[h]) * (float)sc[j];
+      tot += valid[h] ? term : 0.f;
+      if (h == H - 1) {
+        const float sum = wave_sum_m1(tot);
+        const f16 v = (f16)(sum + (float)bias_at_end(braw[(j / H) & 1]));
+        tot = 0.f;
+        if (GLU) {
+          const int row = row0 + wave + (c0 / RING) * NW;  // the pair of this trip
+          if (j / H == 0) {
+            first = (float)v;
+            if (lane == 0) out[row] = v;
+          } else if (lane == 0) {
+            glu.out2[row] = v;
+            glu.y[row] = (f16)first * (f16)glu_activation((float)v, glu.act);
+          }
+        } else {
+          const int i = (c0 + j) / H;
+          if (lane == 0 && i < nr) out[row0 + wave + i * NW] = v;
+        }
+      }
+    }
+  }
+}
+
+template<int NW, int H, int XU = 1>
+__global__ void __launch_bounds__(NW * 64)
+gemv_w4_m1_glu_walk(const f16* __restrict__ x, const uint8_t* __restrict__ w,
+                    const f16* __restrict__ scale, const f16* __restrict__ bias,
+                    f16* __restrict__ out, M1Glu glu, M1Shape sh) {
+  m1_walk_body<NW, H, XU, true>(blockIdx.x, x, w, scale, bias, out, sh.N, sh, glu);
+}
+
+template<int NW, int H, int XU = 1>
+__global__ void __launch_bounds__(NW * 64) gemv_w4_m1_grouped_walk(GemvGroup g, M1Shape sh) {
+  const GemvProblem pr = select_problem(g, (int)blockIdx.x);
+  m1_walk_body<NW, H, XU, false>((int)blockIdx.x - pr.first_block, static_cast<const f16*>(pr.x),
+                                 pr.w, static_cast<const f16*>(pr.scale),
+                                 static_cast<const f16*>(pr.bias), static_cast<f16*>(pr.out), pr.N,
+                                 sh, M1Glu());
+}
+
 template<int NW, int RPW, int H, int XU = 1, int D = H>
 __global__ void __launch_bounds__(NW * 64)
 gemv_w4_m1(const f16* __restrict__ x, const uint8_t* __restrict__ w,

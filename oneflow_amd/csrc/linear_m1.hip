@@ -115,6 +115,65 @@ int launch_m1_grouped_inst(hipStream_t st, const LinearArgs* pr, int count) {
   return ofq_check_launch();
 }
 
+// The fused GLU as a walk of (hidden, gate) row pairs: one block of 16 waves per CU.
+template<int H>
+int launch_m1_glu_walk_inst(hipStream_t st, const LinearArgs& a, const M1Glu& glu) {
+  constexpr int NW = 16;
+  const int rpb = (int)((a.n + 255) / 256);
+  const int grid = (int)((a.n + rpb - 1) / rpb);
+  M1Shape sh;
+  sh.N = (int)a.n;
+  sh.K = (int)a.k;
+  sh.rows_per_block = rpb;
+  sh.gshift = log2_exact(a.group_size);
+  sh.G = (int)(a.k / a.group_size);
+  sh.gn = 1;
+  gemv_w4_m1_glu_walk<NW, H, 1><<<grid, NW * 64, gemv_m1_lds_bytes(H), st>>>(
+      static_cast<const f16*>(a.x), static_cast<const uint8_t*>(a.w),
+      static_cast<const f16*>(a.scale), static_cast<const f16*>(a.bias), static_cast<f16*>(a.out),
+      glu, sh);
+  return ofq_check_launch();
+}
+
+// Several problems as a walk: blocks of 12 waves, two per CU, every block inside one problem;
+// rows per block = the smallest count that fits all problems into 512 blocks.
+template<int H>
+int launch_m1_grouped_walk_inst(hipStream_t st, const LinearArgs* pr, int count) {
+  constexpr int NW = 12;
+  int64_t total = 0;
+  for (int i = 0; i < count; ++i) total += pr[i].n;
+  int rpb = (int)((total + 511) / 512);
+  auto blocks_at = [&](int r) {
+    int64_t b = 0;
+    for (int i = 0; i < count; ++i) b += (pr[i].n + r - 1) / r;
+    return b;
+  };
+  while (blocks_at(rpb) > 512) ++rpb;
+  GemvGroup g{};
+  g.count = count;
+  int first = 0;
+  for (int i = 0; i < count; ++i) {
+    g.p[i].x = pr[i].x;
+    g.p[i].w = static_cast<const uint8_t*>(pr[i].w);
+    g.p[i].scale = pr[i].scale;
+    g.p[i].zero = nullptr;
+    g.p[i].bias = pr[i].bias;
+    g.p[i].out = pr[i].out;
+    g.p[i].N = (int)pr[i].n;
+    g.p[i].first_block = first;
+    first += (int)((pr[i].n + rpb - 1) / rpb);
+  }
+  M1Shape sh;
+  sh.N = 0;  // per problem
+  sh.K = (int)pr[0].k;
+  sh.rows_per_block = rpb;
+  sh.gshift = log2_exact(pr[0].group_size);
+  sh.G = (int)(pr[0].k / pr[0].group_size);
+  sh.gn = 1;
+  gemv_w4_m1_grouped_walk<NW, H, 1><<<first, NW * 64, gemv_m1_lds_bytes(H), st>>>(g, sh);
+  return ofq_check_launch();
+}
+
 // picks the instance for k: NW = 16 up to 2 KB of codes per row, 8 beyond
 #define OFQ_M1_DISPATCH(k, CALL)                      \
   do {                                                \
@@ -202,6 +261,11 @@ int launch_gemv_m1_glu(hipStream_t st, const LinearArgs& a, const LinearArgs& g,
   glu.out2 = static_cast<f16*>(g.out);
   glu.y = static_cast<f16*>(y);
   glu.act = act;
+  // beyond one resident round of one-pair-per-wave blocks (8192 rows of the two weights): the walk
+  if (a.k <= 4096 && a.n > 4096) {
+    return a.k <= 2048 ? launch_m1_glu_walk_inst<1>(st, a, glu)
+                       : launch_m1_glu_walk_inst<2>(st, a, glu);
+  }
 #define OFQ_M1_GLU(NW, H, XU) launch_m1_glu_inst<NW, H, XU>(st, a, glu)
   OFQ_M1_DISPATCH(a.k, OFQ_M1_GLU);
 #undef OFQ_M1_GLU
@@ -218,6 +282,15 @@ int launch_gemv_m1_grouped(hipStream_t st, const LinearArgs* pr, int count) {
     blocks += (pr[i].n + 7) / 8;
   }
   if (blocks > 0x7FFFFFFF) return OFQ_ERR_UNSUPPORTED;
+  {
+    int64_t total = 0;
+    for (int i = 0; i < count; ++i) total += pr[i].n;
+    // more rows than one resident round of one-row-per-wave blocks (2 x 256 x 16) holds
+    if (pr[0].k <= 4096 && total > 8192) {
+      return pr[0].k <= 2048 ? launch_m1_grouped_walk_inst<1>(st, pr, count)
+                             : launch_m1_grouped_walk_inst<2>(st, pr, count);
+    }
+  }
 #define OFQ_M1_GROUPED(NW, H, XU) launch_m1_grouped_inst<NW, H, XU>(st, pr, count)
   OFQ_M1_DISPATCH(pr[0].k, OFQ_M1_GROUPED);
 #undef OFQ_M1_GROUPED

@@ -25,7 +25,9 @@ def _problem(rng, m, n, k, num_bits, symmetric, qdt, g, t, bias=True):
 @pytest.mark.parametrize("t", ["f16", "bf16"])
 @pytest.mark.parametrize("num_bits", [4, 8])
 @pytest.mark.parametrize("m,k,ns", [(1, 1024, (512, 128, 128)), (8, 512, (300, 300)),
-                                    (16, 256, (40, 4099, 17)), (3, 128, (20000, 20000))])
+                                    (16, 256, (40, 4099, 17)), (3, 128, (20000, 20000)),
+                                    (1, 4096, (4096, 4096, 4096)), (1, 2048, (5000, 300, 6000)),
+                                    (1, 256, (9000, 37))])
 @pytest.mark.parametrize("g", [64, 128])
 def test_grouped_decode_one_launch(t, num_bits, m, k, ns, g):
     """Problems of equal (m, k): q/k/v-like row counts, ragged ones, and enough rows for two
@@ -140,13 +142,17 @@ def test_glu_all_activations(t, m, n, k, split, g):
                     assert (yf != yr).mean() < 0.02, act
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 1000, 4096), (2, 344, 2048), (3, 136, 5120), (4, 2000, 4096),
+@pytest.mark.parametrize("m,n,k", [(1, 1000, 4096), (1, 11008, 4096), (1, 4100, 2048), (1, 5003, 1024),
+                                   (1, 12000, 256), (1, 4097, 3840),
+                                   (2, 344, 2048), (3, 136, 5120), (4, 2000, 4096),
                                    (5, 37, 3072), (8, 1100, 4096), (8, 33, 11008), (4, 65, 11008),
                                    (8, 11008, 4096), (16, 2000, 4096), (6, 1200, 8192)])
 def test_glu_and_grouped_few_rows_of_x_symmetric_int4_fp16(m, n, k):
     """fp16, symmetric int4 in an int8 container, groups of 128, 1 .. 16 rows of x at real row
-    lengths (the decode case of both ops; one row of x takes the kernel in which a wave owns
-    whole weight rows; the last three shapes need two stagings of x in the GLU kernel, with one
+    lengths (the decode case of both ops; one row of x takes the kernels in which a wave owns
+    whole weight rows -- one row or row pair per wave up to 4096 rows, beyond that a wave walks
+    its rows, with rows of 1 and 2 KB of codes, row counts off the block sizes and a row that
+    ends inside a KB; the last three shapes need two stagings of x in the GLU kernel, with one
     and with two blocks per CU).  Split GLU + a grouped call with three row counts on a shared
     x."""
     import torch
