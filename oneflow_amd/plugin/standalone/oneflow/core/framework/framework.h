@@ -115,6 +115,45 @@ class Maybe<bool> {
     }                                                                          \
   } while (0)
 
+#define OFQ_OR_RETURN(cond)                                                              \
+  if (!(cond))                                                                           \
+  return ::oneflow::Error::RuntimeError() << "Check failed: " #cond " " << __FILE__ << ":" << __LINE__
+#define CHECK_OR_RETURN(cond) OFQ_OR_RETURN(cond)
+#define CHECK_EQ_OR_RETURN(a, b) OFQ_OR_RETURN((a) == (b))
+#define CHECK_GE_OR_RETURN(a, b) OFQ_OR_RETURN((a) >= (b))
+#define CHECK_GT_OR_RETURN(a, b) OFQ_OR_RETURN((a) > (b))
+#define CHECK_LE_OR_RETURN(a, b) OFQ_OR_RETURN((a) <= (b))
+#define CHECK_LT_OR_RETURN(a, b) OFQ_OR_RETURN((a) < (b))
+#define UNIMPLEMENTED_THEN_RETURN() \
+  return ::oneflow::Error::RuntimeError() << "UNIMPLEMENTED " << __FILE__ << ":" << __LINE__
+#define JUST(expr)                               \
+  do {                                           \
+    auto ofq_just_ = (expr);                     \
+    if (!ofq_just_.IsOk()) return ofq_just_;     \
+  } while (0)
+
+// oneflow/core/common/shape.h: what the op definitions use of it
+class Shape {
+ public:
+  Shape() = default;
+  Shape(std::initializer_list<int64_t> d) : dims_(d) {}
+  explicit Shape(std::vector<int64_t> d) : dims_(std::move(d)) {}
+  int64_t NumAxes() const { return (int64_t)dims_.size(); }
+  int64_t At(int64_t i) const { return dims_[i]; }
+  int64_t& operator[](int64_t i) { return dims_[i]; }
+  int64_t elem_cnt() const {
+    int64_t c = 1;
+    for (int64_t d : dims_) c *= d;
+    return c;
+  }
+  bool operator==(const Shape& o) const { return dims_ == o.dims_; }
+  bool operator!=(const Shape& o) const { return dims_ != o.dims_; }
+  const std::vector<int64_t>& dim_vec() const { return dims_; }
+
+ private:
+  std::vector<int64_t> dims_;
+};
+
 namespace ep {
 class Event {
  public:
@@ -208,20 +247,66 @@ template<> inline float KernelComputeContext::Attr<float>(const std::string& n) 
 template<> inline double KernelComputeContext::Attr<double>(const std::string& n) const { return attrs.at(n).f; }
 template<> inline std::string KernelComputeContext::Attr<std::string>(const std::string& n) const { return attrs.at(n).s; }
 
+// oneflow/core/framework/tensor_desc.h: shape and dtype of an argument
+class TensorDesc {
+ public:
+  TensorDesc() = default;
+  TensorDesc(Shape s, DataType d) : shape_(std::move(s)), dtype_(d) {}
+  const Shape& shape() const { return shape_; }
+  DataType data_type() const { return dtype_; }
+
+ private:
+  Shape shape_;
+  DataType dtype_ = kInvalidDataType;
+};
+
+// oneflow/core/framework/infer_util.h:35-90 (user_op::InferContext): inputs by (name, index),
+// outputs set by the op definition's inference functions.  `shapes` / `dtypes` (index 0 by name)
+// serve the kernels' tmp_buffer sizing; `in` / `out` (by name and index) the op definitions.
 class InferContext {
  public:
   virtual ~InferContext() = default;
   std::map<std::string, std::vector<int64_t>> shapes;
   std::map<std::string, DataType> dtypes;
-  ShapeView InputShape(const std::string& name, int32_t) const { return ShapeView(shapes.at(name)); }
-  DataType InputDType(const std::string& name, int32_t) const { return dtypes.at(name); }
+  ShapeView InputShape(const std::string& name, int32_t index) const {
+    auto it = in.find({name, index});
+    if (it != in.end()) return ShapeView(it->second.shape().dim_vec());
+    return ShapeView(shapes.at(name));
+  }
+  DataType InputDType(const std::string& name, int32_t index) const {
+    auto it = in.find({name, index});
+    return it != in.end() ? it->second.data_type() : dtypes.at(name);
+  }
   std::map<std::string, AttrValue> attrs;
   template<typename T>
   T Attr(const std::string& name) const;
+
+  std::map<std::pair<std::string, int32_t>, TensorDesc> in, out;
+  void AddInput(const std::string& name, int32_t index, std::vector<int64_t> shape, DataType dt) {
+    in[{name, index}] = TensorDesc(Shape(std::move(shape)), dt);
+  }
+  const TensorDesc& InputTensorDesc(const std::string& name, int32_t index) const {
+    return in.at({name, index});
+  }
+  bool has_input(const std::string& name, int32_t index) const { return in.count({name, index}) != 0; }
+  int32_t input_size(const std::string& name) const {
+    int32_t n = 0;
+    while (in.count({name, n}) != 0) ++n;
+    return n;
+  }
+  void SetOutputShape(const std::string& name, int32_t index, const Shape& shape) {
+    out[{name, index}] = TensorDesc(shape, out[{name, index}].data_type());
+  }
+  void SetOutputDType(const std::string& name, int32_t index, DataType dt) {
+    out[{name, index}] = TensorDesc(out[{name, index}].shape(), dt);
+  }
 };
 template<> inline bool InferContext::Attr<bool>(const std::string& n) const { return attrs.at(n).b; }
 template<> inline int32_t InferContext::Attr<int32_t>(const std::string& n) const { return (int32_t)attrs.at(n).i; }
 template<> inline int64_t InferContext::Attr<int64_t>(const std::string& n) const { return attrs.at(n).i; }
+template<> inline double InferContext::Attr<double>(const std::string& n) const { return attrs.at(n).f; }
+template<> inline std::string InferContext::Attr<std::string>(const std::string& n) const { return attrs.at(n).s; }
+template<> inline DataType InferContext::Attr<DataType>(const std::string& n) const { return (DataType)attrs.at(n).i; }
 
 class OpKernelState {};
 class OpKernelCache {};

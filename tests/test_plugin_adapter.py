@@ -306,3 +306,128 @@ def test_errors_of_the_device_runtime_surface_through_get_async_error(plugin):
         assert L.ofq_hip_get_async_error() == 0
     finally:
         plugin.ofq_plugin_stream_delete(view)
+
+
+class _Infer:
+    """One op-definition call described through the plugin's hooks."""
+
+    def __init__(self, plugin, op):
+        vp, ci, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
+        p = plugin
+        p.ofq_plugin_infer_new.restype = vp
+        p.ofq_plugin_infer_delete.argtypes = [vp]
+        p.ofq_plugin_infer_add_input.argtypes = [vp, ctypes.c_char_p, ci, ctypes.POINTER(ll), ci, ci]
+        p.ofq_plugin_infer_attr_int.argtypes = [vp, ctypes.c_char_p, ll]
+        p.ofq_plugin_infer_attr_bool.argtypes = [vp, ctypes.c_char_p, ci]
+        p.ofq_plugin_infer_attr_double.argtypes = [vp, ctypes.c_char_p, ctypes.c_double]
+        p.ofq_plugin_infer_attr_string.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
+        p.ofq_plugin_infer_run.argtypes = [vp, ctypes.c_char_p]
+        p.ofq_plugin_infer_output.argtypes = [vp, ctypes.c_char_p, ci, ctypes.POINTER(ll), ci, ctypes.POINTER(ci)]
+        self.p, self.op, self.c = p, op.encode(), p.ofq_plugin_infer_new()
+
+    def inp(self, name, shape, dtype, index=0):
+        arr = (ctypes.c_longlong * len(shape))(*shape)
+        self.p.ofq_plugin_infer_add_input(self.c, name.encode(), index, arr, len(shape), dtype)
+        return self
+
+    def attrs(self, **kw):
+        for k, v in kw.items():
+            if isinstance(v, bool):
+                self.p.ofq_plugin_infer_attr_bool(self.c, k.encode(), int(v))
+            elif isinstance(v, int):
+                self.p.ofq_plugin_infer_attr_int(self.c, k.encode(), v)
+            elif isinstance(v, float):
+                self.p.ofq_plugin_infer_attr_double(self.c, k.encode(), v)
+            else:
+                self.p.ofq_plugin_infer_attr_string(self.c, k.encode(), v.encode())
+        return self
+
+    def run(self):
+        rc = self.p.ofq_plugin_infer_run(self.c, self.op)
+        if rc != 0:
+            buf = ctypes.create_string_buffer(512)
+            self.p.ofq_plugin_infer_error(buf, 512)
+            return buf.value.decode()
+        return None
+
+    def out(self, name, index=0):
+        shape = (ctypes.c_longlong * 8)()
+        dt = ctypes.c_int()
+        rank = self.p.ofq_plugin_infer_output(self.c, name.encode(), index, shape, 8, ctypes.byref(dt))
+        return (None, None) if rank < 0 else (tuple(shape[:rank]), dt.value)
+
+    def __del__(self):
+        self.p.ofq_plugin_infer_delete(self.c)
+
+
+def test_op_definitions_of_the_added_ops(plugin):
+    """Shape and dtype inference of the four ops without a definition in the reference tree
+    (oneflow_amd/plugin/ofq_oneflow_ops.cpp), in the style of
+    fused_linear_with_groupwise_quantized_weight_op.cpp:27-94: outputs inferred, the same shape
+    rules as the functional layer, violations reported as errors and not as aborts."""
+    quant = dict(num_bits=4, symmetric=True, group_dim=1, group_size=128)
+    # LayerNorm + observer, with the skip_layer_norm inputs
+    c = (_Infer(plugin, "fused_layer_norm_min_max_observer").inp("x", (2, 7, 4096), K_FLOAT16)
+         .inp("gamma", (4096,), K_FLOAT16).inp("beta", (4096,), K_FLOAT16)
+         .inp("skip", (2, 7, 4096), K_FLOAT16).attrs(epsilon=1e-5, alpha=0.5, quantization_bit=8))
+    assert c.run() is None
+    assert c.out("y") == ((2, 7, 4096), K_FLOAT16)
+    assert c.out("scale") == ((1,), K_FLOAT) and c.out("zero_point") == ((1,), K_FLOAT)
+    bad = (_Infer(plugin, "fused_layer_norm_min_max_observer").inp("x", (4, 4096), K_FLOAT16)
+           .inp("gamma", (4095,), K_FLOAT16).attrs(epsilon=1e-5, alpha=0.5, quantization_bit=8))
+    assert "Check failed" in bad.run()
+    bad = (_Infer(plugin, "fused_layer_norm_min_max_observer").inp("x", (4, 4096), K_FLOAT16)
+           .attrs(epsilon=1e-5, alpha=0.5, quantization_bit=9))
+    assert "quantization_bit" in bad.run()
+    bad = (_Infer(plugin, "fused_layer_norm_min_max_observer").inp("x", (4, 4096), K_FLOAT16)
+           .inp("beta", (4096,), K_FLOAT).attrs(epsilon=1e-5, alpha=0.5, quantization_bit=8))
+    assert "Check failed" in bad.run()
+    # matmul_quant
+    c = (_Infer(plugin, "matmul_quant").inp("a", (3, 2048, 4096), K_INT8).inp("b", (11008, 4096), K_INT8)
+         .inp("a_scale", (1,), K_FLOAT).inp("b_scale", (11008,), K_FLOAT)
+         .inp("bias", (11008,), K_FLOAT16).attrs(out_dtype=K_FLOAT16))
+    assert c.run() is None and c.out("out") == ((3, 2048, 11008), K_FLOAT16)
+    bad = (_Infer(plugin, "matmul_quant").inp("a", (8, 4096), K_INT8).inp("b", (64, 4000), K_INT8)
+           .inp("a_scale", (1,), K_FLOAT).inp("b_scale", (64,), K_FLOAT).attrs(out_dtype=K_FLOAT16))
+    assert "Check failed" in bad.run()
+    bad = (_Infer(plugin, "matmul_quant").inp("a", (8, 4096), K_UINT8).inp("b", (64, 4096), K_INT8)
+           .inp("a_scale", (1,), K_FLOAT).inp("b_scale", (64,), K_FLOAT).attrs(out_dtype=K_FLOAT16))
+    assert "Check failed" in bad.run()
+    # GLU over two weights, and over one weight of 2n rows
+    c = (_Infer(plugin, "fused_glu_with_groupwise_quantized_weight").inp("x", (5, 4096), K_FLOAT16)
+         .inp("w", (11008, 2048), K_INT8).inp("w_scale", (11008, 32), K_FLOAT16)
+         .inp("v", (11008, 2048), K_INT8).inp("v_scale", (11008, 32), K_FLOAT16)
+         .attrs(activation="silu", **quant))
+    assert c.run() is None
+    assert c.out("y") == ((5, 11008), K_FLOAT16) and c.out("matmul_vx") == ((5, 11008), K_FLOAT16)
+    c = (_Infer(plugin, "fused_glu_with_groupwise_quantized_weight").inp("x", (5, 4096), K_FLOAT16)
+         .inp("w", (22016, 2048), K_INT8).inp("w_scale", (22016, 32), K_FLOAT16)
+         .inp("b", (22016,), K_FLOAT16).attrs(activation="fast_gelu", **quant))
+    assert c.run() is None
+    assert c.out("y") == ((5, 11008), K_FLOAT16) and c.out("matmul_wx") == ((5, 22016), K_FLOAT16)
+    assert c.out("matmul_vx") == (None, None)
+    bad = (_Infer(plugin, "fused_glu_with_groupwise_quantized_weight").inp("x", (5, 4096), K_FLOAT16)
+           .inp("w", (64, 2048), K_INT8).inp("w_scale", (64, 31), K_FLOAT16)
+           .attrs(activation="silu", **quant))
+    assert "Check failed" in bad.run()
+    bad = (_Infer(plugin, "fused_glu_with_groupwise_quantized_weight").inp("x", (5, 4096), K_FLOAT16)
+           .inp("w", (64, 2048), K_INT8).inp("w_scale", (64, 32), K_FLOAT16)
+           .attrs(activation="swish", **quant))
+    assert "Check failed" in bad.run()
+    # asymmetric codes need uint8 and a zero point
+    asym = dict(quant, symmetric=False)
+    bad = (_Infer(plugin, "fused_glu_with_groupwise_quantized_weight").inp("x", (5, 4096), K_FLOAT16)
+           .inp("w", (64, 2048), K_INT8).inp("w_scale", (64, 32), K_FLOAT16)
+           .inp("w_zero", (64, 32), K_FLOAT16).attrs(activation="silu", **asym))
+    assert "Check failed" in bad.run()
+    # grouped linear: q / k / v
+    c = _Infer(plugin, "grouped_linear_with_groupwise_quantized_weight").attrs(**quant)
+    for i, n in enumerate((4096, 1024, 1024)):
+        c.inp("xs", (1, 4096), K_FLOAT16, i).inp("ws", (n, 2048), K_INT8, i)
+        c.inp("w_scales", (n, 32), K_FLOAT16, i).inp("bs", (n,), K_FLOAT16, i)
+    assert c.run() is None
+    assert [c.out("ys", i) for i in range(3)] == [((1, n), K_FLOAT16) for n in (4096, 1024, 1024)]
+    bad = _Infer(plugin, "grouped_linear_with_groupwise_quantized_weight").attrs(**quant)
+    bad.inp("xs", (1, 4096), K_FLOAT16, 0).inp("ws", (64, 2048), K_INT8, 0).inp("w_scales", (64, 32), K_FLOAT16, 0)
+    bad.inp("xs", (1, 4096), K_FLOAT16, 1).inp("ws", (64, 2048), K_INT8, 1)
+    assert "Check failed" in bad.run()
