@@ -184,3 +184,36 @@ def test_fake_quantization_straight_through_gradient():
     with torch.no_grad():
         y2 = flow._C.fake_quantization(x, s, z, "google", 8, "symmetric")
     assert not y2.requires_grad and torch.equal(y2, y.detach())
+
+
+@pytest.mark.parametrize("per_layer", [True, False])
+@pytest.mark.parametrize("scheme", ["symmetric", "affine"])
+def test_qat_conv_is_the_convolution_of_the_fake_quantized_operands(per_layer, scheme):
+    """python/oneflow/nn/qat/conv.py: QatConv2d = conv(fake_quant(x; moving-average observer),
+    fake_quant(w; min/max observer)).  The fake-quantized operands are checked bit for bit against
+    the oracle's observers and fake quantization, the output against the host framework's
+    convolution on those operands, and the gradient passes straight through to x and w."""
+    import torch
+    import oneflow_amd as flow
+    rng = np.random.default_rng(3)
+    conv = flow.qat.QatConv2d(4, 6, 3, padding=1, quantization_scheme=scheme,
+                              weight_quant_per_layer=per_layer).cuda()
+    x = torch.from_numpy(rng.standard_normal((2, 4, 8, 8)).astype(np.float32)).cuda().requires_grad_()
+    conv.train()
+    y = conv(x)
+    xn, wn = x.detach().cpu().numpy(), conv.weight.detach().cpu().numpy()
+    # input: first training step of the moving-average observer = the tensor's own extremes
+    s_in, z_in = O.moving_average_min_max_observer(
+        xn, 0, np.zeros(1, np.float32), np.zeros(1, np.float32), True, 1, "google", 8, scheme, 0.95)
+    x_fq = O.fake_quantization(xn, s_in, z_in, "google", 8, scheme, zp_mode="cuda")
+    s_w, z_w = O.min_max_observer(wn, "google", 8, scheme, per_layer)
+    w_fq = O.fake_quantization(wn, s_w, z_w, "google", 8, scheme, zp_mode="cuda")
+    want = torch.nn.functional.conv2d(torch.from_numpy(x_fq).cuda(), torch.from_numpy(w_fq).cuda(),
+                                      conv.bias.detach(), padding=1)
+    assert torch.allclose(y.detach(), want, rtol=1e-5, atol=1e-5)
+    y.sum().backward()
+    assert x.grad is not None and conv.weight.grad is not None
+    # straight-through: d y / d x = conv_transpose of ones with the fake-quantized weight
+    xx = x.detach().clone().requires_grad_()
+    torch.nn.functional.conv2d(xx, torch.from_numpy(w_fq).cuda(), None, padding=1).sum().backward()
+    assert torch.allclose(x.grad, xx.grad, rtol=1e-5, atol=1e-5)
