@@ -611,6 +611,17 @@ def secondary(L, _lib, torch, dev, args):
         "roofline": {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gb / HBM_PEAK_GBPS, 4)}}
 
+    # the same call with the row statistics accumulated in fp64 and rounded once
+    def ln_exact():
+        i = it[0] % reps
+        it[0] += 1
+        chk(L.ofq_fused_layer_norm_min_max_observer_stats(
+            cs(), xs[i].data_ptr(), None, None, 0.0, 0, gamma.data_ptr(), beta.data_ptr(),
+            ys[i].data_ptr(), s.data_ptr(), z.data_ptr(), _lib.F16, m, k, 1e-5, 8,
+            _lib.LN_STATS_FP64, ws.data_ptr(), m * 4), "ln_observer_stats")
+    us_exact = timeit(ln_exact, iters=40)
+    out["layer_norm_observer_f16_2048x4096"]["us_with_fp64_row_statistics"] = round(us_exact, 2)
+
     def sln():
         i = it[0] % reps
         it[0] += 1
