@@ -248,6 +248,25 @@ int ofq_fused_layer_norm_min_max_observer_stats(
     void* workspace, size_t workspace_bytes);
 
 /*
+ * fused_layer_norm_quantization: fused_layer_norm_min_max_observer followed by `quantization`
+ *   (symmetric, per layer, google formula, the same quantization_bit) of its output, without the
+ *   normalised tensor reaching memory: codes[rows, cols] (int8), scale[1], zero_point[1] = 0.
+ *   No reference interface: it is the dynamic activation quantisation in front of matmul_quant,
+ *   i.e. the composition of the op above with
+ *   oneflow/user/kernels/quantization_kernel.cu:107-156; the codes and the scale carry the same
+ *   bits as that composition.  statistics as in ofq_fused_layer_norm_min_max_observer_stats.
+ *   Served: fp16 rows of 512, 1024, 2048 or 4096 elements with gamma and beta, 16-byte aligned;
+ *   any other case returns OFQ_ERR_UNSUPPORTED (nothing is launched) and the caller runs the two
+ *   ops.  workspace: ofq_fused_layer_norm_quantization_workspace_bytes(), 16-byte aligned.
+ */
+size_t ofq_fused_layer_norm_quantization_workspace_bytes(int t_dtype, int64_t rows, int64_t cols);
+int ofq_fused_layer_norm_quantization(void* stream, const void* x, const void* gamma,
+                                      const void* beta, void* codes, float* scale,
+                                      float* zero_point, int t_dtype, int64_t rows, int64_t cols,
+                                      double epsilon, int quantization_bit, int statistics,
+                                      void* workspace, size_t workspace_bytes);
+
+/*
  * groupwise_quantize: the producer of the weight format of the two ops above.
  * The reference defines that format only through the helpers of its own test,
  *   python/oneflow/test/modules/test_groupwise_quantization.py:26-35 (int4 packing) and :46-81

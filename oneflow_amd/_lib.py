@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libofq_hip.so")
 
 # mirror of the enums in include/ofq.h
 OK = 0
+ERR_UNSUPPORTED = 5
 F32, F16, BF16, F64, I8, U8 = 0, 1, 2, 3, 4, 5
 SCHEME = {"symmetric": 0, "affine": 1}
 FORMULA = {"google": 0, "cambricon": 1}
@@ -48,6 +49,9 @@ SIGNATURES = {
     "ofq_fused_layer_norm_min_max_observer_stats": (_i, [_vp, _vp, _vp, _vp, ctypes.c_double, _i,
                                                          _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64,
                                                          ctypes.c_double, _i, _i, _vp, _sz]),
+    "ofq_fused_layer_norm_quantization": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64,
+                                               ctypes.c_double, _i, _i, _vp, _sz]),
+    "ofq_fused_layer_norm_quantization_workspace_bytes": (_sz, [_i, _i64, _i64]),
     "ofq_grouped_linear_gq": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _i64]),
     "ofq_fused_glu_gq": (_i, [_vp] * 13 + [_i, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64]),

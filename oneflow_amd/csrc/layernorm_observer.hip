@@ -17,6 +17,7 @@
 // use one block per row.  The absmax of the stored values goes to the workspace (one float per
 // wave or per row) and a second one-wave launch folds them and divides.
 #include <atomic>
+#include <type_traits>
 #include "ofq_device.h"
 
 // Scratch of the entry point that allocates nothing (ofq_fused_layer_norm_min_max_observer_static):
@@ -724,6 +725,302 @@ ln_observer_finalize(const float* __restrict__ part, int64_t n, int bits,
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// LayerNorm -> observer -> int8 codes without the normalised tensor ever reaching memory
+// (ofq_fused_layer_norm_quantization).  fp16 rows of exactly 512 * NP elements with gamma and beta.
+// Two kernels:
+//   first : the row kernel above without its store: a wave normalises its rows in registers,
+//           keeps (mean, inv) of every row and the largest |y| it has seen;
+//   second: every block folds the partial maxima into the scale (the arithmetic of
+//           ln_observer_finalize, so every block gets the same bits), then a wave reads its rows
+//           again -- from L2 where the first kernel left them: the same wave of the same block
+//           took them there --, forms y with the stored statistics exactly as the first kernel
+//           did, and quantises it the way quantize_half_to_bytes_kernel does.
+// The codes are those of fused_layer_norm_min_max_observer followed by quantization (symmetric,
+// per layer) of its y, bit for bit; traffic is x once from HBM, x once more from L2 and the codes
+// (25 MB at 2048 x 4096 where the two ops move 58.7 MB).
+// ---------------------------------------------------------------------------------------------
+constexpr int kLnqBlock = 512;  // 8 waves: one copy of gamma and beta in LDS serves 8 rows
+
+// gamma and beta of a block: fetched once (wave w fetches pack w of each), parked in LDS, read
+// from there pack by pack.  Every wave of the block holding its own copy in registers cost 16 of
+// a wave's 24 requests and as much traffic between L2 and the CU as x itself.
+template<int NP>
+struct LnRowF16 {
+  u32x4 graw, braw;
+  __device__ __forceinline__ void request(const uint16_t* gamma, const uint16_t* beta, int wave,
+                                          int lane) {
+    if (wave < NP) {  // the same for every lane of a wave
+      graw = *reinterpret_cast<const u32x4*>(gamma + lane * 8 + wave * 512);
+      braw = *reinterpret_cast<const u32x4*>(beta + lane * 8 + wave * 512);
+    }
+  }
+  // [gamma NP x 64 pieces][beta NP x 64 pieces]; a barrier must follow before out() is used
+  __device__ __forceinline__ void park(u32x4* lds, int wave, int lane) const {
+    if (wave < NP) {
+      lds[wave * 64 + lane] = graw;
+      lds[(NP + wave) * 64 + lane] = braw;
+    }
+  }
+  // y of pack i from the deviations d[8] = x - mean: T(d * inv), * gamma, + beta, each rounded to T
+  __device__ __forceinline__ f16x8 out(const float* d, float inv, int i, const u32x4* lds,
+                                       int lane) const {
+    f16x8 t;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) t[e] = (f16)normalised<f16>(d[e], inv);
+    t = t * __builtin_bit_cast(f16x8, lds[i * 64 + lane]);
+    t = t + __builtin_bit_cast(f16x8, lds[(NP + i) * 64 + lane]);
+    return t;
+  }
+};
+
+template<int NP, bool EXACT>
+__global__ void __launch_bounds__(kLnqBlock)
+ln_quant_first(const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma,
+               const uint16_t* __restrict__ beta, float* __restrict__ block_absmax,
+               float* __restrict__ stats, int64_t rows, double eps64) {
+  constexpr int kCols = NP * 512;
+  constexpr int kWaves = kLnqBlock / kWave;
+  __shared__ float wmax[kWaves];
+  __shared__ u32x4 params[2 * NP * 64];
+  const float eps = (float)eps64;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t gw = (int64_t)blockIdx.x * kWaves + wave;
+  const int64_t nwaves = (int64_t)gridDim.x * kWaves;
+  LnRowF16<NP> prm;
+  prm.request(gamma, beta, wave, lane);
+  u32x4 cur[NP];
+  {
+    // (a wave past the last row re-reads row 0 and skips the loop: it only joins the barriers)
+    const uint16_t* xr = x + (gw < rows ? gw : 0) * kCols + lane * 8;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) cur[i] = *reinterpret_cast<const u32x4*>(xr + i * 512);
+  }
+  prm.park(params, wave, lane);
+  __syncthreads();
+  f16x8 amax8 = {(f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f, (f16)0.0f};
+  for (int64_t row = gw; row < rows; row += nwaves) {
+    if (row != gw) {
+      const uint16_t* xr = x + row * kCols + lane * 8;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) cur[i] = *reinterpret_cast<const u32x4*>(xr + i * 512);
+    }
+    float f[NP][8];
+    float sum = 0.0f;
+    double sum64 = 0.0;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      RawPack<f16> rp;
+      rp.q[0] = cur[i];
+      widen<f16>(rp, f[i]);
+      if constexpr (EXACT) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum64 += (double)f[i][e];
+      } else {
+        uint32_t ones_bits = 0x3c003c00u;  // (1, 1) held in a register, see ln_observer_wave_full
+        asm volatile("" : "+v"(ones_bits));
+        const f16x2 ones = __builtin_bit_cast(f16x2, ones_bits);
+        const f16x8 h = __builtin_bit_cast(f16x8, cur[i]);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 0, 1), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 2, 3), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 4, 5), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 6, 7), ones, sum, false);
+      }
+    }
+    float mean, inv;
+    if constexpr (EXACT) {
+      sum64 = wave_reduce(sum64, OpSum());
+      const double mean64 = sum64 / (double)kCols;
+      mean = (float)mean64;
+      double q = 0.0;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const double d = (double)f[i][e] - mean64;
+          q = __builtin_fma(d, d, q);
+          f[i][e] = f[i][e] - mean;
+        }
+      }
+      q = wave_reduce(q, OpSum());
+      inv = exact_inv(q, (double)kCols, eps64);
+    } else {
+      sum = wave_reduce(sum, OpSum());
+      mean = sum / (float)kCols;
+      float m2 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          f[i][e] = f[i][e] - mean;
+          m2 = __builtin_fmaf(f[i][e], f[i][e], m2);
+        }
+      }
+      m2 = wave_reduce(m2, OpSum());
+      const float var = fmaxf(m2 / (float)kCols, 0.0f);
+      inv = 1.0f / __builtin_sqrtf(var + eps);
+    }
+    if (lane == 0) {
+      stats[2 * row] = mean;
+      stats[2 * row + 1] = inv;
+    }
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const u32x4 tb = __builtin_bit_cast(u32x4, prm.out(f[i], inv, i, params, lane));
+      const u32x4 ab = {tb[0] & 0x7FFF7FFFu, tb[1] & 0x7FFF7FFFu, tb[2] & 0x7FFF7FFFu,
+                        tb[3] & 0x7FFF7FFFu};
+      amax8 = __builtin_elementwise_max(amax8, __builtin_bit_cast(f16x8, ab));
+    }
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) amax = fmaxf(amax, (float)amax8[e]);
+  amax = wave_reduce(amax, OpMax());
+  // one partial maximum per block, so that the second kernel folds them with one request
+  if (lane == 0) wmax[wave] = amax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    amax = wmax[0];
+#pragma unroll
+    for (int wv = 1; wv < kWaves; ++wv) amax = fmaxf(amax, wmax[wv]);
+    block_absmax[blockIdx.x] = amax;
+  }
+}
+
+// SPLIT: a row is taken by SPLIT waves of SPLIT different blocks, NP / SPLIT packs each (nothing
+// in this kernel crosses the lanes of a row), so that few rows still make enough waves to
+// overlap one wave's arithmetic with another's requests.  Block b works on the rows of block
+// p = (b / (8 * SPLIT)) * 8 + b % 8 of the first kernel, part (b / 8) % SPLIT: b and p agree
+// modulo 8, the number of XCDs the blocks are dealt over, so a row is read again through the L2
+// that holds it.  The grid is ceil(first_grid / 8) * 8 * SPLIT blocks.
+template<int NP, int SPLIT>
+__global__ void __launch_bounds__(kLnqBlock)
+ln_quant_second(const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma,
+                const uint16_t* __restrict__ beta, const float* __restrict__ part, int64_t nparts,
+                const float* __restrict__ stats, int8_t* __restrict__ codes,
+                float* __restrict__ scale, float* __restrict__ zero_point, int64_t rows, int bits,
+                int first_grid) {
+  static_assert(NP % SPLIT == 0, "whole packs per part");
+  constexpr int kCols = NP * 512;
+  constexpr int NPW = NP / SPLIT;  // packs of a row this wave takes
+  constexpr int kWaves = kLnqBlock / kWave;
+  __shared__ float wmax[kWaves];
+  __shared__ u32x4 params[2 * NPW * 64];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t fb = ((int64_t)blockIdx.x / (8 * SPLIT)) * 8 + blockIdx.x % 8;
+  const int part_of_row = (int)((blockIdx.x / 8) % SPLIT);
+  const int pack0 = part_of_row * NPW;
+  const int64_t gw = fb * kWaves + wave;
+  const int64_t nwaves = (int64_t)first_grid * kWaves;
+  const bool active = gw < rows;
+  // Requests in the order of their use: the partial maxima (one 16-byte piece per thread:
+  // nparts <= 512 <= 4 * kLnqBlock), the statistics of the wave's first row, the wave's share of
+  // the parameters, then the row, so that the maxima can be folded and the parameters parked
+  // while the row is still on its way.
+  const int64_t n4 = (nparts + 3) / 4;
+  const int64_t pidx = (int64_t)threadIdx.x < n4 ? threadIdx.x : 0;
+  f32x4 pq = reinterpret_cast<const f32x4*>(part)[pidx];
+  const float* st0 = stats + 2 * (active ? gw : 0);
+  float mean0 = st0[0], inv0 = st0[1];
+  LnRowF16<NPW> prm;
+  prm.request(gamma + pack0 * 512, beta + pack0 * 512, wave, lane);
+  u32x4 cur[NPW];
+  {
+    const uint16_t* xr = x + (active ? gw : 0) * kCols + pack0 * 512 + lane * 8;
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) cur[i] = *reinterpret_cast<const u32x4*>(xr + i * 512);
+  }
+  prm.park(params, wave, lane);
+  // scale = max of the partial maxima / (2^(bits-1) - 1), the same operations in every block
+  // (the last piece may reach up to three floats past the partials: masked)
+  float amax = 0.0f;
+  {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) amax = fmaxf(amax, pidx * 4 + e < nparts ? pq[e] : 0.0f);
+    amax = wave_reduce(amax, OpMax());
+    if (lane == 0) wmax[wave] = amax;
+    __syncthreads();  // (also orders the parked parameters before their use)
+    amax = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < kWaves; ++wv) amax = fmaxf(amax, wmax[wv]);
+  }
+  const float upper = (float)(1 << (bits - 1)) - 1.0f;
+  const float s = amax / upper;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *scale = s;
+    *zero_point = 0.0f;
+  }
+  if (!active) return;
+  // quantisation of quantize_half_to_bytes_kernel, symmetric scheme
+  const float mag = __builtin_fabsf(s);
+  const bool recip_ok = mag >= 0x1p-60f && mag <= 0x1p60f;
+  const float recip = recip_ok ? 1.0f / s : 0.f;
+  const int hi = (int)upper, lo = -hi - 1;
+  // (the branch on the scale's range is taken once per wave: inside the loop both quotients
+  // would be computed for every element and one of them selected)
+  auto walk = [&](auto fast) {
+    for (int64_t row = gw; row < rows; row += nwaves) {
+      if (row != gw) {
+        const uint16_t* xr = x + row * kCols + pack0 * 512 + lane * 8;
+#pragma unroll
+        for (int i = 0; i < NPW; ++i) cur[i] = *reinterpret_cast<const u32x4*>(xr + i * 512);
+      }
+      float mean = mean0, inv = inv0;
+      if (row != gw) {
+        mean = stats[2 * row];
+        inv = stats[2 * row + 1];
+      }
+      int8_t* cr = codes + row * kCols + pack0 * 512 + lane * 8;
+#pragma unroll
+      for (int i = 0; i < NPW; ++i) {
+        RawPack<f16> rp;
+        rp.q[0] = cur[i];
+        float d[8];
+        widen<f16>(rp, d);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d[e] = d[e] - mean;
+        // (held as four packed registers: otherwise the affine is emitted element by element)
+        u32x4 yb = __builtin_bit_cast(u32x4, prm.out(d, inv, i, params, lane));
+        asm volatile("" : "+v"(yb[0]), "+v"(yb[1]), "+v"(yb[2]), "+v"(yb[3]));
+        const f16x8 y = __builtin_bit_cast(f16x8, yb);
+        uint32_t words[2];
+#pragma unroll
+        for (int e4 = 0; e4 < 8; e4 += 4) {
+          uint32_t b[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float v = (float)y[e4 + j];
+            float q;
+            if constexpr (decltype(fast)::value) {
+              // (y is finite here: an infinite y makes the scale infinite, which is the other
+              // branch)
+              q = div_of_finite_half_value(v, s, recip);
+            } else {
+              q = v / s;
+            }
+            const float t = __builtin_rintf(q);
+            int c;
+            asm("v_cvt_i32_f32 %0, %1" : "=v"(c) : "v"(t));  // saturates; NaN -> 0
+            b[j] = (uint32_t)clamp_i32(c, lo, hi);
+          }
+          const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+          const uint32_t hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+          words[e4 / 4] = lo2 | hi2;
+        }
+        const u32x2 w2 = {words[0], words[1]};
+        __builtin_nontemporal_store(w2, reinterpret_cast<u32x2*>(cr + i * 512));
+      }
+    }
+  };
+  if (recip_ok) {
+    walk(std::true_type());
+  } else {
+    walk(std::false_type());
+  }
+}
+
 // host-side rounding of a float to T (round to nearest even)
 template<typename T>
 float round_to_T_host(float v) {
@@ -933,6 +1230,80 @@ extern "C" int ofq_fused_skip_layer_norm_min_max_observer(
   return ofq::run(stream, x, bias, skip, alpha, true, gamma, beta, y, scale, zero_point, t_dtype,
                   rows, cols, epsilon, quantization_bit, OFQ_LN_STATS_FP32, workspace,
                   workspace_bytes);
+}
+
+extern "C" size_t ofq_fused_layer_norm_quantization_workspace_bytes(int, int64_t rows, int64_t) {
+  // [partial maxima: rows floats, padded to 16 bytes][(mean, inv) of every row]
+  return rows > 0 ? (((size_t)rows * sizeof(float) + 15) & ~(size_t)15) + (size_t)rows * 2 * sizeof(float)
+                  : 0;
+}
+
+extern "C" int ofq_fused_layer_norm_quantization(void* stream, const void* x, const void* gamma,
+                                                 const void* beta, void* codes, float* scale,
+                                                 float* zero_point, int t_dtype, int64_t rows,
+                                                 int64_t cols, double epsilon, int quantization_bit,
+                                                 int statistics, void* workspace,
+                                                 size_t workspace_bytes) {
+  using namespace ofq;
+  OFQ_RETURN_IF(quantization_bit <= 1 || quantization_bit > 8, OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(statistics != OFQ_LN_STATS_FP32 && statistics != OFQ_LN_STATS_FP64,
+                OFQ_ERR_BAD_ATTR);
+  OFQ_RETURN_IF(t_dtype != OFQ_F16 && t_dtype != OFQ_BF16 && t_dtype != OFQ_F32,
+                OFQ_ERR_BAD_DTYPE);
+  OFQ_RETURN_IF(rows < 1 || cols < 1 || rows > 0x7FFFFFFF, OFQ_ERR_BAD_SHAPE);
+  OFQ_RETURN_IF(x == nullptr || codes == nullptr || scale == nullptr || zero_point == nullptr,
+                OFQ_ERR_NULL_POINTER);
+  OFQ_RETURN_IF(workspace == nullptr
+                    || workspace_bytes
+                           < ofq_fused_layer_norm_quantization_workspace_bytes(t_dtype, rows, cols)
+                    || !ofq_aligned16(workspace),
+                OFQ_ERR_WORKSPACE);
+  // the shapes the register-resident row kernels take; everything else is the two ops in a row
+  const int np = (int)(cols / 512);
+  if (t_dtype != OFQ_F16 || gamma == nullptr || beta == nullptr || cols % 512 != 0
+      || !(np == 1 || np == 2 || np == 4 || np == 8) || !ofq_aligned16(x) || !ofq_aligned16(gamma)
+      || !ofq_aligned16(beta) || (reinterpret_cast<uintptr_t>(codes) & 7u) != 0) {
+    return OFQ_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* part = static_cast<float*>(workspace);
+  float* stats = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace)
+                                          + (((size_t)rows * sizeof(float) + 15) & ~(size_t)15));
+  const uint16_t* xs = static_cast<const uint16_t*>(x);
+  const uint16_t* gs = static_cast<const uint16_t*>(gamma);
+  const uint16_t* bs = static_cast<const uint16_t*>(beta);
+  // one row per wave up to 16 waves per CU, beyond that the waves walk the rows; both kernels
+  // use the same grid, so a row meets the same wave of the same block twice
+  const int64_t waves = rows < 256 * 16 ? rows : 256 * 16;
+  constexpr int kWavesPerBlock = kLnqBlock / kWave;
+  const int grid = (int)((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+  const int64_t nparts = grid;  // one partial maximum per block of the first kernel (<= 512)
+  const bool exact = statistics == OFQ_LN_STATS_FP64;
+  // parts of a row in the second kernel: enough waves for 16 per CU where the rows allow it
+  int split = 1;
+  while (split < 4 && split * 2 <= np && waves * split * 2 <= 256 * 16) split *= 2;
+  const int grid2 = (grid + 7) / 8 * 8 * split;
+#define OFQ_LNQ1(NPV)                                                                           \
+  if (exact) {                                                                                  \
+    ln_quant_first<NPV, true><<<grid, kLnqBlock, 0, st>>>(xs, gs, bs, part, stats, rows, epsilon);  \
+  } else {                                                                                      \
+    ln_quant_first<NPV, false><<<grid, kLnqBlock, 0, st>>>(xs, gs, bs, part, stats, rows, epsilon); \
+  }
+#define OFQ_LNQ2(NPV, SPV)                                                                      \
+  if (split == SPV) {                                                                           \
+    ln_quant_second<NPV, SPV><<<grid2, kLnqBlock, 0, st>>>(                                     \
+        xs, gs, bs, part, nparts, stats, static_cast<int8_t*>(codes), scale, zero_point, rows,  \
+        quantization_bit, grid);                                                                \
+  }
+  switch (np) {
+    case 1: OFQ_LNQ1(1) OFQ_LNQ2(1, 1) break;
+    case 2: OFQ_LNQ1(2) OFQ_LNQ2(2, 1) OFQ_LNQ2(2, 2) break;
+    case 4: OFQ_LNQ1(4) OFQ_LNQ2(4, 1) OFQ_LNQ2(4, 2) OFQ_LNQ2(4, 4) break;
+    default: OFQ_LNQ1(8) OFQ_LNQ2(8, 1) OFQ_LNQ2(8, 2) OFQ_LNQ2(8, 4) break;
+  }
+#undef OFQ_LNQ1
+#undef OFQ_LNQ2
+  return ofq_check_launch();
 }
 
 extern "C" int ofq_fused_layer_norm_min_max_observer_stats(

@@ -419,8 +419,7 @@ quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
             const float t = t_rint<float>(q);
             int v;
             asm("v_cvt_i32_f32 %0, %1" : "=v"(v) : "v"(t));
-            v = v < lo ? lo : v;
-            b[j] = (uint32_t)(v > hi ? hi : v);
+            b[j] = (uint32_t)clamp_i32(v, lo, hi);
           }
           // low bytes of b[0..3] -> one word
           const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
@@ -479,37 +478,50 @@ quantize_half_to_bytes_kernel(const f16* __restrict__ in, const float* __restric
   const bool recip_ok = mag >= 0x1p-60f && mag <= 0x1p60f;
   const float recip = recip_ok ? 1.0f / s : 0.f;
   const int lo = (int)lower, hi = (int)upper;
-  for (int64_t tile = wave; tile < tiles; tile += nwaves) {
-    const f16* src = in + tile * 1024 + lane * 8;
-    u32x4 raw[2];
-    raw[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
-    raw[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 512));
+  // (the branch on the scale's range is taken once per wave: inside the loop both quotients
+  // were computed for every element and one of them selected)
+  auto walk = [&](auto fast) {
+    for (int64_t tile = wave; tile < tiles; tile += nwaves) {
+      const f16* src = in + tile * 1024 + lane * 8;
+      u32x4 raw[2];
+      raw[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
+      raw[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 512));
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      const f16x8 xv = __builtin_bit_cast(f16x8, raw[hf]);
-      uint32_t words[2];
+      for (int hf = 0; hf < 2; ++hf) {
+        const f16x8 xv = __builtin_bit_cast(f16x8, raw[hf]);
+        uint32_t words[2];
 #pragma unroll
-      for (int e4 = 0; e4 < 8; e4 += 4) {
-        uint32_t b[4];
+        for (int e4 = 0; e4 < 8; e4 += 4) {
+          uint32_t b[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float x = (float)xv[e4 + j];
-          float q = recip_ok ? div_of_half_value(x, s, recip) : x / s;
-          if (MODE != kModeSym) q = q + zp;
-          const float t = t_rint<float>(q);
-          int v;
-          asm("v_cvt_i32_f32 %0, %1" : "=v"(v) : "v"(t));  // saturates; NaN -> 0
-          v = v < lo ? lo : v;
-          b[j] = (uint32_t)(v > hi ? hi : v);
+          for (int j = 0; j < 4; ++j) {
+            const float x = (float)xv[e4 + j];
+            float q;
+            if constexpr (decltype(fast)::value) {
+              q = div_of_half_value(x, s, recip);
+            } else {
+              q = x / s;
+            }
+            if (MODE != kModeSym) q = q + zp;
+            const float t = t_rint<float>(q);
+            int v;
+            asm("v_cvt_i32_f32 %0, %1" : "=v"(v) : "v"(t));  // saturates; NaN -> 0
+            b[j] = (uint32_t)clamp_i32(v, lo, hi);
+          }
+          const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+          const uint32_t hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+          words[e4 / 4] = lo2 | hi2;
         }
-        const uint32_t lo2 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
-        const uint32_t hi2 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
-        words[e4 / 4] = lo2 | hi2;
+        u32x2 w2 = {words[0], words[1]};
+        __builtin_nontemporal_store(
+            w2, reinterpret_cast<u32x2*>(out + tile * 1024 + hf * 512 + lane * 8));
       }
-      u32x2 w2 = {words[0], words[1]};
-      __builtin_nontemporal_store(
-          w2, reinterpret_cast<u32x2*>(out + tile * 1024 + hf * 512 + lane * 8));
     }
+  };
+  if (recip_ok) {
+    walk(std::true_type());
+  } else {
+    walk(std::false_type());
   }
 }
 

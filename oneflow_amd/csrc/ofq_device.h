@@ -144,6 +144,26 @@ __device__ __forceinline__ float div_of_half_value(float a, float b, float y) {
   return __builtin_amdgcn_classf(a, 0x198) ? q : q0;
 }
 
+// The same quotient for a caller that only rounds it to an integer code and knows a is not
+// infinite: the select above is there for a = +-inf alone (the remainders turn it into NaN); NaN
+// stays NaN either way, and a zero comes out as +0 instead of +-0, which no integer code tells
+// apart.
+__device__ __forceinline__ float div_of_finite_half_value(float a, float b, float y) {
+  const float q0 = a * y;
+  const float r0 = __builtin_fmaf(-b, q0, a);
+  const float q1 = __builtin_fmaf(r0, y, q0);
+  const float r1 = __builtin_fmaf(-b, q1, a);
+  return __builtin_fmaf(r1, y, q1);
+}
+
+// min(max(v, lo), hi) for lo <= hi in one instruction (the compiler cannot know lo <= hi and
+// emits the pair)
+__device__ __forceinline__ int clamp_i32(int v, int lo, int hi) {
+  int r;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+  return r;
+}
+
 }  // namespace ofq
 
 // host-side launch helpers -------------------------------------------------------------------

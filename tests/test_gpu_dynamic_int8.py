@@ -110,6 +110,114 @@ def test_layer_norm_observer_exact_statistics_matches_the_oracle_bit_for_bit(t, 
         assert np.array_equal(H.to_numpy(a), O.quantize_to_int8(y_ref, s_ref, 8))
 
 
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (3, 512), (130, 1024), (257, 2048), (4099, 512),
+                                       (5000, 1024)])
+@pytest.mark.parametrize("exact", [False, True])
+def test_layer_norm_quantization_equals_the_two_ops(rows, cols, exact):
+    """LayerNorm -> observer -> int8 codes as one entry point (the normalised tensor is never
+    written) against fused_layer_norm_min_max_observer followed by quantization: identical
+    codes, scale and zero point, with fp32 and with fp64 row statistics, one row per wave and
+    rows walked by a wave (more than 4096 rows); with fp64 statistics also against the oracle.
+    A quarter of the rows carry an offset and a few values are large, so that the scale is set
+    by a single row."""
+    import oneflow_amd as flow
+    import torch
+    x, gamma, beta = _cfg5_inputs(rows, cols, "f16")
+    xf = O.to_f32(x).copy()
+    xf[::4] += 40.0
+    xf[rows // 2, 7] = 300.0
+    x = H.as_T(xf, "f16")
+    xt, gt, bt = H.to_torch(x), H.to_torch(gamma), H.to_torch(beta)
+    y, s, z = flow._C.fused_layer_norm_min_max_observer(xt, gt, bt, 1e-5, 8, exact_statistics=exact)
+    want = flow._C.quantization(y, s, z, "google", 8, "symmetric", out_dtype=torch.int8)
+    codes, s2, z2 = flow._C.fused_layer_norm_quantization(xt, gt, bt, 1e-5, 8, exact_statistics=exact)
+    assert codes.dtype == torch.int8 and codes.shape == xt.shape
+    assert torch.equal(s.view(torch.int32), s2.view(torch.int32)) and z2.item() == 0.0
+    assert torch.equal(codes, want)
+    if exact:
+        y_ref, s_ref, z_ref = O.layer_norm_min_max_observer(x, gamma, beta, 1e-5, 8)
+        assert H.to_numpy(s2)[0] == s_ref[0]
+        assert np.array_equal(H.to_numpy(codes), O.quantize_to_int8(y_ref, s_ref, 8))
+
+
+@pytest.mark.parametrize("bits", [2, 5, 8])
+def test_layer_norm_quantization_bit_widths_and_a_zero_row_tensor(bits):
+    import oneflow_amd as flow
+    import torch
+    x, gamma, beta = _cfg5_inputs(40, 1024, "f16")
+    xt, gt, bt = H.to_torch(x), H.to_torch(gamma), H.to_torch(beta)
+    y, s, z = flow._C.fused_layer_norm_min_max_observer(xt, gt, bt, 1e-5, bits)
+    want = flow._C.quantization(y, s, z, "google", bits, "symmetric", out_dtype=torch.int8)
+    codes, s2, z2 = flow._C.fused_layer_norm_quantization(xt, gt, bt, 1e-5, bits)
+    assert torch.equal(codes, want) and torch.equal(s.view(torch.int32), s2.view(torch.int32))
+    assert int(codes.max()) <= 2 ** (bits - 1) - 1 and int(codes.min()) >= -(2 ** (bits - 1))
+    # y = 0 everywhere (gamma = beta = 0): scale 0, and the codes of 0 / 0 as the two ops give them
+    zeros = torch.zeros_like(gt)
+    y, s, z = flow._C.fused_layer_norm_min_max_observer(xt, zeros, zeros, 1e-5, bits)
+    want = flow._C.quantization(y, s, z, "google", bits, "symmetric", out_dtype=torch.int8)
+    codes, s2, z2 = flow._C.fused_layer_norm_quantization(xt, zeros, zeros, 1e-5, bits)
+    assert s2.item() == 0.0 and torch.equal(codes, want)
+
+
+@pytest.mark.parametrize("t,rows,cols,with_params", [("f16", 9, 1000, True), ("bf16", 33, 1024, True),
+                                                     ("f32", 5, 512, True), ("f16", 12, 8192, True),
+                                                     ("f16", 16, 2048, False)])
+def test_layer_norm_quantization_other_shapes_run_the_two_ops(t, rows, cols, with_params):
+    """Shapes and dtypes outside the fused kernels: the C entry point reports
+    OFQ_ERR_UNSUPPORTED without launching anything, the functional runs the two ops."""
+    import oneflow_amd as flow
+    import torch
+    from oneflow_amd import _lib
+    x, gamma, beta = _cfg5_inputs(rows, cols, t)
+    xt = H.to_torch(x)
+    gt, bt = (H.to_torch(gamma), H.to_torch(beta)) if with_params else (None, None)
+    L = _lib.lib()
+    dt = {"f16": _lib.F16, "bf16": _lib.BF16, "f32": _lib.F32}[t]
+    nbytes = L.ofq_fused_layer_norm_quantization_workspace_bytes(dt, rows, cols)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    codes = torch.full((rows, cols), 77, dtype=torch.int8, device="cuda")
+    s = torch.full((1,), -1.0, device="cuda")
+    z = torch.full((1,), -1.0, device="cuda")
+    st = L.ofq_fused_layer_norm_quantization(
+        torch.cuda.current_stream().cuda_stream, xt.data_ptr(),
+        gt.data_ptr() if with_params else None, bt.data_ptr() if with_params else None,
+        codes.data_ptr(), s.data_ptr(), z.data_ptr(), dt, rows, cols, 1e-5, 8, _lib.LN_STATS_FP32,
+        ws.data_ptr(), nbytes)
+    torch.cuda.synchronize()
+    assert st == _lib.ERR_UNSUPPORTED and s.item() == -1.0 and int(codes.min()) == 77
+    y, s1, z1 = flow._C.fused_layer_norm_min_max_observer(xt, gt, bt, 1e-5, 8)
+    got, s2, z2 = flow._C.fused_layer_norm_quantization(xt, gt, bt, 1e-5, 8)
+    assert torch.equal(s1.view(torch.int32), s2.view(torch.int32))
+    if t == "f16":
+        want = flow._C.quantization(y, s1, z1, "google", 8, "symmetric", out_dtype=torch.int8)
+        assert torch.equal(got, want)
+
+
+def test_layer_norm_quantization_argument_errors():
+    import torch
+    from oneflow_amd import _lib
+    L = _lib.lib()
+    rows, cols = 8, 1024
+    x = torch.zeros(rows, cols, dtype=torch.float16, device="cuda")
+    g = torch.ones(cols, dtype=torch.float16, device="cuda")
+    codes = torch.zeros(rows, cols, dtype=torch.int8, device="cuda")
+    s = torch.zeros(1, device="cuda")
+    nbytes = L.ofq_fused_layer_norm_quantization_workspace_bytes(_lib.F16, rows, cols)
+    assert nbytes == 32 + rows * 8
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(bits=8, stats=_lib.LN_STATS_FP32, wsp=ws.data_ptr(), wsb=nbytes, xp=x.data_ptr()):
+        return L.ofq_fused_layer_norm_quantization(stream, xp, g.data_ptr(), g.data_ptr(),
+                                                   codes.data_ptr(), s.data_ptr(), s.data_ptr(),
+                                                   _lib.F16, rows, cols, 1e-5, bits, stats, wsp, wsb)
+    assert call() == 0
+    assert call(bits=9) == 4 and call(bits=1) == 4 and call(stats=7) == 4
+    assert call(wsp=None) == 6 and call(wsb=nbytes - 1) == 6
+    assert call(xp=None) == 1
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("t,rows,cols", [("f16", 2048, 4096), ("bf16", 300, 4096), ("f32", 33, 1000),
                                          ("f16", 7, 8200), ("bf16", 5, 24), ("bf16", 9, 16384),
                                          ("f16", 4, 20000)])
