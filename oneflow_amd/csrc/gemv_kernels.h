@@ -232,12 +232,6 @@ __device__ __forceinline__ float unit_corr(const u32x4 lo, const u32x4 hi) {
   return 1032.0f * sl + 72.0f * sh;
 }
 
-__device__ __forceinline__ float unit_corr_of(const u32x4 a, const u32x4 b) {
-  u32x4 lo, hi;
-  permute_unit(a, b, lo, hi);
-  return unit_corr(lo, hi);
-}
-
 // Pins the widening of a prefetched bias value to the place of use: without the empty asm the
 // compiler sinks the conversion (and the wait for every load issued so far) up to the load.
 __device__ __forceinline__ f16 bias_at_end(uint16_t raw) {
@@ -259,12 +253,11 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const uint32_t inv_chunks = row_of_inv(nchunks);
   const int npairs = (nchunks + 1) >> 1;
   const int G = K / group_size;
-  // LDS: [reduction NWAVES*64*4 f32][scale tile 16*G halves, padded to 16 B]
-  //      [corr: nchunks x 16 f32][x records]
+  // LDS: [reduction NWAVES*64*4 f32][scale tile 16*G halves, padded to 16 B][64 zero bytes]
+  //      [x records]
   float* red = reinterpret_cast<float*>(smem);
   f16* sl = reinterpret_cast<f16*>(smem + NWAVES * 64 * 16);
-  float* corr_l = reinterpret_cast<float*>(smem + NWAVES * 64 * 16 + ((16 * G * 2 + 15) & ~15));
-  uint8_t* zrec = reinterpret_cast<uint8_t*>(corr_l) + (STAGED ? nchunks * 64 : 0);  // 64 zero bytes
+  uint8_t* zrec = smem + NWAVES * 64 * 16 + ((16 * G * 2 + 15) & ~15);  // 64 zero bytes
   uint8_t* xs = zrec + 64;
 
   const int tid = threadIdx.x;
@@ -350,16 +343,7 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
         dst[0] = lo;
         dst[1] = hi;
       }
-      // the 8 units of a chunk sit in 8 consecutive lanes (K/16 is a multiple of 8): fold
-      float cpart = u < nunits ? unit_corr_of(xu[i][0], xu[i][1]) : 0.f;
-      cpart += __shfl_xor(cpart, 1, 64);
-      cpart += __shfl_xor(cpart, 2, 64);
-      cpart += __shfl_xor(cpart, 4, 64);
-      if (u < nunits && (u & 7) == 0) {
-        const int m = row_of(u >> 3, inv_chunks);
-        const int c = (u >> 3) - m * nchunks;
-        corr_l[c * 16 + m] = -cpart;  // negated: it seeds the MFMA accumulator
-      }
+      // (no correction sums here: the waves get them from the matrix core, see below)
     }
   }
   __syncthreads();
@@ -368,9 +352,9 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
   const int xrec_stride = has_x ? 256 : 0;
   const f16* xrow = x + (int64_t)(has_x ? r : 0) * K + kb * 32;
   const f16* slr = sl + r * G;
-  const f16 c_lo = (f16)1032.0f, c_hi = (f16)72.0f;
-  const f16x8 k1032 = {c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo};
-  const f16x8 k72 = {c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi};
+  const f16 c_lo = (f16)(-1032.0f), c_hi = (f16)(-72.0f);
+  const f16x8 kn1032 = {c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo};
+  const f16x8 kn72 = {c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi};
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
 
@@ -404,10 +388,18 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
           permute_unit(raw[2], raw[3], xa[2], xa[3]);
         }
         const float s = (float)slr[cpg_shift >= 0 ? (c >> cpg_shift) : (c * 128 / group_size)];
-        // the accumulator starts at -corr (staged), or corr is built alongside (not staged)
+        // the accumulator starts at -(1032 * sum_lo x + 72 * sum_hi x) of the chunk: the x
+        // operands against constant operands, four matrix instructions that do not depend on
+        // the codes (summing the terms with vector instructions while x is staged was two thirds
+        // of the staging pass)
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        f32x4 corr = {0.f, 0.f, 0.f, 0.f};
-        if (STAGED) acc = *reinterpret_cast<const f32x4*>(corr_l + c * 16 + kb * 4);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h]), kn1032,
+                                                       acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h + 1]),
+                                                       kn72, acc, 0, 0, 0);
+        }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const uint32_t w0 = wq[u][2 * h];
@@ -429,16 +421,9 @@ gemv_w4s_f16(const f16* __restrict__ x, const uint8_t* __restrict__ w,
                                                        0, 0, 0);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, __builtin_bit_cast(f16x8, bhi), acc,
                                                        0, 0, 0);
-          if (!STAGED) {
-            corr = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, k1032, corr, 0, 0, 0);
-            corr = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, k72, corr, 0, 0, 0);
-          }
         }
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const float q = STAGED ? acc[v] : acc[v] - corr[v];
-          total[v] = __builtin_fmaf(q, s, total[v]);
-        }
+        for (int v = 0; v < 4; ++v) total[v] = __builtin_fmaf(acc[v], s, total[v]);
       }
     }
     if (pn < npairs) {
@@ -564,17 +549,15 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   auto srow_of = [&](int vt) { return (GLU && vt >= ntiles ? rows_per_block : 0) + trow_of(vt); };
 
   // LDS: [red NMAT*tiles_per_block*NWAVES*M*16 f32][scales NMAT*rows_per_block*G halves, padded to 16 B]
-  //      [zeros, same size (asymmetric only)][corr nchunks*16 f32 (unrounded path only)]
-  //      [64 zero bytes][x records M*ncs*256 B, ncs = chunks of a phase]
+  //      [zeros, same size (asymmetric only)][64 zero bytes]
+  //      [x records M*ncs*256 B, ncs = chunks of a phase]
   float* red = reinterpret_cast<float*>(smem);
   const int tiles_per_block = (rows_per_block + 15) >> 4;
   const int red_floats = NMAT * tiles_per_block * NWAVES * M * 16;  // <= kW4pMaxTiles tiles
   const int tile_bytes = (NMAT * rows_per_block * G * 2 + 15) & ~15;
   f16* sl = reinterpret_cast<f16*>(smem + (size_t)red_floats * 4);
   f16* zl = reinterpret_cast<f16*>(reinterpret_cast<uint8_t*>(sl) + tile_bytes);
-  float* corr_l = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(sl)
-                                           + (ZMODE == kZeroAsym ? 2 : 1) * tile_bytes);
-  uint8_t* zrec = reinterpret_cast<uint8_t*>(corr_l) + (EXACT ? 0 : nchunks * 64);
+  uint8_t* zrec = reinterpret_cast<uint8_t*>(sl) + (ZMODE == kZeroAsym ? 2 : 1) * tile_bytes;
   uint8_t* xs = zrec + 64;
 
   // ---- requests that feed LDS go out first ----------------------------------------------------
@@ -765,15 +748,9 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
         dst[0] = lo;
         dst[1] = hi;
       }
-      float cpart = u < nunits ? unit_corr_of(xu[i][0], xu[i][1]) : 0.f;
-      cpart += __shfl_xor(cpart, 1, 64);
-      cpart += __shfl_xor(cpart, 2, 64);
-      cpart += __shfl_xor(cpart, 4, 64);
-      if (u < nunits && (u & 7) == 0) {
-        const int m = row_of(u >> 3, inv_chunks);
-        const int c = (u >> 3) - m * ncs;  // chunk within the phase
-        corr_l[c * 16 + m] = -cpart;
-      }
+      // (the correction terms are not summed here: sixteen conversions and additions per unit
+      // were two thirds of this pass; the waves get them from the matrix core instead, see
+      // process())
     }
   };
   stage_x();
@@ -794,6 +771,11 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
   const uint8_t* xrec = has_x ? xs + (size_t)r * (ncs * 256 + 16) + kb * 64 : zrec;
   const int xrec_stride = has_x ? 256 : 0;
   bool add_to_red = false;  // later phases: the (tile, wave) slots already hold earlier sums
+  const f16 c_lo = (f16)(-1032.0f), c_hi = (f16)(-72.0f);
+  const f16x8 kn1032 = {c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo, c_lo};
+  const f16x8 kn72 = {c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi, c_hi};
+  f32x4 cneg[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  int cneg_chunk[2] = {-1, -1};  // chunk (within the phase) whose correction terms cneg holds
   f32x4 total = {0.f, 0.f, 0.f, 0.f};
   f32x4 total1 = {0.f, 0.f, 0.f, 0.f};  // second accumulator of the exact path
   auto flush = [&](int t) {
@@ -852,7 +834,23 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
           continue;
         }
         const float s = (float)slr[grp];
-        f32x4 acc = *reinterpret_cast<const f32x4*>(corr_l + cl * 16 + kb * 4);
+        // -(1032 * sum_lo x + 72 * sum_hi x) of the chunk for the lane's rows of x: the x operands
+        // against constant operands, four matrix instructions that depend on LDS only and so
+        // issue while the codes are still on their way.  Kept from one tile of the block to the
+        // next: the tiles a wave walks mostly share their chunk pair.
+        if (cl != cneg_chunk[u]) {
+          f32x4 c0 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h]), kn1032,
+                                                        c0, 0, 0, 0);
+            c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa[2 * h + 1]),
+                                                        kn72, c0, 0, 0, 0);
+          }
+          cneg[u] = c0;
+          cneg_chunk[u] = cl;
+        }
+        f32x4 acc = cneg[u];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const uint32_t w0 = wq[d][u][2 * h];
@@ -934,6 +932,7 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
       inv_chunks = row_of_inv(ncs);
       nunits = M * ncs * 8;
       add_to_red = true;
+      cneg_chunk[0] = cneg_chunk[1] = -1;  // the chunk indices start over with other x
       total = f32x4{0.f, 0.f, 0.f, 0.f};
       first_items();
       __syncthreads();  // every wave has read its last x record and correction of the part before
@@ -1065,8 +1064,7 @@ inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int r
                                  bool exact, bool asym, int nmat = 1, int phases = 1) {
   const int G = K / group_size;
   return (size_t)nmat * ((rows_per_block + 15) / 16) * nwaves * M * 16 * 4
-         + (size_t)(asym ? 2 : 1) * ((nmat * rows_per_block * G * 2 + 15) & ~15)
-         + (exact ? 0 : (size_t)(K >> 7) * 64) + 64
+         + (size_t)(asym ? 2 : 1) * ((nmat * rows_per_block * G * 2 + 15) & ~15) + 64
          + (size_t)M * (gemv_w4p_phase_chunks(K, phases) * 256 + 16);
 }
 
@@ -1074,7 +1072,7 @@ inline size_t gemv_w4p_lds_bytes(int nwaves, int M, int K, int group_size, int r
 inline size_t gemv_w4s_lds_bytes(int nwaves, bool staged, int M, int K, int group_size) {
   const int G = K / group_size;
   return (size_t)nwaves * 64 * 16 + ((16 * G * 2 + 15) & ~15) + 64
-         + (staged ? (size_t)(K >> 7) * 64 + (size_t)M * (K * 2 + 16) : 0);
+         + (staged ? (size_t)M * (K * 2 + 16) : 0);
 }
 
 }  // namespace

@@ -463,8 +463,10 @@ quantize_kernel(const IN* __restrict__ in, const C* __restrict__ scale,
 // 1 KB requests (lane l: elements 8l.. and 512 + 8l..), so that every request and both 8-byte
 // stores of a wave are whole cache lines; the generic kernel's 32 bytes per lane make each request
 // touch half of every line.  elem_cnt a multiple of 1024.  Arithmetic as in quantize_kernel.
+// (waves_per_eu: without the cap the scheduler interleaves all 16 quotients of a turn on 96
+// registers, 5 waves per SIMD fit instead of 8, and the one-turn-per-wave launch runs in two rounds)
 template<typename OUT, int MODE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8)))
 quantize_half_to_bytes_kernel(const f16* __restrict__ in, const float* __restrict__ scale,
                               const float* __restrict__ zero_point, OUT* __restrict__ out,
                               int64_t tiles, float upper, float lower, int cambricon) {
