@@ -801,8 +801,17 @@ gemv_w4p_body(int block, const f16* __restrict__ x, const uint8_t* __restrict__ 
       if (c < nchunks) {
         const u32x4* xp = reinterpret_cast<const u32x4*>(xrec + cl * xrec_stride);
         u32x4 xa[4];
+        if (!EXACT) {
+          // only the lanes of rows of x that exist read: the other lanes' operands feed output
+          // rows that are never stored, so whatever their registers hold will do
+          if (has_x) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) xa[t] = xp[t];
+            for (int t = 0; t < 4; ++t) xa[t] = xp[t];
+          }
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) xa[t] = xp[t];
+        }
         const int grp = cpg_shift >= 0 ? (c >> cpg_shift) : (c * 128 / group_size);
         if (EXACT) {
           const f16 sh = slr[grp];
