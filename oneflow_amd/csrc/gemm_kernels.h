@@ -210,6 +210,8 @@ __device__ __forceinline__ int swizzle_key(int row) { return (row >> 1) & 7; }
 // random operands.  The kernel waits for its copies by hand (wait_vmem_le / wait_vmem_all below) and
 // a barrier, as it did before.  Every copy of a kernel must come through here: the compiler is
 // told that M0 changes, not what it holds.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // "clobber list contains reserved registers: m0"
 __device__ __forceinline__ void async_copy16_at(const uint8_t* base_uniform, uint32_t lane_off,
                                                 uint32_t lds_addr_uniform) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
@@ -217,6 +219,7 @@ __device__ __forceinline__ void async_copy16_at(const uint8_t* base_uniform, uin
                : "v"(lane_off), "s"(base_uniform), "s"(lds_addr_uniform)
                : "memory", "m0");
 }
+#pragma clang diagnostic pop
 // wait until at most N of this wave's vector-memory operations (incl. global->LDS copies) are
 // still outstanding; they complete in issue order, so this retires everything but the N newest
 template<int N>
