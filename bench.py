@@ -36,9 +36,9 @@ HBM_PEAK_GBPS = 8000.0
 # of 4096x4096 to one of 4096x11008) from two `rocprofv3 --pmc` runs of `bench.py --pmc-calibration`
 # (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for an elementwise
 # kernel of known size: x2.0 and x1.0); the summary is
-# profiles/gemv_w4_m1__llama7b_decode_m1__hbm_traffic_pmc.txt (11,742,271 B; rounded to 1000 B
+# profiles/gemv_w4_m1__llama7b_decode_m1__hbm_traffic_pmc.txt (11,747,966 B; rounded to 1000 B
 # here).  Valid for m = 1 only.
-PMC_TRAFFIC_BYTES_PER_LAUNCH_M1 = 11742000
+PMC_TRAFFIC_BYTES_PER_LAUNCH_M1 = 11748000
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "i8": 5000.0}
 
 LLAMA7B_LAYER = [  # (name, n, k, count per decoder layer)
