@@ -16,6 +16,7 @@
 // Added registrations (ops without a kernel in the reference tree; their op definitions would sit
 // next to OneFlowUserOps.td:8248-8387 with the argument names used here):
 //   fused_layer_norm_min_max_observer      x, [gamma], [beta], [bias], [skip] -> y, scale, zero_point
+//   fused_layer_norm_quantization          x, [gamma], [beta] -> out (int8), scale, zero_point
 //   matmul_quant                           a, b, a_scale, b_scale, [bias] -> out
 //   fused_glu_with_groupwise_quantized_weight      arguments of fused_glu + the weights' scales / zeros
 //   grouped_linear_with_groupwise_quantized_weight variadic xs, ws, w_scales, [w_zeros], [bs] -> ys
@@ -393,6 +394,90 @@ class OfqLayerNormObserverKernel final : public user_op::OpKernel, public user_o
 REGISTER_OFQ_LN_OBSERVER(DataType::kFloat16);
 REGISTER_OFQ_LN_OBSERVER(DataType::kBFloat16);
 REGISTER_OFQ_LN_OBSERVER(DataType::kFloat);
+
+// ---- fused_layer_norm_quantization: x, [gamma], [beta] -> out (int8 codes), scale, zero_point;
+//      attrs epsilon (double), quantization_bit (int32): fused_layer_norm_min_max_observer followed
+//      by quantization (symmetric, per layer) of its y.  The library serves the register-resident
+//      shapes with two kernels that never write y; for every other shape this kernel runs the two
+//      ops itself, y in the op's tmp_buffer -- the same bits either way -------------------------
+inline size_t LnQuantYBytes(DataType dtype, int64_t rows, int64_t cols) {
+  const size_t elem = dtype == DataType::kFloat ? 4 : 2;
+  return ((size_t)rows * (size_t)cols * elem + 255) & ~(size_t)255;
+}
+inline size_t LnQuantTmpBytes(DataType dtype, int64_t rows, int64_t cols) {
+  const size_t fused = ofq_fused_layer_norm_quantization_workspace_bytes(ToOfq(dtype), rows, cols);
+  const size_t two_ops = LnQuantYBytes(dtype, rows, cols)
+                         + ofq_fused_layer_norm_min_max_observer_workspace_bytes(ToOfq(dtype), rows,
+                                                                                 cols);
+  return fused > two_ops ? fused : two_ops;
+}
+class OfqLayerNormQuantizationKernel final : public user_op::OpKernel,
+                                             public user_op::CudaGraphSupport {
+ public:
+  using user_op::OpKernel::Compute;
+  void Compute(user_op::KernelComputeContext* ctx, user_op::OpKernelState*,
+               const user_op::OpKernelCache*) const override {
+    const user_op::Tensor* x = ctx->Tensor4ArgNameAndIndex("x", 0);
+    const user_op::Tensor* gamma =
+        ctx->has_input("gamma", 0) ? ctx->Tensor4ArgNameAndIndex("gamma", 0) : nullptr;
+    const user_op::Tensor* beta =
+        ctx->has_input("beta", 0) ? ctx->Tensor4ArgNameAndIndex("beta", 0) : nullptr;
+    user_op::Tensor* out = ctx->Tensor4ArgNameAndIndex("out", 0);
+    user_op::Tensor* scale = ctx->Tensor4ArgNameAndIndex("scale", 0);
+    user_op::Tensor* zero_point = ctx->Tensor4ArgNameAndIndex("zero_point", 0);
+    user_op::Tensor* tmp = ctx->Tensor4ArgNameAndIndex("tmp_buffer", 0);
+    CHECK_GE(x->shape_view().NumAxes(), 2);
+    const int64_t cols = x->shape_view().At(x->shape_view().NumAxes() - 1);
+    const int64_t rows = x->shape_view().elem_cnt() / cols;
+    if (gamma != nullptr) { CHECK_EQ(gamma->shape_view().elem_cnt(), cols); }
+    if (beta != nullptr) { CHECK_EQ(beta->shape_view().elem_cnt(), cols); }
+    CHECK_EQ(out->data_type(), DataType::kInt8);
+    CHECK_EQ(scale->data_type(), DataType::kFloat);
+    CHECK(tmp != nullptr);
+    const size_t tmp_bytes = (size_t)tmp->shape_view().elem_cnt();
+    CHECK_GE(tmp_bytes, LnQuantTmpBytes(x->data_type(), rows, cols));
+    const int dt = ToOfq(x->data_type());
+    const double epsilon = ctx->Attr<double>("epsilon");
+    const int32_t bits = ctx->Attr<int32_t>("quantization_bit");
+    const int status = ofq_fused_layer_norm_quantization(
+        RawStream(ctx), x->dptr(), gamma ? gamma->dptr() : nullptr, beta ? beta->dptr() : nullptr,
+        out->mut_dptr(), scale->mut_dptr<float>(), zero_point->mut_dptr<float>(), dt, rows, cols,
+        epsilon, bits, OFQ_LN_STATS_FP32, tmp->mut_dptr(), tmp_bytes);
+    if (status != OFQ_ERR_UNSUPPORTED) {
+      CheckOk(status, "fused_layer_norm_quantization");
+      return;
+    }
+    // the two ops: y at the front of tmp_buffer, the observer's partial maxima behind it
+    char* y = tmp->mut_dptr<char>();
+    const size_t y_bytes = LnQuantYBytes(x->data_type(), rows, cols);
+    CheckOk(ofq_fused_layer_norm_min_max_observer(
+                RawStream(ctx), x->dptr(), gamma ? gamma->dptr() : nullptr,
+                beta ? beta->dptr() : nullptr, y, scale->mut_dptr<float>(),
+                zero_point->mut_dptr<float>(), dt, rows, cols, epsilon, bits, y + y_bytes,
+                tmp_bytes - y_bytes),
+            "fused_layer_norm_min_max_observer");
+    CheckOk(ofq_quantization(RawStream(ctx), y, scale->dptr(), zero_point->dptr(), out->mut_dptr(),
+                             dt, OFQ_I8, rows * cols, 1, bits, OFQ_SCHEME_SYMMETRIC,
+                             OFQ_FORMULA_GOOGLE, OFQ_ZP_FLOAT),
+            "quantization");
+  }
+  bool AlwaysComputeWhenAllOutputsEmpty() const override { return false; }
+};
+
+#define REGISTER_OFQ_LN_QUANTIZATION(dtype)                                                    \
+  REGISTER_USER_KERNEL("fused_layer_norm_quantization")                                        \
+      .SetCreateFn<OfqLayerNormQuantizationKernel>()                                           \
+      .SetIsMatchedHob((user_op::HobDeviceType() == DeviceType::kCUDA)                         \
+                       && (user_op::HobDataType("x", 0) == dtype))                             \
+      .SetInferTmpSizeFn([](user_op::InferContext* ctx) -> size_t {                            \
+        const ShapeView xs = ctx->InputShape("x", 0);                                          \
+        const int64_t cols = xs.At(xs.NumAxes() - 1);                                          \
+        return LnQuantTmpBytes(dtype, xs.elem_cnt() / cols, cols);                             \
+      })                                                                                       \
+      .SetPriority(user_op::kKernelPriorityOptimized)
+REGISTER_OFQ_LN_QUANTIZATION(DataType::kFloat16);
+REGISTER_OFQ_LN_QUANTIZATION(DataType::kBFloat16);
+REGISTER_OFQ_LN_QUANTIZATION(DataType::kFloat);
 
 // ---- matmul_quant: a [m,k] int8, b [n,k] int8, a_scale [1] float, b_scale [n] float, [bias]
 //      -> out [m,n] (operand layout of fused_matmul_bias, OneFlowUserOps.td:5615-5633) ----------
@@ -804,6 +889,46 @@ extern "C" int ofq_plugin_run_layer_norm_observer(void* stream, void* x, void* g
   ctx.AddTensor("tmp_buffer", {tmp_bytes}, DataType::kUInt8, tmp);
   ctx.attrs["epsilon"].f = epsilon;
   ctx.attrs["alpha"].f = alpha;
+  ctx.attrs["quantization_bit"].i = bits;
+  auto kernel = r->create();
+  return ComputeLikeTheRuntime(*kernel, &ctx);
+}
+
+// Runs the registered LayerNorm -> int8 kernel; tmp must hold ofq_plugin_ln_quantization_tmp_bytes.
+extern "C" long long ofq_plugin_ln_quantization_tmp_bytes(int t_dtype, long long rows,
+                                                          long long cols) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["x"] = (DataType)t_dtype;
+  const auto* r = Lookup("fused_layer_norm_quantization", c);
+  if (r == nullptr || !r->infer_tmp_size) return -1;
+  user_op::InferContext ic;
+  ic.shapes["x"] = {rows, cols};
+  return (long long)r->infer_tmp_size(&ic);
+}
+extern "C" int ofq_plugin_run_layer_norm_quantization(void* stream, void* x, void* gamma,
+                                                      void* beta, void* out, void* scale,
+                                                      void* zero_point, void* tmp,
+                                                      long long tmp_bytes, int t_dtype,
+                                                      long long rows, long long cols,
+                                                      double epsilon, int bits) {
+  user_op::KernelRegContext c;
+  c.device = DeviceType::kCUDA;
+  c.arg_dtypes["x"] = (DataType)t_dtype;
+  const auto* r = Lookup("fused_layer_norm_quantization", c);
+  if (r == nullptr) return -1;
+  ep::CudaStream st(CurrentDevice(), stream);
+  user_op::KernelComputeContext ctx;
+  ctx.stream_ = &st;
+  const DataType T = (DataType)t_dtype;
+  ctx.AddTensor("x", {rows, cols}, T, x);
+  if (gamma) ctx.AddTensor("gamma", {cols}, T, gamma);
+  if (beta) ctx.AddTensor("beta", {cols}, T, beta);
+  ctx.AddTensor("out", {rows, cols}, DataType::kInt8, out);
+  ctx.AddTensor("scale", {1}, DataType::kFloat, scale);
+  ctx.AddTensor("zero_point", {1}, DataType::kFloat, zero_point);
+  ctx.AddTensor("tmp_buffer", {tmp_bytes}, DataType::kUInt8, tmp);
+  ctx.attrs["epsilon"].f = epsilon;
   ctx.attrs["quantization_bit"].i = bits;
   auto kernel = r->create();
   return ComputeLikeTheRuntime(*kernel, &ctx);

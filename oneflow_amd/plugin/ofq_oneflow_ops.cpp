@@ -125,6 +125,48 @@ struct FusedLayerNormMinMaxObserverOp {
   }
 };
 
+// ---- fused_layer_norm_quantization: x, [gamma], [beta] -> out (int8 codes, the shape of x),
+//      scale, zero_point; attrs epsilon (double), quantization_bit (int32).  The op above followed
+//      by `quantization` (symmetric, per layer) of its y (quantization_op.cpp: the output has the
+//      shape of the input) ------------------------------------------------------------------------
+struct FusedLayerNormQuantizationOp {
+  static Maybe<void> InferLogicalTensorDesc(user_op::InferContext* ctx) {
+    const user_op::TensorDesc& x_desc = ctx->InputTensorDesc("x", 0);
+    CHECK_GE_OR_RETURN(x_desc.shape().NumAxes(), 2);
+    const int64_t cols = x_desc.shape().At(x_desc.shape().NumAxes() - 1);
+    for (const char* name : {"gamma", "beta"}) {
+      if (ctx->has_input(name, 0)) {
+        const user_op::TensorDesc& d = ctx->InputTensorDesc(name, 0);
+        CHECK_EQ_OR_RETURN(d.shape().NumAxes(), 1);
+        CHECK_EQ_OR_RETURN(d.shape().At(0), cols);
+      }
+    }
+    const int32_t quantization_bit = ctx->Attr<int32_t>("quantization_bit");
+    CHECK_GT_OR_RETURN(quantization_bit, 1);
+    CHECK_LE_OR_RETURN(quantization_bit, 8);
+    CHECK_GE_OR_RETURN(ctx->Attr<double>("epsilon"), 0.0);
+    ctx->SetOutputShape("out", 0, x_desc.shape());
+    ctx->SetOutputShape("scale", 0, Shape({1}));
+    ctx->SetOutputShape("zero_point", 0, Shape({1}));
+    return Maybe<void>::Ok();
+  }
+  static Maybe<void> InferPhysicalTensorDesc(user_op::InferContext* ctx) {
+    return InferLogicalTensorDesc(ctx);
+  }
+  static Maybe<void> InferDataType(user_op::InferContext* ctx) {
+    const DataType data_type = ctx->InputDType("x", 0);
+    CHECK_OR_RETURN(data_type == DataType::kFloat16 || data_type == DataType::kBFloat16
+                    || data_type == DataType::kFloat);
+    for (const char* name : {"gamma", "beta"}) {
+      if (ctx->has_input(name, 0)) { CHECK_EQ_OR_RETURN(ctx->InputDType(name, 0), data_type); }
+    }
+    ctx->SetOutputDType("out", 0, DataType::kInt8);
+    ctx->SetOutputDType("scale", 0, DataType::kFloat);
+    ctx->SetOutputDType("zero_point", 0, DataType::kFloat);
+    return Maybe<void>::Ok();
+  }
+};
+
 // ---- matmul_quant: a [.., k] int8, b [n, k] int8, a_scale [1], b_scale [n], [bias] [n] -> out
 //      [.., n]; attr out_dtype ------------------------------------------------------------------
 struct MatmulQuantOp {
@@ -309,6 +351,7 @@ extern "C" int ofq_plugin_infer_run(void* c, const char* op) {
   auto* ctx = static_cast<user_op::InferContext*>(c);
   const std::string name = op;
   if (name == "fused_layer_norm_min_max_observer") return RunInference<FusedLayerNormMinMaxObserverOp>(ctx);
+  if (name == "fused_layer_norm_quantization") return RunInference<FusedLayerNormQuantizationOp>(ctx);
   if (name == "matmul_quant") return RunInference<MatmulQuantOp>(ctx);
   if (name == "fused_glu_with_groupwise_quantized_weight") {
     return RunInference<FusedGluWithGroupwiseQuantizedWeightOp>(ctx);

@@ -31,7 +31,8 @@ def test_registrations(plugin):
         seen.setdefault(name.value.decode(), []).append((prio.value, tmp.value))
     assert set(seen) == {"groupwise_dequantize", "fused_linear_with_groupwise_quantized_weight",
                          "min_max_observer", "moving_average_min_max_observer", "quantization",
-                         "fake_quantization", "fused_layer_norm_min_max_observer", "matmul_quant",
+                         "fake_quantization", "fused_layer_norm_min_max_observer",
+                         "fused_layer_norm_quantization", "matmul_quant",
                          "fused_glu_with_groupwise_quantized_weight",
                          "grouped_linear_with_groupwise_quantized_weight"}
     for name in ("fused_layer_norm_min_max_observer", "matmul_quant",
@@ -137,6 +138,30 @@ def test_dynamic_int8_ops_through_the_adapter(plugin):
         assert rc == 0
         torch.cuda.synchronize()
         assert torch.equal(y, want[0]) and torch.equal(s, want[1]) and torch.equal(z, want[2])
+    # LayerNorm -> int8 codes as one op: the shapes the library serves with its two kernels, and
+    # one it does not (the kernel class then runs the two ops inside the op's tmp_buffer)
+    lnq = plugin.ofq_plugin_run_layer_norm_quantization
+    lnq.argtypes = [vp] * 8 + [ll, ci, ll, ll, dbl, ci]
+    tmpb = plugin.ofq_plugin_ln_quantization_tmp_bytes
+    tmpb.argtypes = [ci, ll, ll]
+    tmpb.restype = ll
+    for r2, c2 in ((64, 1024), (9, 1000)):
+        x2 = H.to_torch(rng.standard_normal((r2, c2)).astype(np.float16))
+        g2 = H.to_torch((1 + 0.1 * rng.standard_normal(c2)).astype(np.float16))
+        b2 = H.to_torch((0.1 * rng.standard_normal(c2)).astype(np.float16))
+        y2, s2, z2 = flow._C.fused_layer_norm_min_max_observer(x2, g2, b2, 1e-5, 8)
+        want = flow._C.quantization(y2, s2, z2, "google", 8, "symmetric", out_dtype=torch.int8)
+        nbytes = tmpb(K_FLOAT16, r2, c2)
+        assert nbytes >= r2 * c2 * 2
+        tmp = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        codes = torch.full((r2, c2), 99, dtype=torch.int8, device="cuda")
+        s = torch.empty(1, dtype=torch.float32, device="cuda")
+        z = torch.empty(1, dtype=torch.float32, device="cuda")
+        rc = lnq(stream, x2.data_ptr(), g2.data_ptr(), b2.data_ptr(), codes.data_ptr(), s.data_ptr(),
+                 z.data_ptr(), tmp.data_ptr(), nbytes, K_FLOAT16, r2, c2, 1e-5, 8)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(codes, want) and torch.equal(s, s2) and z.item() == 0.0
     m, n, k = 48, 200, 256
     a = H.to_torch(rng.integers(-128, 128, size=(m, k)).astype(np.int8))
     b = H.to_torch(rng.integers(-127, 128, size=(n, k)).astype(np.int8))
@@ -381,6 +406,19 @@ def test_op_definitions_of_the_added_ops(plugin):
     assert "quantization_bit" in bad.run()
     bad = (_Infer(plugin, "fused_layer_norm_min_max_observer").inp("x", (4, 4096), K_FLOAT16)
            .inp("beta", (4096,), K_FLOAT).attrs(epsilon=1e-5, alpha=0.5, quantization_bit=8))
+    assert "Check failed" in bad.run()
+    # LayerNorm -> int8 codes
+    c = (_Infer(plugin, "fused_layer_norm_quantization").inp("x", (2, 7, 4096), K_FLOAT16)
+         .inp("gamma", (4096,), K_FLOAT16).inp("beta", (4096,), K_FLOAT16)
+         .attrs(epsilon=1e-5, quantization_bit=8))
+    assert c.run() is None
+    assert c.out("out") == ((2, 7, 4096), K_INT8)
+    assert c.out("scale") == ((1,), K_FLOAT) and c.out("zero_point") == ((1,), K_FLOAT)
+    bad = (_Infer(plugin, "fused_layer_norm_quantization").inp("x", (4096,), K_FLOAT16)
+           .attrs(epsilon=1e-5, quantization_bit=8))
+    assert "Check failed" in bad.run()
+    bad = (_Infer(plugin, "fused_layer_norm_quantization").inp("x", (4, 4096), K_FLOAT16)
+           .inp("gamma", (4096,), K_BFLOAT16).attrs(epsilon=1e-5, quantization_bit=8))
     assert "Check failed" in bad.run()
     # matmul_quant
     c = (_Infer(plugin, "matmul_quant").inp("a", (3, 2048, 4096), K_INT8).inp("b", (11008, 4096), K_INT8)
