@@ -102,10 +102,16 @@ __device__ __forceinline__ u32x4 dequant8_b4(uint32_t word, float s, float z) {
   u32x4 o;
   if constexpr (TT<T>::dtype == OFQ_BF16) {
     const float off = SIGNED ? -8.0f * s : 0.f;
+    // the two masked words stay as they are, so that byte b of each converts with one
+    // v_cvt_f32_ubyte<b>; folded into the original word every element costs a bit-field
+    // extract in front of its conversion
+    uint32_t hi_pinned = hi, lo_pinned = lo;
+    asm("" : "+v"(hi_pinned));
+    asm("" : "+v"(lo_pinned));
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      const float u0 = (float)((hi >> (8 * b)) & 0xFFu);
-      const float u1 = (float)((lo >> (8 * b)) & 0xFFu);
+      const float u0 = (float)((hi_pinned >> (8 * b)) & 0xFFu);
+      const float u1 = (float)((lo_pinned >> (8 * b)) & 0xFFu);
       const float p0 = SIGNED ? __builtin_fmaf(u0, s, off) : u0 * s;
       const float p1 = SIGNED ? __builtin_fmaf(u1, s, off) : u1 * s;
       uint32_t r = pack_bf16(p0, p1);
@@ -178,10 +184,13 @@ __device__ __forceinline__ u32x4 dequant8_b4_v(uint32_t word, const u32x4 s, con
   const uint32_t lo = word & 0x0F0F0F0Fu;         // elements 1, 3, 5, 7
   u32x4 o;
   if constexpr (TT<T>::dtype == OFQ_BF16) {
+    uint32_t hi_pinned = hi, lo_pinned = lo;  // as in dequant8_b4
+    asm("" : "+v"(hi_pinned));
+    asm("" : "+v"(lo_pinned));
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      const float u0 = (float)((hi >> (8 * b)) & 0xFFu);
-      const float u1 = (float)((lo >> (8 * b)) & 0xFFu);
+      const float u0 = (float)((hi_pinned >> (8 * b)) & 0xFFu);
+      const float u1 = (float)((lo_pinned >> (8 * b)) & 0xFFu);
       o[b] = dequant_pair_bf16<T, 4, SIGNED, ZMODE>(u0, u1, s[b], z[b]);
     }
   } else {
